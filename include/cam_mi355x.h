@@ -1,0 +1,271 @@
+/*
+ * cam_mi355x.h -- C ABI of the MI355X (gfx950) implementation of CAM's MoE hot path.
+ *
+ * Drop-in boundary.  The reference's PyTorch binding reaches its kernels through CANN's two-phase
+ * "aclnn" C ABI: EXEC_NPU_CMD resolves "aclnn<Op>GetWorkspaceSize" and "aclnn<Op>" with dlsym and
+ * calls them with tensors, attributes, then outputs (src/cam/comm_operator/pybind/pytorch_extension/
+ * pytorch_npu_helper.hpp:136-151,533-582).  This library exports the same pairs under the prefix
+ * "cam" with the same argument order.  Differences, all forced by the platform:
+ *   - aclTensor / aclTensorList (opaque CANN handles) become the plain structs camTensor /
+ *     camTensorList below; the library never allocates, frees or retains device memory;
+ *   - aclrtStream becomes camStream_t, which is a hipStream_t passed as void*;
+ *   - aclOpExecutor becomes camOpExecutor: created by phase 1, consumed and freed by phase 2
+ *     (single use, any thread).  camDestroyExecutor() frees one that will not be run.
+ * Phase 1 validates everything on the host and never touches the GPU.  Phase 2 only enqueues kernels
+ * on the given stream: no allocation, no synchronisation, no host read of device data.
+ * Every function returns 0 on success and a CAM_ERR_* code otherwise; camGetRecentErrMsg() returns
+ * the calling thread's last message (the counterpart of aclGetRecentErrMsg).
+ *
+ * One GPU: epWorldSize / numRanks > 1 is accepted where the arithmetic is rank-local
+ * (camDispatchLayout) and refused with CAM_ERR_UNSUPPORTED where peers would be needed.
+ * Limits kept from the reference: hidden size, top-k and expert-count ranges, dtypes and ranks.
+ * Limits lifted: tokens per call (reference: 256 fused / 8000 normal), local experts per rank
+ * (reference: 24), and epWorldSize >= 2 for the normal ops (1 is allowed here).
+ *
+ * Paths in comments are relative to the reference tree; AUTOGEN =
+ * src/cam/comm_operator/ascend_kernels/pregen/build_out/autogen.
+ */
+#ifndef CAM_MI355X_H_
+#define CAM_MI355X_H_
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define CAM_API __attribute__((visibility("default")))
+
+typedef int32_t camStatus;
+
+enum {
+    CAM_OK = 0,
+    CAM_ERR_NULL = 1,        /* a required pointer is NULL */
+    CAM_ERR_DTYPE = 2,       /* wrong element type */
+    CAM_ERR_SHAPE = 3,       /* wrong rank / extent / contiguity */
+    CAM_ERR_RANGE = 4,       /* attribute outside the supported range */
+    CAM_ERR_ALIGN = 5,       /* pointer or extent not aligned as the kernels need */
+    CAM_ERR_UNSUPPORTED = 6, /* valid in the reference, not built here (e.g. more than one rank) */
+    CAM_ERR_WORKSPACE = 7,   /* workspace NULL or smaller than phase 1 asked for */
+    CAM_ERR_EXECUTOR = 8,    /* executor NULL or not produced by the matching phase 1 */
+    CAM_ERR_LAUNCH = 9       /* the HIP runtime refused a launch */
+};
+
+/* Element types; numbering follows aclDataType so a binding can pass its codes through. */
+enum {
+    CAM_DT_FLOAT = 0,
+    CAM_DT_FLOAT16 = 1,
+    CAM_DT_INT8 = 2,
+    CAM_DT_INT32 = 3,
+    CAM_DT_UINT8 = 4,
+    CAM_DT_INT64 = 9,
+    CAM_DT_BOOL = 12,
+    CAM_DT_BF16 = 27
+};
+
+/* Storage formats.  CAM_FORMAT_ND is plain row-major.  CAM_FORMAT_MFMA_B is the weight layout
+ * produced by camPrepackWeight (this build's counterpart of the reference's FRACTAL_NZ cast,
+ * test/cam/ut/fused_deep_moe/test_fused_deep_moe.py:243-246). */
+enum {
+    CAM_FORMAT_ND = 2,
+    CAM_FORMAT_MFMA_B = 100
+};
+
+#define CAM_MAX_DIMS 8
+
+typedef struct camTensor {
+    void *data;                    /* device pointer */
+    int32_t dtype;                 /* CAM_DT_* */
+    int32_t ndim;
+    int64_t sizes[CAM_MAX_DIMS];
+    int64_t strides[CAM_MAX_DIMS]; /* in elements */
+    int32_t format;                /* CAM_FORMAT_* */
+    int32_t reserved;
+} camTensor;
+
+typedef struct camTensorList {
+    const camTensor *const *tensors;
+    uint64_t count;
+} camTensorList;
+
+typedef struct camOpExecutor camOpExecutor;
+typedef void *camStream_t; /* hipStream_t */
+
+CAM_API const char *camGetRecentErrMsg(void);
+CAM_API camStatus camDestroyExecutor(camOpExecutor *executor);
+CAM_API const char *camGetVersion(void);
+
+/* ------------------------------------------------------------------------------------------------
+ * DispatchLayout -- replaces aclnnDispatchLayout (AUTOGEN/aclnn_dispatch_layout.h:32-54).
+ * topkIdx int64 [T,K] (int32 also accepted) -> numTokensPerRank int32 [R], numTokensPerExpert
+ * int32 [E], isTokenInRank int32 [T,R] (bool/uint8 also accepted).  Ids < 0 are skipped; ids >= E are
+ * ignored and counted nowhere.  Outputs need not be zeroed by the caller.
+ * Limits (AK/dispatch_layout/op_host/dispatch_layout_tiling.cc:43-50): 0 < R <= 384, 0 < K <= 16;
+ * E <= 512 here (reference: 384). */
+CAM_API camStatus camDispatchLayoutGetWorkspaceSize(const camTensor *topkIdx, int64_t numTokens,
+                                                    int64_t numRanks, int64_t numExperts, int64_t numTopk,
+                                                    const camTensor *numTokensPerRank,
+                                                    const camTensor *numTokensPerExpert,
+                                                    const camTensor *isTokenInRank, uint64_t *workspaceSize,
+                                                    camOpExecutor **executor);
+CAM_API camStatus camDispatchLayout(void *workspace, uint64_t workspaceSize, camOpExecutor *executor,
+                                    camStream_t stream);
+
+/* ------------------------------------------------------------------------------------------------
+ * NotifyDispatch -- replaces aclnnNotifyDispatch (AUTOGEN/aclnn_notify_dispatch.h:35-63).
+ * tokenPerExpertData int32 [E] -> sendDataOffset int32 [E] (exclusive prefix sum), sendData int32 [3E]
+ * ((count, offset, numTokens) per expert; AK/notify_dispatch/op_kernel/notify_dispatch.h:121-152) and
+ * recvData int32 [3E].  With rankSize == 1 the all-to-all is the identity, so recvData == sendData.
+ * rankSize > 1 -> CAM_ERR_UNSUPPORTED. */
+CAM_API camStatus camNotifyDispatchGetWorkspaceSize(const camTensor *sendData,
+                                                    const camTensor *tokenPerExpertData, int64_t sendCount,
+                                                    int64_t numTokens, char *commGroup, int64_t rankSize,
+                                                    int64_t rankId, int64_t localRankSize,
+                                                    int64_t localRankId, const camTensor *sendDataOffset,
+                                                    const camTensor *recvData, uint64_t *workspaceSize,
+                                                    camOpExecutor **executor);
+CAM_API camStatus camNotifyDispatch(void *workspace, uint64_t workspaceSize, camOpExecutor *executor,
+                                    camStream_t stream);
+
+/* ------------------------------------------------------------------------------------------------
+ * MoeDispatchPlan -- replaces the two host loops of the reference binding, which copy the ids and
+ * the exchanged counts to the CPU and synchronise twice (src/cam/comm_operator/pybind/
+ * moe_dispatch_prefill.cpp:96-112 and :114-149), by one device kernel.
+ * topkIdx int64/int32 [T,K] ->
+ *   sendTokenIdx int32 [T,K]   rank of (t,k) among earlier flat entries with the same id (-1 if id<0)
+ *   numTokensPerExpert int32 [E], sendOffset int32 [E] (exclusive scan), recvOffset int32 [E],
+ *   recvCount int32 [E] (inclusive cumsum in (local expert, source rank) order),
+ *   numRecvTokensPerExpert int64 [E/R], totalRecvTokens int64 [1].  Any output except sendTokenIdx
+ *   may be NULL.  numRanks must be 1. */
+CAM_API camStatus camMoeDispatchPlanGetWorkspaceSize(const camTensor *topkIdx, int64_t numExperts,
+                                                     int64_t numRanks, int64_t rankId,
+                                                     const camTensor *sendTokenIdx,
+                                                     const camTensor *numTokensPerExpert,
+                                                     const camTensor *sendOffset, const camTensor *recvOffset,
+                                                     const camTensor *recvCount,
+                                                     const camTensor *numRecvTokensPerExpert,
+                                                     const camTensor *totalRecvTokens,
+                                                     uint64_t *workspaceSize, camOpExecutor **executor);
+CAM_API camStatus camMoeDispatchPlan(void *workspace, uint64_t workspaceSize, camOpExecutor *executor,
+                                     camStream_t stream);
+
+/* ------------------------------------------------------------------------------------------------
+ * MoeDispatchNormal -- replaces aclnnMoeDispatchNormal (AUTOGEN/aclnn_moe_dispatch_normal.h:17-25).
+ * x bf16 [T,H]; topkIdx int32 [T,K]; sendOffset, recvOffset, recvCount int32 [E]; sendTokenIdx
+ * int32 [T,K] -> recvX [A,H] (int8 when quantMode == 2, else x's dtype), recvXScales fp32 [A],
+ * assistInfoForCombine int32 [3A] = (srcRank, token, k) per row.
+ * Row of (t,k) with e = topkIdx[t,k] >= 0 (AK/moe_dispatch_normal/op_kernel/moe_dispatch_normal.h:
+ * 366-372 send side, :501-532 receive side): window row w = sendOffset[e] + sendTokenIdx[t,k];
+ * output row = (e ? recvCount[e-1] : 0) + (w - recvOffset[e]).  Rows outside [0,A) are dropped.
+ * quantMode 0: copy; 2: per-token dynamic int8, scale = 127/(max|x| + 1e-12), recvXScales = 1/scale
+ * (moe_dispatch_normal.h:278-316); 3 (extension): the fused kernel's variant without the epsilon
+ * (…/grouped_matmul_slice_m_per_token_dequant_swiglu_quant_multistage_workspace.h:780-818).
+ * quantMode 1 (static) -> CAM_ERR_UNSUPPORTED.  epWorldSize must be 1 (reference: >= 2).
+ * Limits (AK/moe_dispatch_normal/op_host/moe_dispatch_normal_tiling.cc:87-100): 1024 <= H <= 7168,
+ * 0 < K <= 16, 0 < E <= 512.  H must be a multiple of 16. */
+CAM_API camStatus camMoeDispatchNormalGetWorkspaceSize(
+    const camTensor *x, const camTensor *topkIdx, const camTensor *sendOffset, const camTensor *sendTokenIdx,
+    const camTensor *recvOffset, const camTensor *recvCount, char *groupEp, int64_t epWorldSize,
+    int64_t epRankId, char *groupTpOptional, int64_t tpWorldSize, int64_t tpRankId, int64_t moeExpertNum,
+    int64_t quantMode, int64_t globalBs, const camTensor *recvX, const camTensor *recvXScales,
+    const camTensor *assistInfoForCombine, uint64_t *workspaceSize, camOpExecutor **executor);
+CAM_API camStatus camMoeDispatchNormal(void *workspace, uint64_t workspaceSize, camOpExecutor *executor,
+                                       camStream_t stream);
+
+/* ------------------------------------------------------------------------------------------------
+ * MoeCombineNormal -- replaces aclnnMoeCombineNormal (AUTOGEN/aclnn_moe_combine_normal.h:37-65).
+ * recvX bf16 [A,H]; tokenSrcInfo int32 [3A]; epRecvCounts int32 [E]; recvTopkWeights fp32 [T,K]
+ * -> out bf16 [T,H].  out[t] = bf16(sum over k ascending of float(recvX[row(t,k)]) * w[t,k]), multiply
+ * and add rounded separately (AK/moe_combine_normal/op_kernel/moe_combine_normal.h:303-338); row(t,k) is
+ * the row whose triple names (t,k) (:232-238).  Slots no row names contribute nothing.
+ * Workspace: T*K int32 (the inverse map). */
+CAM_API camStatus camMoeCombineNormalGetWorkspaceSize(
+    const camTensor *recvX, const camTensor *tokenSrcInfo, const camTensor *epRecvCounts,
+    const camTensor *recvTopkWeights, const camTensor *tpRecvCountsOptional, char *epGroupName,
+    int64_t epWorldSize, int64_t epRankId, char *tpGroupNameOptional, int64_t tpWorldSize, int64_t tpRankId,
+    int64_t moeExpertNum, int64_t globalBs, const camTensor *out, uint64_t *workspaceSize,
+    camOpExecutor **executor);
+CAM_API camStatus camMoeCombineNormal(void *workspace, uint64_t workspaceSize, camOpExecutor *executor,
+                                      camStream_t stream);
+
+/* ------------------------------------------------------------------------------------------------
+ * PrepackWeight -- one-time weight layout conversion, off the timed path; the counterpart of
+ * torch_npu.npu_format_cast(w, FRACTAL_NZ) (test/cam/ut/fused_deep_moe/test_fused_deep_moe.py:243-246).
+ * src int8 [G,Kd,N] or [Kd,N], row-major -> dst int8, same extents, CAM_FORMAT_MFMA_B.
+ * gateUp != 0 pairs column c of the gate half [0,N/2) with column N/2 + c of the up half so that the
+ * SwiGLU product can be formed in registers (GMM1); 0 keeps column order (GMM2).
+ * Requires Kd % 128 == 0 and N % 64 == 0 (gateUp: N % 128 == 0). */
+CAM_API camStatus camPrepackWeightGetWorkspaceSize(const camTensor *src, int64_t gateUp, const camTensor *dst,
+                                                   uint64_t *workspaceSize, camOpExecutor **executor);
+CAM_API camStatus camPrepackWeight(void *workspace, uint64_t workspaceSize, camOpExecutor *executor,
+                                   camStream_t stream);
+
+/* ------------------------------------------------------------------------------------------------
+ * GroupedMatmulSwigluQuant -- the GMM1 stage of the fused kernel as an operator of its own
+ * (GroupedMatmulSliceMPerTokenDequantSwigluQuantMultiStageWorkspace, FDM/gemm/kernel/
+ * grouped_matmul_slice_m_per_token_dequant_swiglu_quant_multistage_workspace.h:355-1718; epilogue
+ * FDM/epilogue/block/block_epilogue_per_token_dequant_swiglu.h:164-275; re-quant :160-277).
+ * x int8 [A,H]; xScale fp32 [A]; weight list: one [G,H,2I] or G tensors [H,2I], CAM_FORMAT_MFMA_B with
+ * gateUp=1; weightScale list fp32 [G,2I] / G x [2I]; groupList int64 [G], cumulative row counts when
+ * groupListType == 0, per-expert counts when 1 -> y int8 [A,I], yScale fp32 [A].
+ * Workspace holds the fp32 SwiGLU product [A,I] and the tile table. */
+CAM_API camStatus camGroupedMatmulSwigluQuantGetWorkspaceSize(
+    const camTensor *x, const camTensor *xScale, const camTensorList *weight, const camTensorList *weightScale,
+    const camTensor *groupList, int64_t groupListType, const camTensor *y, const camTensor *yScale,
+    uint64_t *workspaceSize, camOpExecutor **executor);
+CAM_API camStatus camGroupedMatmulSwigluQuant(void *workspace, uint64_t workspaceSize, camOpExecutor *executor,
+                                              camStream_t stream);
+
+/* ------------------------------------------------------------------------------------------------
+ * GroupedMatmulDequant -- the GMM2 stage (GroupedMatmulSliceMPerTokenDequantMultiStageWorkspace,
+ * FDM/gemm/kernel/grouped_matmul_slice_m_per_token_dequant_multistage_workspace.h:24-378; epilogue
+ * FDM/epilogue/block/block_epilogue_per_token_dequant.hpp:572-703).
+ * x int8 [A,I]; xScale fp32 [A]; weight list [G,I,H] / G x [I,H], CAM_FORMAT_MFMA_B with gateUp=0;
+ * weightScale fp32 [G,H] -> out bf16 [A,H] = bf16((float(acc) * weightScale[g][h]) * xScale[m]). */
+CAM_API camStatus camGroupedMatmulDequantGetWorkspaceSize(
+    const camTensor *x, const camTensor *xScale, const camTensorList *weight, const camTensorList *weightScale,
+    const camTensor *groupList, int64_t groupListType, const camTensor *out, uint64_t *workspaceSize,
+    camOpExecutor **executor);
+CAM_API camStatus camGroupedMatmulDequant(void *workspace, uint64_t workspaceSize, camOpExecutor *executor,
+                                          camStream_t stream);
+
+/* ------------------------------------------------------------------------------------------------
+ * GroupedMatmulInt32 -- the raw int32 accumulators of either GEMM, before any epilogue; the tile the
+ * reference's cube cores hand to its vector cores (…swiglu_quant_multistage_workspace.h:558-632).
+ * Exists so that accumulation can be checked bit-for-bit.  gateUp says how `weight` was prepacked;
+ * out int32 [A,N] is in logical column order either way. */
+CAM_API camStatus camGroupedMatmulInt32GetWorkspaceSize(const camTensor *x, const camTensorList *weight,
+                                                        int64_t gateUp, const camTensor *groupList,
+                                                        int64_t groupListType, const camTensor *out,
+                                                        uint64_t *workspaceSize, camOpExecutor **executor);
+CAM_API camStatus camGroupedMatmulInt32(void *workspace, uint64_t workspaceSize, camOpExecutor *executor,
+                                        camStream_t stream);
+
+/* ------------------------------------------------------------------------------------------------
+ * FusedDeepMoe -- replaces aclnnFusedDeepMoe (AUTOGEN/aclnn_fused_deep_moe.h:19-46).
+ * x bf16 [bs,H]; expertIds int32 [bs,K]; gmm1PermutedWeight int8 [Epr,H,2I] (or Epr x [H,2I]),
+ * CAM_FORMAT_MFMA_B gateUp=1; gmm1PermutedWeightScale fp32 [Epr,2I]; gmm2Weight int8 [Epr,I,H],
+ * CAM_FORMAT_MFMA_B gateUp=0; gmm2WeightScale fp32 [Epr,H]; expertScales fp32 [bs,K];
+ * expertSmoothScalesOptional must be NULL (the reference stores and never uses it,
+ * AK/fused_deep_moe/op_kernel/fused_deep_moe.h:307); xActiveMaskOptional bool [bs], prefix semantics
+ * (…swiglu_quant_multistage_workspace.h:647-678) -> output bf16 [bs,H], expertTokenNums int64 [Epr].
+ * quantMode is accepted and ignored, as in the reference (fused_deep_moe.h:148,326).
+ * epRankSize must be 1 and sharedExpertRankNum 0.  Output rows of masked tokens are zero.
+ * Limits kept (AK/fused_deep_moe/op_host/fused_deep_moe_tiling.cpp:49-61): 512 <= H <= 7168,
+ * 1024 <= 2I <= 6144, K <= 12, moeExpertNum <= 512; H and I multiples of 128. */
+CAM_API camStatus camFusedDeepMoeGetWorkspaceSize(
+    const camTensor *x, const camTensor *expertIds, const camTensorList *gmm1PermutedWeight,
+    const camTensorList *gmm1PermutedWeightScale, const camTensorList *gmm2Weight,
+    const camTensorList *gmm2WeightScale, const camTensor *expertScales,
+    const camTensor *expertSmoothScalesOptional, const camTensor *xActiveMaskOptional, char *groupEp,
+    int64_t epRankSize, int64_t epRankId, int64_t moeExpertNum, int64_t sharedExpertNum,
+    int64_t sharedExpertRankNum, int64_t quantMode, int64_t globalBs, const camTensor *output,
+    const camTensor *expertTokenNums, uint64_t *workspaceSize, camOpExecutor **executor);
+CAM_API camStatus camFusedDeepMoe(void *workspace, uint64_t workspaceSize, camOpExecutor *executor,
+                                  camStream_t stream);
+
+#ifdef __cplusplus
+}
+#endif
+
+#endif /* CAM_MI355X_H_ */

@@ -1,0 +1,474 @@
+/*
+ * cam_oracle.c -- CPU restatement of the CAM MoE hot path.  TEST INFRASTRUCTURE ONLY.
+ *
+ * This file is the checker the HIP kernels are compared against.  Nothing in the shipped library
+ * links, loads or calls it; only tests/, the smoke test and the benchmark's cpu_baseline leg do.
+ *
+ * Every function restates one piece of the reference's arithmetic, in the reference's operation
+ * order, with IEEE-754 binary32 operations rounded once each.  Compile with -ffp-contract=off.
+ * Paths are relative to the reference tree; AK = src/cam/comm_operator/ascend_kernels,
+ * PB = src/cam/comm_operator/pybind, FDM = AK/fused_deep_moe/op_kernel/fused_deep_moe.
+ *
+ * Parity status.  Integer functions (layout, offsets, ranks, receive bookkeeping, int32 GEMM) and the
+ * dispatch quantisation are pinned by closed forms and brute-force definitions in tests/test_oracle.py.
+ * The reference ships no golden vectors for this path, and its kernels cannot be built without the
+ * Ascend toolkit, so no function here is checked against reference *outputs*.  Two functions rest on
+ * a deliberate definition the reference does not give portably and are therefore "parity unpinned"
+ * against the Ascend hardware bit-for-bit:
+ *   - cam_oracle_gmm1_epilogue: SiLU uses cam_expf_spec() in place of the Ascend Exp instruction;
+ *   - everything downstream of it (cam_oracle_swiglu_quant's int8 values, the bf16 layer output)
+ *     inherits that; the reference's own acceptance bound there is atol 2.0 / rtol 0.02.
+ * All-zero rows (division by zero in the reference, AK/.../grouped_matmul_slice_m_per_token_dequant_
+ * swiglu_quant_multistage_workspace.h:804 and :252-255) are defined here as q = 0, scale = 0.
+ */
+#include <stdint.h>
+#include <stdlib.h>
+#include <string.h>
+#include <math.h>
+
+#include "../include/cam_expf_spec.h"
+
+#ifdef _OPENMP
+#include <omp.h>
+#endif
+
+#define ORACLE_API __attribute__((visibility("default")))
+
+/* ---------------------------------------------------------------- bf16 helpers */
+
+static inline float bf16_to_f32(uint16_t v)
+{
+    uint32_t u = (uint32_t)v << 16;
+    float f;
+    memcpy(&f, &u, 4);
+    return f;
+}
+
+/* round-to-nearest-even, the CAST_RINT of FDM/raw_distributed/cam_moe_distribute_combine.h:778 */
+static inline uint16_t f32_to_bf16(float f)
+{
+    uint32_t u;
+    memcpy(&u, &f, 4);
+    if ((u & 0x7fffffffu) > 0x7f800000u) {
+        return (uint16_t)((u >> 16) | 0x0040u); /* quiet NaN */
+    }
+    uint32_t lsb = (u >> 16) & 1u;
+    u += 0x7fffu + lsb;
+    return (uint16_t)(u >> 16);
+}
+
+ORACLE_API int cam_oracle_num_threads(void)
+{
+#ifdef _OPENMP
+    return omp_get_max_threads();
+#else
+    return 1;
+#endif
+}
+
+ORACLE_API float cam_oracle_expf(float x) { return cam_expf_spec(x); }
+ORACLE_API float cam_oracle_silu(float x) { return cam_silu_spec(x); }
+ORACLE_API uint16_t cam_oracle_f32_to_bf16(float x) { return f32_to_bf16(x); }
+
+/* ---------------------------------------------------------------- A.1 layout
+ * AK/dispatch_layout/op_kernel/dispatch_layout.h:83-134 (counts, rank = e / (E/R), first-seen flag
+ * per token and rank); negative ids are skipped as in PB/moe_dispatch_prefill.cpp:106.
+ * Returns -1 if an id >= E is met. */
+ORACLE_API int cam_oracle_layout(const int64_t *idx, int64_t T, int64_t K, int64_t E, int64_t R,
+                                 int32_t *cnt, int32_t *per_rank, uint8_t *in_rank)
+{
+    int64_t epr = E / R;
+    memset(cnt, 0, sizeof(int32_t) * (size_t)E);
+    memset(per_rank, 0, sizeof(int32_t) * (size_t)R);
+    memset(in_rank, 0, (size_t)(T * R));
+    for (int64_t t = 0; t < T; ++t) {
+        for (int64_t k = 0; k < K; ++k) {
+            int64_t e = idx[t * K + k];
+            if (e < 0) {
+                continue;
+            }
+            if (e >= E) {
+                return -1;
+            }
+            cnt[e] += 1;
+            int64_t r = e / epr;
+            if (!in_rank[t * R + r]) {
+                in_rank[t * R + r] = 1;
+                per_rank[r] += 1;
+            }
+        }
+    }
+    return 0;
+}
+
+/* ---------------------------------------------------------------- A.2 offsets
+ * AK/notify_dispatch/op_kernel/notify_dispatch.h:121-152: exclusive prefix sum in global expert
+ * order, and the (count, offset, numTokens) triplet per expert. */
+ORACLE_API void cam_oracle_offsets(const int32_t *cnt, int64_t E, int32_t num_tokens, int32_t *off,
+                                   int32_t *triplets)
+{
+    int32_t run = 0;
+    for (int64_t e = 0; e < E; ++e) {
+        off[e] = run;
+        if (triplets) {
+            triplets[3 * e + 0] = cnt[e];
+            triplets[3 * e + 1] = run;
+            triplets[3 * e + 2] = num_tokens;
+        }
+        run += cnt[e];
+    }
+}
+
+/* ---------------------------------------------------------------- A.3 within-expert rank
+ * PB/moe_dispatch_prefill.cpp:96-112 (running counter per expert over the flat (t,k) order); the
+ * fused kernel's CalExpandxIdx (…swiglu_quant_multistage_workspace.h:680-708) computes the same
+ * number by counting earlier equal ids.  Entries with idx < 0 receive -1 (the reference leaves
+ * them uninitialised). */
+ORACLE_API void cam_oracle_send_token_idx(const int64_t *idx, int64_t T, int64_t K, int64_t E,
+                                          int32_t *pos)
+{
+    int32_t *run = (int32_t *)calloc((size_t)E, sizeof(int32_t));
+    for (int64_t i = 0; i < T * K; ++i) {
+        int64_t e = idx[i];
+        if (e < 0 || e >= E) {
+            pos[i] = -1;
+            continue;
+        }
+        pos[i] = run[e];
+        run[e] += 1;
+    }
+    free(run);
+}
+
+/* ---------------------------------------------------------------- A.4 receive bookkeeping
+ * PB/moe_dispatch_prefill.cpp:126-145.  recv_data is what rank `me` holds after the count exchange:
+ * for source rank s and local expert le the triplet sits at 3*(s*Epr + le).  Emits the inclusive
+ * cumsum in (local expert, source rank) order, the per-pair source offset, and the per-expert totals
+ * (int64, the binding's fourth return value; the fused kernel's expert_token_nums,
+ * …swiglu_quant_multistage_workspace.h:1540-1544).  Returns the total row count. */
+ORACLE_API int64_t cam_oracle_recv_bookkeeping(const int32_t *recv_data, int64_t R, int64_t epr,
+                                               int32_t *recv_count, int32_t *recv_offset,
+                                               int64_t *tokens_per_expert, int64_t *max_bs)
+{
+    int64_t total = 0;
+    int64_t mx = 0;
+    for (int64_t le = 0; le < epr; ++le) {
+        int64_t local = 0;
+        for (int64_t s = 0; s < R; ++s) {
+            int64_t index = le * R + s;
+            int64_t pair = 3 * (s * epr + le);
+            total += recv_data[pair];
+            recv_count[index] = (int32_t)total;
+            recv_offset[index] = recv_data[pair + 1];
+            if (recv_data[pair + 2] > mx) {
+                mx = recv_data[pair + 2];
+            }
+            local += recv_data[pair];
+        }
+        tokens_per_expert[le] = local;
+    }
+    if (max_bs) {
+        *max_bs = mx;
+    }
+    return total;
+}
+
+/* ---------------------------------------------------------------- A.6 per-token int8 quantisation
+ * variant 1 ("Q1"): AK/moe_dispatch_normal/op_kernel/moe_dispatch_normal.h:278-316
+ *     s = 127.0f / (max|x| + 1e-12f); q = int8(rint(x * s)); scale_out = 1.0f / s
+ * variant 2 ("Q2"): FDM/gemm/kernel/…swiglu_quant_multistage_workspace.h:780-818
+ *     s = 127.0f / max|x| (no epsilon); an all-zero row is defined as q = 0, scale_out = 0. */
+static void quant_token(const uint16_t *x, int64_t H, int variant, int8_t *q, float *scale_out)
+{
+    float m = 0.0f;
+    for (int64_t h = 0; h < H; ++h) {
+        float a = fabsf(bf16_to_f32(x[h]));
+        if (a > m) {
+            m = a;
+        }
+    }
+    float s;
+    if (variant == 1) {
+        s = 127.0f / (m + 1e-12f);
+    } else {
+        if (m == 0.0f) {
+            memset(q, 0, (size_t)H);
+            *scale_out = 0.0f;
+            return;
+        }
+        s = 127.0f / m;
+    }
+    for (int64_t h = 0; h < H; ++h) {
+        float v = bf16_to_f32(x[h]) * s;
+        q[h] = (int8_t)(int32_t)nearbyintf(v);
+    }
+    *scale_out = 1.0f / s;
+}
+
+ORACLE_API void cam_oracle_quant_rows(const uint16_t *x, int64_t rows, int64_t H, int variant,
+                                      int8_t *q, float *scales)
+{
+#pragma omp parallel for schedule(static)
+    for (int64_t r = 0; r < rows; ++r) {
+        quant_token(x + r * H, H, variant, q + r * H, scales + r);
+    }
+}
+
+/* ---------------------------------------------------------------- A.5 permute (+quant)
+ * moe_dispatch_normal.h:330-396 (send side: row = send_offset[e] + send_token_idx, source row
+ * tokenIndex / K, triple (srcRank, token, k) :318-328) and :486-535 (receive side: rows land at
+ * recv_count[i-1] + j).  With one rank the window row equals the output row.
+ * quant: 0 = copy bf16 rows, 1 = Q1, 2 = Q2.  out is bf16 [A,H] or int8 [A,H]. */
+ORACLE_API void cam_oracle_dispatch(const uint16_t *x, const int64_t *idx, const int32_t *off,
+                                    const int32_t *pos, int64_t T, int64_t K, int64_t H, int64_t E,
+                                    int quant, int32_t src_rank, void *out, float *scales,
+                                    int32_t *src_info)
+{
+#pragma omp parallel for schedule(static)
+    for (int64_t i = 0; i < T * K; ++i) {
+        int64_t e = idx[i];
+        if (e < 0 || e >= E) {
+            continue;
+        }
+        int64_t t = i / K;
+        int64_t row = (int64_t)off[e] + pos[i];
+        if (quant == 0) {
+            memcpy((uint16_t *)out + row * H, x + t * H, (size_t)H * 2);
+        } else {
+            quant_token(x + t * H, H, quant, (int8_t *)out + row * H, scales + row);
+        }
+        if (src_info) {
+            src_info[3 * row + 0] = src_rank;
+            src_info[3 * row + 1] = (int32_t)t;
+            src_info[3 * row + 2] = (int32_t)(i % K);
+        }
+    }
+}
+
+/* ---------------------------------------------------------------- A.7 / A.9 grouped int8 GEMM
+ * …swiglu_quant_multistage_workspace.h:558-632 and …per_token_dequant_multistage_workspace.h:115-215:
+ * for local expert g with rows [group_list[g-1], group_list[g]):  C[m,n] = sum_k A[m,k] * W[g][k][n],
+ * int8 x int8 accumulated exactly in int32.  group_list is cumulative (int64).  W is [G, Kd, N]. */
+ORACLE_API void cam_oracle_gmm_int32(const int8_t *a, const int8_t *w, const int64_t *group_list,
+                                     int64_t G, int64_t Kd, int64_t N, int32_t *c)
+{
+    for (int64_t g = 0; g < G; ++g) {
+        int64_t m0 = g == 0 ? 0 : group_list[g - 1];
+        int64_t m1 = group_list[g];
+        const int8_t *wg = w + g * Kd * N;
+#pragma omp parallel for schedule(static)
+        for (int64_t m = m0; m < m1; ++m) {
+            int32_t *cr = c + m * N;
+            for (int64_t n = 0; n < N; ++n) {
+                cr[n] = 0;
+            }
+            const int8_t *ar = a + m * Kd;
+            for (int64_t k = 0; k < Kd; ++k) {
+                int32_t av = ar[k];
+                if (av == 0) {
+                    continue;
+                }
+                const int8_t *wr = wg + k * N;
+                for (int64_t n = 0; n < N; ++n) {
+                    cr[n] += av * (int32_t)wr[n];
+                }
+            }
+        }
+    }
+}
+
+/* ---------------------------------------------------------------- A.7 GMM1 epilogue
+ * FDM/epilogue/block/block_epilogue_per_token_dequant_swiglu.h:236-264:
+ *   t = (float(C) * w_scale[g][n]) * x_scale[m]   (weight scale first, then token scale)
+ *   left half n < I: d = t / (1 + exp(-t));  right half: d = t.   d is fp32 [M, 2I]. */
+ORACLE_API void cam_oracle_gmm1_epilogue(const int32_t *c, const float *w_scale, const float *x_scale,
+                                         const int64_t *group_list, int64_t G, int64_t I, float *d)
+{
+    int64_t N = 2 * I;
+    for (int64_t g = 0; g < G; ++g) {
+        int64_t m0 = g == 0 ? 0 : group_list[g - 1];
+        int64_t m1 = group_list[g];
+        const float *ws = w_scale + g * N;
+#pragma omp parallel for schedule(static)
+        for (int64_t m = m0; m < m1; ++m) {
+            for (int64_t n = 0; n < N; ++n) {
+                float t = ((float)c[m * N + n] * ws[n]) * x_scale[m];
+                d[m * N + n] = n < I ? cam_silu_spec(t) : t;
+            }
+        }
+    }
+}
+
+/* ---------------------------------------------------------------- A.8 SwiGLU product + re-quant
+ * …swiglu_quant_multistage_workspace.h:198-265:  y = d_left * d_right; m = max|y|;
+ *   y_scale = m * (1.0f/127.0f);  q = int8(rint((y * 127.0f) * (1.0f / m))). */
+ORACLE_API void cam_oracle_swiglu_quant(const float *d, int64_t M, int64_t I, int8_t *q,
+                                        float *y_scale)
+{
+    const float inv127 = 1.0f / 127.0f;
+#pragma omp parallel for schedule(static)
+    for (int64_t m = 0; m < M; ++m) {
+        const float *dl = d + m * 2 * I;
+        const float *dr = dl + I;
+        float mx = 0.0f;
+        for (int64_t i = 0; i < I; ++i) {
+            float a = fabsf(dl[i] * dr[i]);
+            if (a > mx) {
+                mx = a;
+            }
+        }
+        if (mx == 0.0f) {
+            memset(q + m * I, 0, (size_t)I);
+            y_scale[m] = 0.0f;
+            continue;
+        }
+        y_scale[m] = mx * inv127;
+        float rcp = 1.0f / mx;
+        for (int64_t i = 0; i < I; ++i) {
+            float y = dl[i] * dr[i];
+            q[m * I + i] = (int8_t)(int32_t)nearbyintf((y * 127.0f) * rcp);
+        }
+    }
+}
+
+/* ---------------------------------------------------------------- A.9 GMM2 epilogue
+ * FDM/epilogue/block/block_epilogue_per_token_dequant.hpp:665-684:
+ *   out = bf16_rne((float(C2) * w2_scale[g][h]) * y_scale[m]). */
+ORACLE_API void cam_oracle_gmm2_epilogue(const int32_t *c, const float *w_scale, const float *y_scale,
+                                         const int64_t *group_list, int64_t G, int64_t H,
+                                         uint16_t *out)
+{
+    for (int64_t g = 0; g < G; ++g) {
+        int64_t m0 = g == 0 ? 0 : group_list[g - 1];
+        int64_t m1 = group_list[g];
+        const float *ws = w_scale + g * H;
+#pragma omp parallel for schedule(static)
+        for (int64_t m = m0; m < m1; ++m) {
+            for (int64_t h = 0; h < H; ++h) {
+                out[m * H + h] = f32_to_bf16(((float)c[m * H + h] * ws[h]) * y_scale[m]);
+            }
+        }
+    }
+}
+
+/* ---------------------------------------------------------------- A.10 combine
+ * FDM/raw_distributed/cam_moe_distribute_combine.h:726-780 and
+ * AK/moe_combine_normal/op_kernel/moe_combine_normal.h:303-338:  acc = 0; for k ascending, skipping
+ * idx < 0:  acc = acc + (float(row) * w[t,k])  (rounded multiply, then rounded add); bf16_rne(acc).
+ * row_of[t*K+k] is the expert-output row of slot (t,k), or < 0 to skip. */
+ORACLE_API void cam_oracle_combine(const uint16_t *y, const int32_t *row_of, const float *w, int64_t T,
+                                   int64_t K, int64_t H, uint16_t *out)
+{
+#pragma omp parallel for schedule(static)
+    for (int64_t t = 0; t < T; ++t) {
+        float *acc = (float *)calloc((size_t)H, sizeof(float));
+        for (int64_t k = 0; k < K; ++k) {
+            int32_t row = row_of[t * K + k];
+            if (row < 0) {
+                continue;
+            }
+            float wk = w[t * K + k];
+            const uint16_t *yr = y + (int64_t)row * H;
+            for (int64_t h = 0; h < H; ++h) {
+                float p = bf16_to_f32(yr[h]) * wk;
+                acc[h] = acc[h] + p;
+            }
+        }
+        for (int64_t h = 0; h < H; ++h) {
+            out[t * H + h] = f32_to_bf16(acc[h]);
+        }
+        free(acc);
+    }
+}
+
+/* row_of for the fused op: off[e] + pos (cam_moe_distribute_combine.h:737-742), -1 where idx < 0. */
+ORACLE_API void cam_oracle_rows_from_pos(const int64_t *idx, const int32_t *off, const int32_t *pos,
+                                         int64_t n, int64_t E, int32_t *row_of)
+{
+    for (int64_t i = 0; i < n; ++i) {
+        int64_t e = idx[i];
+        row_of[i] = (e < 0 || e >= E) ? -1 : off[e] + pos[i];
+    }
+}
+
+/* row_of for the "normal" op: invert the (srcRank, token, k) triples each row carries
+ * (moe_combine_normal.h:232-238: row r goes to slot token*K + k of its source rank). */
+ORACLE_API void cam_oracle_rows_from_src_info(const int32_t *src_info, int64_t A, int64_t T, int64_t K,
+                                              int32_t *row_of)
+{
+    for (int64_t i = 0; i < T * K; ++i) {
+        row_of[i] = -1;
+    }
+    for (int64_t r = 0; r < A; ++r) {
+        int64_t t = src_info[3 * r + 1];
+        int64_t k = src_info[3 * r + 2];
+        if (t >= 0 && t < T && k >= 0 && k < K) {
+            row_of[t * K + k] = (int32_t)r;
+        }
+    }
+}
+
+/* ---------------------------------------------------------------- the whole layer, one rank
+ * Composition of AK/fused_deep_moe/op_kernel/fused_deep_moe.h:346-440 for epRankSize == 1:
+ * counts -> offsets -> ranks -> Q2 permute -> GMM1 -> dequant+SiLU -> product+requant -> GMM2 ->
+ * dequant -> combine.  n_active tokens (x_active_mask prefix semantics,
+ * …swiglu_quant_multistage_workspace.h:647-678); output rows >= n_active are zero.
+ * w1 is [E, H, 2I], w2 is [E, I, H].  Optional debug outputs may be NULL. */
+ORACLE_API int cam_oracle_fused_layer(const uint16_t *x, const int64_t *idx, const float *topk_w,
+                                      const int8_t *w1, const float *w1_scale, const int8_t *w2,
+                                      const float *w2_scale, int64_t T, int64_t n_active, int64_t K,
+                                      int64_t H, int64_t I, int64_t E, uint16_t *out,
+                                      int64_t *expert_token_nums, int8_t *dbg_x1, float *dbg_x1_scale,
+                                      int8_t *dbg_x2, float *dbg_x2_scale, uint16_t *dbg_y)
+{
+    int64_t Ta = n_active;
+    int64_t A = Ta * K;
+    int32_t *cnt = (int32_t *)calloc((size_t)E, 4);
+    int32_t *off = (int32_t *)calloc((size_t)E, 4);
+    int32_t per_rank = 0;
+    uint8_t *in_rank = (uint8_t *)calloc((size_t)(Ta > 0 ? Ta : 1), 1);
+    if (cam_oracle_layout(idx, Ta, K, E, 1, cnt, &per_rank, in_rank) != 0) {
+        free(cnt);
+        free(off);
+        free(in_rank);
+        return -1;
+    }
+    cam_oracle_offsets(cnt, E, (int32_t)Ta, off, NULL);
+    int64_t *gl = (int64_t *)calloc((size_t)E, 8);
+    int64_t run = 0;
+    for (int64_t e = 0; e < E; ++e) {
+        run += cnt[e];
+        gl[e] = run;
+        expert_token_nums[e] = cnt[e];
+    }
+    int64_t rows = run;
+    size_t ra = (size_t)(A > 0 ? A : 1);
+    int32_t *pos = (int32_t *)malloc(ra * 4);
+    int32_t *row_of = (int32_t *)malloc(ra * 4);
+    cam_oracle_send_token_idx(idx, Ta, K, E, pos);
+    cam_oracle_rows_from_pos(idx, off, pos, A, E, row_of);
+    int8_t *x1 = (int8_t *)malloc(ra * (size_t)H);
+    float *x1s = (float *)malloc(ra * 4);
+    cam_oracle_dispatch(x, idx, off, pos, Ta, K, H, E, 2, 0, x1, x1s, NULL);
+    int32_t *c1 = (int32_t *)malloc(ra * (size_t)(2 * I) * 4);
+    cam_oracle_gmm_int32(x1, w1, gl, E, H, 2 * I, c1);
+    float *d = (float *)malloc(ra * (size_t)(2 * I) * 4);
+    cam_oracle_gmm1_epilogue(c1, w1_scale, x1s, gl, E, I, d);
+    int8_t *x2 = (int8_t *)malloc(ra * (size_t)I);
+    float *x2s = (float *)malloc(ra * 4);
+    cam_oracle_swiglu_quant(d, rows, I, x2, x2s);
+    int32_t *c2 = (int32_t *)malloc(ra * (size_t)H * 4);
+    cam_oracle_gmm_int32(x2, w2, gl, E, I, H, c2);
+    uint16_t *y = (uint16_t *)malloc(ra * (size_t)H * 2);
+    cam_oracle_gmm2_epilogue(c2, w2_scale, x2s, gl, E, H, y);
+    memset(out, 0, (size_t)(T * H) * 2);
+    cam_oracle_combine(y, row_of, topk_w, Ta, K, H, out);
+    if (dbg_x1) memcpy(dbg_x1, x1, (size_t)rows * (size_t)H);
+    if (dbg_x1_scale) memcpy(dbg_x1_scale, x1s, (size_t)rows * 4);
+    if (dbg_x2) memcpy(dbg_x2, x2, (size_t)rows * (size_t)I);
+    if (dbg_x2_scale) memcpy(dbg_x2_scale, x2s, (size_t)rows * 4);
+    if (dbg_y) memcpy(dbg_y, y, (size_t)rows * (size_t)H * 2);
+    free(cnt); free(off); free(in_rank); free(gl); free(pos); free(row_of); free(x1); free(x1s);
+    free(c1); free(d); free(x2); free(x2s); free(c2); free(y);
+    return 0;
+}

@@ -1,0 +1,245 @@
+"""ctypes/numpy front end of the CPU oracle (oracle/cam_oracle.c).
+
+TEST INFRASTRUCTURE ONLY: imported by tests/, by the smoke test and by the benchmark's cpu_baseline
+leg.  The shipped package never imports this module.
+
+bf16 tensors are carried as numpy uint16 arrays holding the raw bit patterns.
+"""
+import ctypes
+import os
+import subprocess
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_LIB_PATH = os.path.join(_HERE, "libcam_oracle.so")
+_lib = None
+
+
+def build(force=False):
+    """Compile the oracle with gcc (see oracle/Makefile)."""
+    if force and os.path.exists(_LIB_PATH):
+        os.remove(_LIB_PATH)
+    subprocess.check_call(["make", "-s", "-C", _HERE])
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        if not os.path.exists(_LIB_PATH):
+            build()
+        _lib = ctypes.CDLL(_LIB_PATH)
+        _lib.cam_oracle_expf.restype = ctypes.c_float
+        _lib.cam_oracle_expf.argtypes = [ctypes.c_float]
+        _lib.cam_oracle_silu.restype = ctypes.c_float
+        _lib.cam_oracle_silu.argtypes = [ctypes.c_float]
+        _lib.cam_oracle_f32_to_bf16.restype = ctypes.c_uint16
+        _lib.cam_oracle_f32_to_bf16.argtypes = [ctypes.c_float]
+        _lib.cam_oracle_recv_bookkeeping.restype = ctypes.c_int64
+        _lib.cam_oracle_num_threads.restype = ctypes.c_int
+    return _lib
+
+
+def _p(a):
+    return None if a is None else a.ctypes.data_as(ctypes.c_void_p)
+
+
+def _i64(v):
+    return ctypes.c_int64(int(v))
+
+
+def _c(a, dtype):
+    return np.ascontiguousarray(a, dtype=dtype)
+
+
+def num_threads():
+    return int(lib().cam_oracle_num_threads())
+
+
+def expf(x):
+    return float(lib().cam_oracle_expf(ctypes.c_float(x)))
+
+
+def silu(x):
+    return float(lib().cam_oracle_silu(ctypes.c_float(x)))
+
+
+def f32_to_bf16_bits(a):
+    """Round-to-nearest-even float32 -> bf16 bit patterns (vectorised, same rule as the C code)."""
+    u = np.ascontiguousarray(a, dtype=np.float32).view(np.uint32).astype(np.uint64)
+    lsb = (u >> 16) & 1
+    r = ((u + 0x7FFF + lsb) >> 16).astype(np.uint16)
+    return r
+
+
+def bf16_bits_to_f32(a):
+    return (np.ascontiguousarray(a, dtype=np.uint16).astype(np.uint32) << 16).view(np.float32)
+
+
+def layout(idx, E, R):
+    idx = _c(idx, np.int64)
+    T, K = idx.shape
+    cnt = np.empty(E, np.int32)
+    per_rank = np.empty(R, np.int32)
+    in_rank = np.empty((T, R), np.uint8)
+    rc = lib().cam_oracle_layout(_p(idx), _i64(T), _i64(K), _i64(E), _i64(R), _p(cnt), _p(per_rank),
+                                 _p(in_rank))
+    if rc != 0:
+        raise ValueError("expert id out of range")
+    return per_rank, cnt, in_rank.astype(bool)
+
+
+def offsets(cnt, num_tokens):
+    cnt = _c(cnt, np.int32)
+    E = cnt.shape[0]
+    off = np.empty(E, np.int32)
+    trip = np.empty(3 * E, np.int32)
+    lib().cam_oracle_offsets(_p(cnt), _i64(E), ctypes.c_int32(num_tokens), _p(off), _p(trip))
+    return off, trip
+
+
+def send_token_idx(idx, E):
+    idx = _c(idx, np.int64)
+    T, K = idx.shape
+    pos = np.empty((T, K), np.int32)
+    lib().cam_oracle_send_token_idx(_p(idx), _i64(T), _i64(K), _i64(E), _p(pos))
+    return pos
+
+
+def recv_bookkeeping(recv_data, R, epr):
+    recv_data = _c(recv_data, np.int32)
+    rc = np.empty(R * epr, np.int32)
+    ro = np.empty(R * epr, np.int32)
+    tpe = np.empty(epr, np.int64)
+    mx = ctypes.c_int64(0)
+    total = lib().cam_oracle_recv_bookkeeping(_p(recv_data), _i64(R), _i64(epr), _p(rc), _p(ro), _p(tpe),
+                                              ctypes.byref(mx))
+    return int(total), rc, ro, tpe, int(mx.value)
+
+
+def quant_rows(x_bits, variant):
+    x_bits = _c(x_bits, np.uint16)
+    rows, H = x_bits.shape
+    q = np.empty((rows, H), np.int8)
+    s = np.empty(rows, np.float32)
+    lib().cam_oracle_quant_rows(_p(x_bits), _i64(rows), _i64(H), ctypes.c_int(variant), _p(q), _p(s))
+    return q, s
+
+
+def dispatch(x_bits, idx, off, pos, E, quant, total_rows, src_rank=0):
+    x_bits = _c(x_bits, np.uint16)
+    idx = _c(idx, np.int64)
+    off = _c(off, np.int32)
+    pos = _c(pos, np.int32)
+    T, H = x_bits.shape
+    K = idx.shape[1]
+    A = max(int(total_rows), 1)
+    out = np.zeros((A, H), np.uint16 if quant == 0 else np.int8)
+    scales = np.zeros(A, np.float32)
+    src = np.zeros(3 * A, np.int32)
+    lib().cam_oracle_dispatch(_p(x_bits), _p(idx), _p(off), _p(pos), _i64(T), _i64(K), _i64(H), _i64(E),
+                              ctypes.c_int(quant), ctypes.c_int32(src_rank), _p(out), _p(scales), _p(src))
+    return out, scales, src
+
+
+def gmm_int32(a, w, group_list):
+    a = _c(a, np.int8)
+    w = _c(w, np.int8)
+    gl = _c(group_list, np.int64)
+    G, Kd, N = w.shape
+    c = np.zeros((a.shape[0], N), np.int32)
+    lib().cam_oracle_gmm_int32(_p(a), _p(w), _p(gl), _i64(G), _i64(Kd), _i64(N), _p(c))
+    return c
+
+
+def gmm1_epilogue(c, w_scale, x_scale, group_list):
+    c = _c(c, np.int32)
+    ws = _c(w_scale, np.float32)
+    xs = _c(x_scale, np.float32)
+    gl = _c(group_list, np.int64)
+    G, N = ws.shape
+    d = np.zeros((c.shape[0], N), np.float32)
+    lib().cam_oracle_gmm1_epilogue(_p(c), _p(ws), _p(xs), _p(gl), _i64(G), _i64(N // 2), _p(d))
+    return d
+
+
+def swiglu_quant(d, rows=None):
+    d = _c(d, np.float32)
+    M, N = d.shape
+    rows = M if rows is None else rows
+    q = np.zeros((M, N // 2), np.int8)
+    s = np.zeros(M, np.float32)
+    lib().cam_oracle_swiglu_quant(_p(d), _i64(rows), _i64(N // 2), _p(q), _p(s))
+    return q, s
+
+
+def gmm2_epilogue(c, w_scale, y_scale, group_list):
+    c = _c(c, np.int32)
+    ws = _c(w_scale, np.float32)
+    ys = _c(y_scale, np.float32)
+    gl = _c(group_list, np.int64)
+    G, H = ws.shape
+    out = np.zeros((c.shape[0], H), np.uint16)
+    lib().cam_oracle_gmm2_epilogue(_p(c), _p(ws), _p(ys), _p(gl), _i64(G), _i64(H), _p(out))
+    return out
+
+
+def rows_from_pos(idx, off, pos, E):
+    idx = _c(idx, np.int64)
+    off = _c(off, np.int32)
+    pos = _c(pos, np.int32)
+    row_of = np.empty(idx.shape, np.int32)
+    lib().cam_oracle_rows_from_pos(_p(idx), _p(off), _p(pos), _i64(idx.size), _i64(E), _p(row_of))
+    return row_of
+
+
+def rows_from_src_info(src_info, A, T, K):
+    src_info = _c(src_info, np.int32)
+    row_of = np.empty((T, K), np.int32)
+    lib().cam_oracle_rows_from_src_info(_p(src_info), _i64(A), _i64(T), _i64(K), _p(row_of))
+    return row_of
+
+
+def combine(y_bits, row_of, w):
+    y_bits = _c(y_bits, np.uint16)
+    row_of = _c(row_of, np.int32)
+    w = _c(w, np.float32)
+    T, K = row_of.shape
+    H = y_bits.shape[1]
+    out = np.zeros((T, H), np.uint16)
+    lib().cam_oracle_combine(_p(y_bits), _p(row_of), _p(w), _i64(T), _i64(K), _i64(H), _p(out))
+    return out
+
+
+def fused_layer(x_bits, idx, topk_w, w1, w1_scale, w2, w2_scale, n_active=None, debug=False):
+    """One rank's whole layer. w1 [E,H,2I] int8, w2 [E,I,H] int8. Returns (out bits, expert_token_nums[, dbg])."""
+    x_bits = _c(x_bits, np.uint16)
+    idx = _c(idx, np.int64)
+    topk_w = _c(topk_w, np.float32)
+    w1 = _c(w1, np.int8)
+    w2 = _c(w2, np.int8)
+    w1s = _c(w1_scale, np.float32)
+    w2s = _c(w2_scale, np.float32)
+    T, H = x_bits.shape
+    K = idx.shape[1]
+    E, _, N1 = w1.shape
+    I = N1 // 2
+    n_active = T if n_active is None else int(n_active)
+    out = np.zeros((T, H), np.uint16)
+    etn = np.zeros(E, np.int64)
+    A = max(n_active * K, 1)
+    dbg = None
+    args = [None] * 5
+    if debug:
+        dbg = dict(x1=np.zeros((A, H), np.int8), x1_scale=np.zeros(A, np.float32),
+                   x2=np.zeros((A, I), np.int8), x2_scale=np.zeros(A, np.float32),
+                   y=np.zeros((A, H), np.uint16))
+        args = [dbg["x1"], dbg["x1_scale"], dbg["x2"], dbg["x2_scale"], dbg["y"]]
+    rc = lib().cam_oracle_fused_layer(_p(x_bits), _p(idx), _p(topk_w), _p(w1), _p(w1s), _p(w2), _p(w2s),
+                                      _i64(T), _i64(n_active), _i64(K), _i64(H), _i64(I), _i64(E), _p(out),
+                                      _p(etn), *[_p(a) for a in args])
+    if rc != 0:
+        raise ValueError("expert id out of range")
+    if debug:
+        return out, etn, dbg
+    return out, etn

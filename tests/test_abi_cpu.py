@@ -1,0 +1,221 @@
+"""CPU-side checks of the C ABI: the library loads, exports every symbol the header declares, and
+phase 1 rejects bad arguments without touching a GPU (the reference's op_host validation,
+e.g. src/cam/comm_operator/ascend_kernels/fused_deep_moe/op_host/fused_deep_moe_tiling.cpp:278-316)."""
+import ctypes
+import os
+import re
+
+import pytest
+import torch
+
+from umdk_original_amd import _lib
+from umdk_original_amd._lib import (CAM_ERR_DTYPE, CAM_ERR_NULL, CAM_ERR_RANGE, CAM_ERR_SHAPE, CAM_ERR_UNSUPPORTED,
+                                    CAM_ERR_ALIGN, CAM_ERR_EXECUTOR, CAM_ERR_WORKSPACE, CAM_OK, CAM_FORMAT_MFMA_B)
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _header_symbols():
+    text = open(os.path.join(ROOT, "include", "cam_mi355x.h")).read()
+    return sorted(set(re.findall(r"CAM_API\s+[\w\s\*]*?\b(cam\w+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    names = _header_symbols()
+    assert len(names) == 23, names
+    handle = ctypes.CDLL(_lib.LIB_PATH)
+    for n in names:
+        assert hasattr(handle, n), n
+    assert sorted(_lib.EXPORTS) == names
+
+
+def test_version_and_error_string():
+    assert b"gfx950" in _lib.lib().camGetVersion()
+    st, _, msg = _lib.phase1("DispatchLayout", [None, 1, 1, 1, 1, None, None, None])
+    assert st == CAM_ERR_NULL and "topkIdx" in msg
+
+
+def _t(shape, dtype):
+    return torch.zeros(shape, dtype=dtype)
+
+
+def _layout_args(T=8, K=2, E=4, R=2, idx_dtype=torch.int64):
+    return [_t((T, K), idx_dtype), T, R, E, K, _t((R,), torch.int32), _t((E,), torch.int32), _t((T, R), torch.int32)]
+
+
+def test_dispatch_layout_validation():
+    assert _lib.phase1("DispatchLayout", _layout_args())[0] == CAM_OK
+    assert _lib.phase1("DispatchLayout", _layout_args(R=385, E=385))[0] == CAM_ERR_RANGE
+    assert _lib.phase1("DispatchLayout", _layout_args(E=513, R=1))[0] == CAM_ERR_RANGE
+    assert _lib.phase1("DispatchLayout", _layout_args(K=17))[0] == CAM_ERR_RANGE
+    assert _lib.phase1("DispatchLayout", _layout_args(E=5, R=2))[0] == CAM_ERR_RANGE  # E % R
+    assert _lib.phase1("DispatchLayout", _layout_args(idx_dtype=torch.float32))[0] == CAM_ERR_DTYPE
+    a = _layout_args()
+    a[0] = _t((8, 2, 1), torch.int64)
+    assert _lib.phase1("DispatchLayout", a)[0] == CAM_ERR_SHAPE
+    a = _layout_args()
+    a[0] = _t((8, 4), torch.int64)[:, ::2]  # not contiguous
+    assert _lib.phase1("DispatchLayout", a)[0] == CAM_ERR_SHAPE
+    a = _layout_args()
+    a[6] = _t((3,), torch.int32)
+    assert _lib.phase1("DispatchLayout", a)[0] == CAM_ERR_SHAPE
+
+
+def _dispatch_args(T=4, K=2, E=8, H=1024, quant=0, R=1, x_dtype=torch.bfloat16, A=None):
+    A = T * K if A is None else A
+    return [_t((T, H), x_dtype), _t((T, K), torch.int32), _t((E,), torch.int32), _t((T, K), torch.int32),
+            _t((E,), torch.int32), _t((E,), torch.int32), "g", R, 0, "g", 1, 0, E, quant, 0,
+            _t((A, H), torch.int8 if quant else x_dtype), _t((A,), torch.float32), _t((3 * A,), torch.int32)]
+
+
+def test_moe_dispatch_normal_validation():
+    assert _lib.phase1("MoeDispatchNormal", _dispatch_args())[0] == CAM_OK
+    assert _lib.phase1("MoeDispatchNormal", _dispatch_args(quant=2))[0] == CAM_OK
+    assert _lib.phase1("MoeDispatchNormal", _dispatch_args(H=512))[0] == CAM_ERR_RANGE
+    assert _lib.phase1("MoeDispatchNormal", _dispatch_args(H=7184))[0] == CAM_ERR_RANGE
+    assert _lib.phase1("MoeDispatchNormal", _dispatch_args(H=1032))[0] == CAM_ERR_ALIGN
+    assert _lib.phase1("MoeDispatchNormal", _dispatch_args(K=17, E=32))[0] == CAM_ERR_RANGE
+    assert _lib.phase1("MoeDispatchNormal", _dispatch_args(E=513))[0] == CAM_ERR_RANGE
+    assert _lib.phase1("MoeDispatchNormal", _dispatch_args(quant=4))[0] == CAM_ERR_RANGE
+    assert _lib.phase1("MoeDispatchNormal", _dispatch_args(quant=1))[0] == CAM_ERR_UNSUPPORTED
+    st, _, msg = _lib.phase1("MoeDispatchNormal", _dispatch_args(R=2))
+    assert st == CAM_ERR_UNSUPPORTED and "single-GPU" in msg
+    a = _dispatch_args(quant=2)
+    a[15] = _t((8, 1024), torch.bfloat16)  # quantised output must be int8
+    assert _lib.phase1("MoeDispatchNormal", a)[0] == CAM_ERR_DTYPE
+    a = _dispatch_args()
+    a[1] = _t((5, 2), torch.int32)  # ids disagree with x on dim 0
+    assert _lib.phase1("MoeDispatchNormal", a)[0] == CAM_ERR_SHAPE
+    a = _dispatch_args()
+    a[1] = _t((4, 2), torch.int64)  # kernels take int32 ids
+    assert _lib.phase1("MoeDispatchNormal", a)[0] == CAM_ERR_DTYPE
+    a = _dispatch_args()
+    a[17] = _t((5,), torch.int32)
+    assert _lib.phase1("MoeDispatchNormal", a)[0] == CAM_ERR_SHAPE
+
+
+def _combine_args(T=4, K=2, E=8, H=1024, R=1, gbs=0):
+    A = T * K
+    return [_t((A, H), torch.bfloat16), _t((3 * A,), torch.int32), _t((E,), torch.int32), _t((T, K), torch.float32),
+            None, "g", R, 0, "g", 1, 0, E, gbs, _t((T, H), torch.bfloat16)]
+
+
+def test_moe_combine_normal_validation():
+    st, ws, _ = _lib.phase1("MoeCombineNormal", _combine_args())
+    assert st == CAM_OK and ws >= 4 * 2 * 4
+    assert _lib.phase1("MoeCombineNormal", _combine_args(H=1000))[0] == CAM_ERR_RANGE
+    assert _lib.phase1("MoeCombineNormal", _combine_args(K=17))[0] == CAM_ERR_RANGE
+    assert _lib.phase1("MoeCombineNormal", _combine_args(R=4))[0] == CAM_ERR_UNSUPPORTED
+    assert _lib.phase1("MoeCombineNormal", _combine_args(gbs=3))[0] == CAM_ERR_RANGE
+    a = _combine_args()
+    a[3] = _t((4, 2), torch.float16)
+    assert _lib.phase1("MoeCombineNormal", a)[0] == CAM_ERR_DTYPE
+    a = _combine_args()
+    a[13] = _t((4, 2048), torch.bfloat16)
+    assert _lib.phase1("MoeCombineNormal", a)[0] == CAM_ERR_SHAPE
+    a = _combine_args()
+    a[0] = _t((8, 1024), torch.float32)
+    assert _lib.phase1("MoeCombineNormal", a)[0] == CAM_ERR_DTYPE
+
+
+def _packed(shape):
+    w = _t(shape, torch.int8)
+    w._cam_format = CAM_FORMAT_MFMA_B
+    return w
+
+
+def _fused_args(bs=4, K=2, E=4, H=1024, I=512, R=1, packed=True, smooth=None, mask=None):
+    mk = _packed if packed else (lambda s: _t(s, torch.int8))
+    return [_t((bs, H), torch.bfloat16), _t((bs, K), torch.int32), [mk((E, H, 2 * I))], [_t((E, 2 * I), torch.float32)],
+            [mk((E, I, H))], [_t((E, H), torch.float32)], _t((bs, K), torch.float32), smooth, mask, "g", R, 0, E, 1, 0,
+            0, 0, _t((bs, H), torch.bfloat16), _t((E,), torch.int64)]
+
+
+def test_fused_deep_moe_validation():
+    st, ws, _ = _lib.phase1("FusedDeepMoe", _fused_args())
+    assert st == CAM_OK and ws > 0
+    assert _lib.phase1("FusedDeepMoe", _fused_args(H=384))[0] == CAM_ERR_RANGE
+    assert _lib.phase1("FusedDeepMoe", _fused_args(I=256))[0] == CAM_ERR_RANGE     # 2I < 1024
+    assert _lib.phase1("FusedDeepMoe", _fused_args(I=3200))[0] == CAM_ERR_RANGE    # 2I > 6144
+    assert _lib.phase1("FusedDeepMoe", _fused_args(K=13, E=16))[0] == CAM_ERR_RANGE
+    assert _lib.phase1("FusedDeepMoe", _fused_args(E=513))[0] == CAM_ERR_RANGE
+    assert _lib.phase1("FusedDeepMoe", _fused_args(R=2))[0] == CAM_ERR_UNSUPPORTED
+    st, _, msg = _lib.phase1("FusedDeepMoe", _fused_args(packed=False))
+    assert st == CAM_ERR_UNSUPPORTED and "camPrepackWeight" in msg
+    assert _lib.phase1("FusedDeepMoe", _fused_args(smooth=_t((4, 1024), torch.float32)))[0] == CAM_ERR_UNSUPPORTED
+    assert _lib.phase1("FusedDeepMoe", _fused_args(mask=_t((5,), torch.bool)))[0] == CAM_ERR_SHAPE
+    assert _lib.phase1("FusedDeepMoe", _fused_args(mask=_t((4,), torch.bool)))[0] == CAM_OK
+    a = _fused_args()
+    a[1] = _t((5, 2), torch.int32)
+    assert _lib.phase1("FusedDeepMoe", a)[0] == CAM_ERR_SHAPE
+    a = _fused_args()
+    a[2] = [_packed((4, 1024, 512))]  # wrong 2I
+    assert _lib.phase1("FusedDeepMoe", a)[0] == CAM_ERR_SHAPE
+    a = _fused_args()
+    a[18] = _t((4,), torch.int32)
+    assert _lib.phase1("FusedDeepMoe", a)[0] == CAM_ERR_DTYPE
+    a = _fused_args()
+    a[2] = [_packed((1024, 1024)), _packed((1024, 1024))]  # list length neither 1 nor E
+    a[3] = [_t((1024,), torch.float32)] * 2
+    assert _lib.phase1("FusedDeepMoe", a)[0] == CAM_ERR_SHAPE
+
+
+def test_gemm_and_prepack_validation():
+    ok = [_t((2, 128, 128), torch.int8), 0, _t((2, 128, 128), torch.int8)]
+    assert _lib.phase1("PrepackWeight", ok)[0] == CAM_OK
+    assert _lib.phase1("PrepackWeight", [_t((2, 100, 128), torch.int8), 0, _t((2, 100, 128), torch.int8)])[0] == \
+        CAM_ERR_UNSUPPORTED
+    assert _lib.phase1("PrepackWeight", [_t((2, 128, 64), torch.int8), 1, _t((2, 128, 64), torch.int8)])[0] == \
+        CAM_ERR_UNSUPPORTED
+    assert _lib.phase1("PrepackWeight", [_t((2, 128, 128), torch.int8), 0, _t((2, 128, 256), torch.int8)])[0] == \
+        CAM_ERR_SHAPE
+    x = _t((10, 128), torch.int8)
+    gl = _t((2,), torch.int64)
+    out = _t((10, 128), torch.int32)
+    assert _lib.phase1("GroupedMatmulInt32", [x, [_packed((2, 128, 128))], 0, gl, 0, out])[0] == CAM_OK
+    assert _lib.phase1("GroupedMatmulInt32", [x, [_t((2, 128, 128), torch.int8)], 0, gl, 0, out])[0] == \
+        CAM_ERR_UNSUPPORTED
+    assert _lib.phase1("GroupedMatmulInt32", [x, [_packed((2, 128, 128))], 0, gl, 2, out])[0] == CAM_ERR_RANGE
+    assert _lib.phase1("GroupedMatmulInt32", [x, [_packed((2, 128, 128))], 0, _t((2,), torch.int32), 0, out])[0] == \
+        CAM_ERR_DTYPE
+
+
+def test_phase2_rejects_wrong_executor_and_small_workspace():
+    handle = _lib.lib()
+    assert handle.camDispatchLayout(None, 0, None, None) == CAM_ERR_EXECUTOR
+    # a combine executor handed to the layout op
+    args = _combine_args()
+    keep = [_lib.as_cam_tensor(a) if isinstance(a, torch.Tensor) else a for a in args]
+    cargs = [ctypes.byref(k) if isinstance(k, _lib.camTensor) else (k.encode() if isinstance(k, str) else k)
+             for k in keep]
+    ws = ctypes.c_uint64(0)
+    ex = ctypes.c_void_p(None)
+    assert handle.camMoeCombineNormalGetWorkspaceSize(*cargs, ctypes.byref(ws), ctypes.byref(ex)) == CAM_OK
+    assert handle.camDispatchLayout(None, 0, ex, None) == CAM_ERR_EXECUTOR  # consumed and freed
+    ex = ctypes.c_void_p(None)
+    assert handle.camMoeCombineNormalGetWorkspaceSize(*cargs, ctypes.byref(ws), ctypes.byref(ex)) == CAM_OK
+    assert handle.camMoeCombineNormal(None, 0, ex, None) == CAM_ERR_WORKSPACE  # no launch attempted
+    assert "workspace" in _lib.recent_error()
+
+
+def test_ops_refuse_cpu_tensors_and_unpacked_weights():
+    import umdk_original_amd as cam
+    with pytest.raises(RuntimeError, match="ROCm device"):
+        cam.get_dispatch_layout(torch.zeros(4, 2, dtype=torch.int64), 4, 1)
+    with pytest.raises(RuntimeError, match="Assertion failed"):
+        cam.get_dispatch_layout(torch.zeros(4, dtype=torch.int64), 4, 1)
+    with pytest.raises(cam.CamError):
+        cam.grouped_matmul_int32(torch.zeros(4, 128, dtype=torch.int8), torch.zeros(1, 128, 128, dtype=torch.int8),
+                                 torch.zeros(1, dtype=torch.int64))
+
+
+def test_torch_ops_registered_with_reference_schemas():
+    import umdk_original_amd  # noqa: F401
+    s = str(torch.ops.umdk_cam_op_lib.fused_deep_moe.default._schema)
+    assert "Tensor[] gmm1PermutedWeight" in s and "Tensor? xActiveMask" in s and "-> Tensor[]" in s
+    s = str(torch.ops.umdk_cam_op_lib.moe_dispatch_prefill.default._schema)
+    assert "int num_worst_tokens" in s and "str group_ep" in s
+    out = torch.ops.umdk_cam_op_lib.fused_deep_moe(
+        torch.empty(4, 1024, device="meta", dtype=torch.bfloat16), torch.empty(4, 2, device="meta", dtype=torch.int32),
+        [], [], [], [], torch.empty(4, 2, device="meta"), None, None, "g", 1, 0, 8, 1, 0, 0, 0)
+    assert out[0].shape == (4, 1024) and out[1].shape == (8,) and out[1].dtype == torch.int64

@@ -1,0 +1,127 @@
+"""GPU parity: grouped w8a8 GEMM (int32 accumulators bit-exact) and its two epilogues against the oracle."""
+import numpy as np
+import pytest
+import torch
+
+import umdk_original_amd as cam
+from umdk_original_amd import synth
+from gpu_util import announce, to_np, assert_bits_equal
+
+pytestmark = pytest.mark.gpu
+
+
+def _inputs(sizes, Kd, N, seed, wrange=127):
+    G = len(sizes)
+    gl = torch.tensor(np.cumsum(sizes), dtype=torch.int64)
+    A = int(gl[-1])
+    a = synth.uniform_int8((max(A, 1), Kd), seed)
+    w = synth.uniform_int8((G, Kd, N), seed + 1, -wrange, wrange)
+    return a, w, gl, A
+
+
+@pytest.mark.parametrize("gate_up", [False, True])
+@pytest.mark.parametrize("sizes,Kd,N", [
+    ([5], 128, 128),
+    ([1, 0, 33, 128, 129, 0, 7], 256, 256),
+    ([300, 2, 0, 64], 384, 640),
+    ([17, 40], 1024, 1152),
+])
+def test_int32_accumulators_bit_exact(gpu, oracle, sizes, Kd, N, gate_up):
+    announce("gemm int32 sizes=%s Kd=%d N=%d gate_up=%s" % (sizes, Kd, N, gate_up))
+    a, w, gl, A = _inputs(sizes, Kd, N, seed=Kd + N)
+    wp = cam.prepack_weight(w.to(gpu), gate_up)
+    got = cam.grouped_matmul_int32(a.to(gpu), wp, gl.to(gpu))
+    want = oracle.gmm_int32(a.numpy(), w.numpy(), gl.numpy())
+    assert_bits_equal(to_np(got)[:A], want[:A], "int32 accumulators")
+
+
+def test_int32_extreme_operands(gpu, oracle):
+    announce("gemm int32 extremes")
+    Kd, N = 7168, 128
+    a = torch.full((3, Kd), -128, dtype=torch.int8)
+    a[1] = 127
+    a[2, ::2] = 127
+    w = torch.full((1, Kd, N), -128, dtype=torch.int8)
+    w[0, :, ::3] = 127
+    gl = torch.tensor([3], dtype=torch.int64)
+    got = cam.grouped_matmul_int32(a.to(gpu), cam.prepack_weight(w.to(gpu), False), gl.to(gpu))
+    want = oracle.gmm_int32(a.numpy(), w.numpy(), gl.numpy())
+    assert_bits_equal(to_np(got), want, "int32 accumulators")
+    assert int(got.max()) == Kd * 128 * 128
+
+
+def test_group_list_as_counts_and_per_expert_tensors(gpu, oracle):
+    announce("gemm counts + tensor list")
+    sizes = [9, 0, 140, 3]
+    a, w, gl, A = _inputs(sizes, 256, 128, seed=21)
+    want = oracle.gmm_int32(a.numpy(), w.numpy(), gl.numpy())
+    counts = torch.tensor(sizes, dtype=torch.int64)
+    wp = cam.prepack_weight(w.to(gpu), False)
+    got = cam.grouped_matmul_int32(a.to(gpu), wp, counts.to(gpu), group_list_type=1)
+    assert_bits_equal(to_np(got)[:A], want[:A], "counts form")
+    per = [cam.prepack_weight(w[g].to(gpu), False) for g in range(len(sizes))]
+    got = cam.grouped_matmul_int32(a.to(gpu), per, gl.to(gpu))
+    assert_bits_equal(to_np(got)[:A], want[:A], "tensor list form")
+
+
+@pytest.mark.parametrize("sizes,H,I", [([4, 0, 131, 60], 256, 128), ([128, 1, 77], 1024, 512), ([3, 200], 512, 1536)])
+def test_gmm1_swiglu_quant_bit_exact(gpu, oracle, sizes, H, I):
+    announce("gmm1 sizes=%s H=%d I=%d" % (sizes, H, I))
+    a, w, gl, A = _inputs(sizes, H, 2 * I, seed=H + I, wrange=16)
+    G = len(sizes)
+    ws = synth.channel_scales((G, 2 * I), seed=31)
+    xs = synth.channel_scales((max(A, 1),), seed=32, lo=0.005, hi=0.05)
+    a[min(5, A - 1)] = 0  # an all-zero activation row -> all-zero product row
+    y, ysc = cam.grouped_matmul_swiglu_quant(a.to(gpu), xs.to(gpu), cam.prepack_weight(w.to(gpu), True), ws.to(gpu),
+                                             gl.to(gpu))
+    c = oracle.gmm_int32(a.numpy(), w.numpy(), gl.numpy())
+    d = oracle.gmm1_epilogue(c, ws.numpy(), xs.numpy(), gl.numpy())
+    want_q, want_s = oracle.swiglu_quant(d, rows=A)
+    assert_bits_equal(to_np(ysc)[:A].view(np.uint32), want_s[:A].view(np.uint32), "y_scale")
+    assert_bits_equal(to_np(y)[:A], want_q[:A], "y int8")
+    assert (to_np(y)[min(5, A - 1)] == 0).all() and float(ysc[min(5, A - 1)]) == 0.0
+
+
+@pytest.mark.parametrize("sizes,I,H", [([4, 0, 131, 60], 128, 256), ([128, 1, 77], 512, 1024), ([3, 200], 2048, 7168)])
+def test_gmm2_dequant_bit_exact(gpu, oracle, sizes, I, H):
+    announce("gmm2 sizes=%s I=%d H=%d" % (sizes, I, H))
+    a, w, gl, A = _inputs(sizes, I, H, seed=I + H, wrange=16)
+    G = len(sizes)
+    ws = synth.channel_scales((G, H), seed=33)
+    xs = synth.channel_scales((max(A, 1),), seed=34, lo=0.001, hi=0.01)
+    out = cam.grouped_matmul_dequant(a.to(gpu), xs.to(gpu), cam.prepack_weight(w.to(gpu), False), ws.to(gpu), gl.to(gpu))
+    c = oracle.gmm_int32(a.numpy(), w.numpy(), gl.numpy())
+    want = oracle.gmm2_epilogue(c, ws.numpy(), xs.numpy(), gl.numpy())
+    assert out.dtype == torch.bfloat16
+    assert_bits_equal(to_np(out)[:A], want[:A], "bf16 output")
+
+
+def test_full_size_grouped_gemm_sampled_rows(gpu):
+    """One GPU's 32 local experts at the benchmark shape; sampled rows against an exact CPU integer matmul."""
+    announce("gemm C3 full size, sampled rows")
+    G, H, I, rows = 32, 7168, 2048, 8192
+    sizes = synth.zipf_group_sizes(G, rows, seed=45)
+    assert int((sizes == 0).sum()) >= 3
+    gl = torch.cumsum(sizes, 0)
+    a = synth.uniform_int8((rows, H), 45)
+    g_cpu = torch.Generator().manual_seed(451)
+    w1 = torch.randint(-127, 128, (G, H, 2 * I), generator=g_cpu, dtype=torch.int8)
+    wp = cam.prepack_weight(w1.to(gpu), True)
+    got = cam.grouped_matmul_int32(a.to(gpu), wp, gl.to(gpu))
+    starts = (gl - sizes).tolist()
+    checked = 0
+    for g in range(G):
+        n = int(sizes[g])
+        if n == 0:
+            continue
+        pick = sorted({0, n - 1, n // 2})
+        r = torch.tensor([starts[g] + p for p in pick])
+        want = a[r].to(torch.int32) @ w1[g].to(torch.int32)  # exact
+        assert torch.equal(got[r.to(gpu)].cpu(), want), "expert %d" % g
+        checked += len(pick)
+    assert checked >= 29
+    # linearity in the activations: doubling a (within int8 range) doubles every accumulator
+    a_small = torch.clamp(a, -60, 60)
+    c1 = cam.grouped_matmul_int32(a_small.to(gpu), wp, gl.to(gpu))
+    c2 = cam.grouped_matmul_int32((a_small * 2).to(gpu), wp, gl.to(gpu))
+    assert torch.equal(c2, c1 * 2)

@@ -1,0 +1,430 @@
+"""Pins the CPU oracle against closed forms, brute-force definitions and library routines.
+
+The reference holds no golden vectors for this path and cannot be built or imported here, so every
+oracle function is checked against what the mathematics fixes, with cases chosen so that a plausible
+mistake (dropped epsilon, swapped halves, wrong scale order, fused multiply-add, wrong rounding) fails.
+"""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+from umdk_original_amd import synth
+
+
+def _rng(seed):
+    return np.random.default_rng(seed)
+
+
+# ------------------------------------------------------------------ layout / offsets / ranks
+@pytest.mark.parametrize("T,K,E,R", [(1, 1, 1, 1), (17, 3, 8, 2), (128, 8, 256, 8), (33, 16, 48, 48), (64, 2, 8, 1)])
+def test_layout_matches_bincount_and_set_logic(oracle, T, K, E, R):
+    rng = _rng(T * 1000 + E)
+    idx = rng.integers(-1, E, size=(T, K)).astype(np.int64)  # -1 entries are skipped
+    per_rank, cnt, in_rank = oracle.layout(idx, E, R)
+    valid = idx[idx >= 0]
+    assert np.array_equal(cnt, np.bincount(valid, minlength=E).astype(np.int32))
+    epr = E // R
+    want = np.zeros((T, R), bool)
+    for t in range(T):
+        for e in idx[t]:
+            if e >= 0:
+                want[t, e // epr] = True
+    assert np.array_equal(in_rank, want)
+    assert np.array_equal(per_rank, want.sum(0).astype(np.int32))
+
+
+def test_layout_duplicate_expert_counts_rank_once(oracle):
+    idx = np.array([[3, 3, 3, 1]], np.int64)
+    per_rank, cnt, in_rank = oracle.layout(idx, 4, 2)
+    assert cnt.tolist() == [0, 1, 0, 3]
+    assert per_rank.tolist() == [1, 1]  # token counted once per rank although three ids hit rank 1
+    assert in_rank.tolist() == [[True, True]]
+
+
+def test_layout_rejects_out_of_range(oracle):
+    with pytest.raises(ValueError):
+        oracle.layout(np.array([[0, 8]], np.int64), 8, 1)
+
+
+def test_offsets_are_exclusive_cumsum_with_triplets(oracle):
+    cnt = _rng(1).integers(0, 50, size=37).astype(np.int32)
+    off, trip = oracle.offsets(cnt, 99)
+    want = np.concatenate([[0], np.cumsum(cnt)[:-1]]).astype(np.int32)
+    assert np.array_equal(off, want)
+    assert np.array_equal(trip.reshape(-1, 3)[:, 0], cnt)
+    assert np.array_equal(trip.reshape(-1, 3)[:, 1], want)
+    assert (trip.reshape(-1, 3)[:, 2] == 99).all()
+
+
+def test_send_token_idx_brute_force_definition(oracle):
+    rng = _rng(2)
+    idx = rng.integers(-1, 5, size=(23, 4)).astype(np.int64)
+    pos = oracle.send_token_idx(idx, 5).reshape(-1)
+    flat = idx.reshape(-1)
+    for i, e in enumerate(flat):
+        if e < 0:
+            assert pos[i] == -1
+        else:
+            assert pos[i] == sum(1 for j in range(i) if flat[j] == e)
+
+
+@pytest.mark.parametrize("T,K,E", [(4096, 8, 256), (777, 6, 64)])
+def test_permutation_is_the_stable_sort_by_expert(oracle, T, K, E):
+    ids, _ = synth.sigmoid_zipf_routing(T, E, K, seed=44)
+    idx = ids.numpy()
+    _, cnt, _ = oracle.layout(idx, E, 1)
+    off, _ = oracle.offsets(cnt, T)
+    pos = oracle.send_token_idx(idx, E)
+    row = oracle.rows_from_pos(idx, off, pos, E).reshape(-1)
+    order = np.argsort(idx.reshape(-1), kind="stable")
+    # entry order[p] must land on row p
+    assert np.array_equal(row[order], np.arange(T * K, dtype=np.int32))
+    # bijection onto [0, A)
+    assert np.array_equal(np.sort(row), np.arange(T * K))
+
+
+def test_recv_bookkeeping_one_rank_closed_form(oracle):
+    cnt = _rng(3).integers(0, 9, size=16).astype(np.int32)
+    off, trip = oracle.offsets(cnt, 40)
+    total, rc, ro, tpe, mx = oracle.recv_bookkeeping(trip, 1, 16)
+    assert total == cnt.sum()
+    assert np.array_equal(rc, np.cumsum(cnt).astype(np.int32))
+    assert np.array_equal(ro, off)
+    assert np.array_equal(tpe, cnt.astype(np.int64))
+    assert mx == 40
+
+
+def test_recv_bookkeeping_two_ranks_hand_example(oracle):
+    # rank "me" owns 2 local experts; source ranks 0 and 1 send (count, offset, bs):
+    #   src0: le0 (3, 10, 7)  le1 (0, 13, 7)      src1: le0 (2, 0, 5)   le1 (4, 2, 5)
+    recv = np.array([3, 10, 7, 0, 13, 7, 2, 0, 5, 4, 2, 5], np.int32)
+    total, rc, ro, tpe, mx = oracle.recv_bookkeeping(recv, 2, 2)
+    # order (le0,s0) (le0,s1) (le1,s0) (le1,s1): counts 3,2,0,4 -> inclusive cumsum 3,5,5,9
+    assert rc.tolist() == [3, 5, 5, 9]
+    assert ro.tolist() == [10, 0, 13, 2]
+    assert tpe.tolist() == [5, 4]
+    assert total == 9 and mx == 7
+
+
+# ------------------------------------------------------------------ bf16 rounding
+def test_bf16_rounding_matches_torch(oracle):
+    x = torch.randn(20000, generator=torch.Generator().manual_seed(5)) * 100
+    x[:8] = torch.tensor([0.0, -0.0, 1.0, 1.00390625, 1.01171875, 3.3895313892515355e38, 65504.0, 1e-40])
+    got = oracle.f32_to_bf16_bits(x.numpy())
+    want = synth.bf16_bits(x.bfloat16())
+    assert np.array_equal(got, want)
+    one = np.array([oracle.lib().cam_oracle_f32_to_bf16(float(v)) for v in x[:64].tolist()], np.uint16)
+    assert np.array_equal(one, want[:64])
+
+
+# ------------------------------------------------------------------ token quantisation
+def _quant_ref_f32(xf, variant):
+    """Vectorised float32 restatement used as an independent implementation (numpy, not C)."""
+    m = np.max(np.abs(xf), axis=1).astype(np.float32)
+    if variant == 1:
+        s = np.float32(127.0) / (m + np.float32(1e-12))
+    else:
+        with np.errstate(divide="ignore"):
+            s = np.float32(127.0) / m
+    q = np.rint(xf * s[:, None]).astype(np.int32)
+    inv = np.float32(1.0) / s
+    if variant == 2:
+        zero = m == 0
+        q[zero] = 0
+        inv[zero] = 0
+    return q.astype(np.int8), inv.astype(np.float32)
+
+
+@pytest.mark.parametrize("variant", [1, 2])
+def test_quant_invariants_and_numpy_cross_check(oracle, variant):
+    x = synth.normal_bf16(257, 1024, seed=6)
+    bits = synth.bf16_bits(x)
+    q, s = oracle.quant_rows(bits, variant)
+    xf = x.float().numpy()
+    q_np, s_np = _quant_ref_f32(xf, variant)
+    assert np.array_equal(q, q_np)
+    assert np.array_equal(s.view(np.uint32), s_np.view(np.uint32))
+    assert (np.abs(q.astype(np.int32)).max(axis=1) == 127).all()
+    # reconstruction error bounded by half a step
+    err = np.abs(xf - q.astype(np.float32) * s[:, None])
+    assert (err <= s[:, None] * 0.5 * (1 + 1e-4)).all()
+    # against exact arithmetic: scale_out ~ max/127 and q ~ rint(x*127/max) up to rare ties
+    m = np.abs(xf.astype(np.float64)).max(axis=1)
+    assert np.allclose(s, m / 127.0, rtol=3e-7)
+    q64 = np.rint(xf.astype(np.float64) * 127.0 / m[:, None])
+    assert (q64 != q).mean() < 1e-3 and np.abs(q64 - q).max() <= 1
+
+
+def test_quant_special_rows(oracle):
+    H = 64
+    rows = np.zeros((5, H), np.float32)
+    rows[0] = 3.0 * np.where(np.arange(H) % 2 == 0, 1, -1)  # equal magnitudes -> all +-127
+    rows[1] = 2.0 ** -(np.arange(H) % 7)                      # powers of two: 127 * 2^-j
+    rows[2] = 0.0                                             # all-zero row
+    rows[3, 0] = 1e-13                                        # the epsilon matters here
+    rows[4] = np.linspace(-1, 1, H)
+    bits = synth.bf16_bits(torch.from_numpy(rows).bfloat16())
+    xf = oracle.bf16_bits_to_f32(bits)
+    for variant in (1, 2):
+        q, s = oracle.quant_rows(bits, variant)
+        assert (np.abs(q[0]) == 127).all() and (np.sign(q[0]) == np.sign(rows[0])).all()
+        assert np.array_equal(q[1], np.rint(127.0 * xf[1].astype(np.float64)).astype(np.int8))
+        assert (q[2] == 0).all()
+    q1, s1 = oracle.quant_rows(bits, 1)
+    q2, s2 = oracle.quant_rows(bits, 2)
+    # zero row: variant 1 keeps the reference's finite scale 1/(127/1e-12); variant 2 is defined as 0
+    assert s1[2] == np.float32(1.0) / (np.float32(127.0) / np.float32(1e-12)) and s2[2] == 0.0
+    # tiny row: with the epsilon the maximum maps to 127*m/(m+1e-12), without it to exactly 127
+    m = float(xf[3, 0])
+    assert q1[3, 0] == int(np.rint(127.0 * m / (m + 1e-12))) and q1[3, 0] < 127
+    assert q2[3, 0] == 127
+    # ordinary rows: both variants agree bit for bit (epsilon vanishes in float32)
+    assert np.array_equal(q1[4], q2[4]) and s1[4] == s2[4]
+
+
+def test_dispatch_rows_and_triples(oracle):
+    T, K, E, H = 50, 4, 8, 64
+    ids, _ = synth.softmax_topk_routing(T, E, K, seed=7)
+    idx = ids.numpy().copy()
+    idx[3, 1] = -1
+    x = synth.normal_bf16(T, H, seed=8)
+    bits = synth.bf16_bits(x)
+    _, cnt, _ = oracle.layout(idx, E, 1)
+    off, _ = oracle.offsets(cnt, T)
+    pos = oracle.send_token_idx(idx, E)
+    total = int(cnt.sum())
+    assert total == T * K - 1
+    out, scales, src = oracle.dispatch(bits, idx, off, pos, E, 0, total)
+    src = src.reshape(-1, 3)
+    for r in range(total):
+        _, t, k = src[r]
+        assert idx[t, k] >= 0 and off[idx[t, k]] + pos[t, k] == r
+        assert np.array_equal(out[r], bits[t])
+    outq, sq, _ = oracle.dispatch(bits, idx, off, pos, E, 1, total)
+    q_all, s_all = oracle.quant_rows(bits, 1)
+    for r in range(total):
+        t = src[r, 1]
+        assert np.array_equal(outq[r], q_all[t]) and sq[r] == s_all[t]
+    # rows of one expert are contiguous and in ascending flat order
+    flat = (src[:, 1] * K + src[:, 2])
+    experts = idx.reshape(-1)[flat]
+    assert (np.diff(experts) >= 0).all()
+    for e in range(E):
+        assert (np.diff(flat[experts == e]) > 0).all()
+
+
+# ------------------------------------------------------------------ GEMM and epilogues
+def test_gmm_int32_matches_int64_matmul(oracle):
+    rng = _rng(9)
+    G, Kd, N = 5, 96, 40
+    sizes = np.array([7, 0, 13, 1, 4])
+    gl = np.cumsum(sizes).astype(np.int64)
+    a = rng.integers(-128, 128, size=(int(gl[-1]), Kd)).astype(np.int8)
+    w = rng.integers(-128, 128, size=(G, Kd, N)).astype(np.int8)
+    c = oracle.gmm_int32(a, w, gl)
+    m0 = 0
+    for g in range(G):
+        want = a[m0:gl[g]].astype(np.int64) @ w[g].astype(np.int64)
+        assert np.array_equal(c[m0:gl[g]], want.astype(np.int32))
+        m0 = gl[g]
+
+
+def test_gmm_int32_extreme_values_do_not_overflow(oracle):
+    Kd = 7168
+    a = np.full((1, Kd), -128, np.int8)
+    w = np.full((1, Kd, 2), -128, np.int8)
+    c = oracle.gmm_int32(a, w, np.array([1], np.int64))
+    assert c[0, 0] == Kd * 128 * 128 and c[0, 0] < 2 ** 31
+
+
+def test_expf_spec_accuracy_and_edges(oracle):
+    xs = np.concatenate([np.linspace(-87.0, 88.0, 40001), _rng(10).normal(0, 5, 20000)]).astype(np.float32)
+    got = np.array([oracle.expf(float(v)) for v in xs], np.float64)
+    want = np.exp(xs.astype(np.float64))
+    rel = np.abs(got - want) / want
+    assert rel.max() < 2.5e-7, rel.max()  # about 2 ulp of float32
+    assert oracle.expf(0.0) == 1.0
+    assert oracle.expf(-200.0) == 0.0 and math.isinf(oracle.expf(100.0))
+    assert math.isnan(oracle.expf(float("nan")))
+    mono = np.array([oracle.expf(float(v)) for v in np.linspace(-3, 3, 5001, dtype=np.float32)])
+    assert (np.diff(mono) >= 0).all()
+
+
+def test_silu_against_float64(oracle):
+    ts = _rng(11).normal(0, 4, 5000).astype(np.float32)
+    got = np.array([oracle.silu(float(t)) for t in ts], np.float64)
+    want = ts.astype(np.float64) / (1.0 + np.exp(-ts.astype(np.float64)))
+    assert np.allclose(got, want, rtol=5e-7, atol=1e-30)
+    assert oracle.silu(0.0) == 0.0
+    assert oracle.silu(-1000.0) == 0.0 or oracle.silu(-1000.0) == -0.0
+    assert oracle.silu(1000.0) == 1000.0
+
+
+def test_gmm1_epilogue_halves_scale_order_and_grouping(oracle):
+    rng = _rng(12)
+    G, I = 3, 8
+    sizes = np.array([4, 0, 5])
+    gl = np.cumsum(sizes).astype(np.int64)
+    M = int(gl[-1])
+    c = rng.integers(-2 ** 20, 2 ** 20, size=(M, 2 * I)).astype(np.int32)
+    ws = rng.uniform(0.0015, 0.0045, size=(G, 2 * I)).astype(np.float32)
+    xs = rng.uniform(0.01, 0.05, size=M).astype(np.float32)
+    d = oracle.gmm1_epilogue(c, ws, xs, gl)
+    grp = np.repeat(np.arange(G), sizes)
+    t32 = (c.astype(np.float32) * ws[grp]) * xs[:, None]  # weight scale first, then token scale
+    # right half is the dequantised value itself, bit for bit
+    assert np.array_equal(d[:, I:].view(np.uint32), t32[:, I:].view(np.uint32))
+    # the other association differs somewhere, so the order is really pinned
+    t_other = c.astype(np.float32) * (ws[grp] * xs[:, None])
+    assert not np.array_equal(t_other[:, I:].view(np.uint32), t32[:, I:].view(np.uint32))
+    # left half is SiLU of the dequantised value
+    t64 = t32[:, :I].astype(np.float64)
+    assert np.allclose(d[:, :I], t64 / (1 + np.exp(-t64)), rtol=1e-6, atol=1e-30)
+    assert not np.allclose(d[:, :I], t32[:, :I])  # and not the identity
+
+
+def test_swiglu_quant_definition(oracle):
+    rng = _rng(13)
+    M, I = 9, 64
+    d = rng.normal(0, 3, size=(M, 2 * I)).astype(np.float32)
+    d[4] = 0.0
+    q, s = oracle.swiglu_quant(d)
+    y = d[:, :I] * d[:, I:]
+    m = np.abs(y).max(axis=1)
+    inv127 = np.float32(1.0) / np.float32(127.0)
+    want_s = (m * inv127).astype(np.float32)
+    want_s[4] = 0
+    assert np.array_equal(s.view(np.uint32), want_s.view(np.uint32))
+    with np.errstate(divide="ignore", invalid="ignore"):
+        rcp = np.float32(1.0) / m
+        want_q = np.rint((y * np.float32(127.0)) * rcp[:, None])
+    want_q[4] = 0
+    assert np.array_equal(q, want_q.astype(np.int8))
+    assert (q[4] == 0).all()
+    live = [i for i in range(M) if i != 4]
+    assert (np.abs(q[live].astype(int)).max(axis=1) == 127).all()
+    # gate*up really is left*right: swapping in a wrong pairing changes the result
+    assert not np.array_equal(y, d[:, :I] * d[:, :I])
+    # m * (1/127) is not always m / 127: the constant is rounded first
+    mm = np.float32(1.0) + np.arange(1, 4000, dtype=np.float32) * np.float32(1e-3)
+    assert (mm * inv127 != mm / np.float32(127.0)).any()
+
+
+def test_gmm2_epilogue_bits(oracle):
+    rng = _rng(14)
+    G, H = 2, 16
+    gl = np.array([3, 7], np.int64)
+    c = rng.integers(-2 ** 22, 2 ** 22, size=(7, H)).astype(np.int32)
+    ws = rng.uniform(0.0015, 0.0045, size=(G, H)).astype(np.float32)
+    ys = rng.uniform(0.001, 0.01, size=7).astype(np.float32)
+    out = oracle.gmm2_epilogue(c, ws, ys, gl)
+    grp = np.array([0, 0, 0, 1, 1, 1, 1])
+    v = (c.astype(np.float32) * ws[grp]) * ys[:, None]
+    want = synth.bf16_bits(torch.from_numpy(v).bfloat16())
+    assert np.array_equal(out, want)
+
+
+# ------------------------------------------------------------------ combine
+def test_combine_sequential_fp32_semantics(oracle):
+    rng = _rng(15)
+    T, K, H, A = 6, 8, 32, 60
+    y = torch.from_numpy(rng.normal(0, 1, size=(A, H)).astype(np.float32)).bfloat16()
+    bits = synth.bf16_bits(y)
+    row_of = rng.permutation(A)[: T * K].reshape(T, K).astype(np.int32)
+    row_of[2, 3] = -1
+    w = rng.uniform(0, 1, size=(T, K)).astype(np.float32)
+    out = oracle.combine(bits, row_of, w)
+    yf = y.float().numpy()
+    acc = np.zeros((T, H), np.float32)
+    for k in range(K):  # ascending k, multiply rounded, then add rounded
+        ok = row_of[:, k] >= 0
+        p = yf[np.maximum(row_of[:, k], 0)] * w[:, k][:, None]
+        acc = np.where(ok[:, None], acc + p, acc)
+    want = synth.bf16_bits(torch.from_numpy(acc).bfloat16())
+    assert np.array_equal(out, want)
+    # float64 cross-check within bf16 rounding
+    acc64 = np.zeros((T, H))
+    for k in range(K):
+        ok = (row_of[:, k] >= 0)[:, None]
+        acc64 += np.where(ok, yf[np.maximum(row_of[:, k], 0)].astype(np.float64) * w[:, k][:, None], 0)
+    got = oracle.bf16_bits_to_f32(out).astype(np.float64)
+    assert np.allclose(got, acc64, rtol=2 ** -8, atol=1e-6)
+
+
+def test_combine_identity_mean_and_no_fma(oracle):
+    H = 16
+    y = torch.arange(1, 4 * H + 1, dtype=torch.float32).view(4, H).bfloat16()
+    bits = synth.bf16_bits(y)
+    # K = 1, weight 1 -> the un-permute alone
+    out = oracle.combine(bits, np.array([[2], [0], [3], [1]], np.int32), np.ones((4, 1), np.float32))
+    assert np.array_equal(out, bits[[2, 0, 3, 1]])
+    # equal weights -> mean
+    out = oracle.combine(bits, np.array([[0, 1, 2, 3]], np.int32), np.full((1, 4), 0.25, np.float32))
+    want = synth.bf16_bits((y.float().sum(0, keepdim=True) * 0.25).bfloat16())
+    assert np.array_equal(out, want)
+    # a*b + c with a separately rounded product differs from a fused multiply-add here
+    a = np.float32(1.0 + 2.0 ** -7)          # exactly representable in bf16
+    wv = np.float32(1.0 + 2.0 ** -23)
+    prod = np.float32(a * wv)                 # rounded product
+    c = -prod
+    yb = synth.bf16_bits(torch.tensor([[float(a)] * 8, [1.0] * 8]).bfloat16())
+    out = oracle.combine(yb, np.array([[0, 1]], np.int32), np.array([[wv, c]], np.float32))
+    assert (oracle.bf16_bits_to_f32(out) == 0.0).all()  # fused arithmetic would leave a residue
+
+
+def test_rows_from_src_info_inverts_dispatch(oracle):
+    T, K, E, H = 31, 3, 6, 16
+    ids, _ = synth.softmax_topk_routing(T, E, K, seed=16)
+    idx = ids.numpy()
+    _, cnt, _ = oracle.layout(idx, E, 1)
+    off, _ = oracle.offsets(cnt, T)
+    pos = oracle.send_token_idx(idx, E)
+    x = synth.normal_bf16(T, H, seed=17)
+    _, _, src = oracle.dispatch(synth.bf16_bits(x), idx, off, pos, E, 0, T * K)
+    assert np.array_equal(oracle.rows_from_src_info(src, T * K, T, K), oracle.rows_from_pos(idx, off, pos, E))
+
+
+# ------------------------------------------------------------------ whole layer
+def test_fused_layer_is_the_composition_and_close_to_exact_math(oracle):
+    d = synth.ut_recipe(batch_size=24, hidden=256, intermediate=128, num_experts=6, top_k=4, seed=42)
+    bits = synth.bf16_bits(d["x"])
+    idx = d["ids"].numpy().astype(np.int64)
+    out, etn, dbg = oracle.fused_layer(bits, idx, d["gates"].numpy(), d["w1"].numpy(), d["w1_scale"].numpy(),
+                                       d["w2"].numpy(), d["w2_scale"].numpy(), debug=True)
+    T, K = idx.shape
+    E = 6
+    assert np.array_equal(etn, np.bincount(idx.reshape(-1), minlength=E))
+    # exact-arithmetic model of the same pipeline (float64 everywhere except the two int8 roundings)
+    xf = d["x"].double().numpy()
+    w1 = d["w1"].double().numpy() * d["w1_scale"].double().numpy()[:, None, :]
+    w2 = d["w2"].double().numpy() * d["w2_scale"].double().numpy()[:, None, :]
+    I = 128
+    want = np.zeros_like(xf)
+    for t in range(T):
+        m = np.abs(xf[t]).max()
+        xq = np.rint(xf[t] * 127 / m) * (m / 127)
+        for k in range(K):
+            e = idx[t, k]
+            h1 = xq @ w1[e]
+            y = h1[:I] / (1 + np.exp(-h1[:I])) * h1[I:]
+            my = np.abs(y).max()
+            yq = np.rint(y * 127 / my) * (my / 127)
+            want[t] += d["gates"][t, k].item() * (yq @ w2[e])
+    got = oracle.bf16_bits_to_f32(out).astype(np.float64)
+    scale = np.abs(want).max()
+    assert np.abs(got - want).max() <= 0.02 * scale
+    assert np.corrcoef(got.reshape(-1), want.reshape(-1))[0, 1] > 0.9995
+
+
+def test_fused_layer_active_mask_prefix(oracle):
+    d = synth.ut_recipe(batch_size=10, hidden=128, intermediate=64, num_experts=4, top_k=2, seed=43)
+    bits = synth.bf16_bits(d["x"])
+    idx = d["ids"].numpy().astype(np.int64)
+    args = (d["gates"].numpy(), d["w1"].numpy(), d["w1_scale"].numpy(), d["w2"].numpy(), d["w2_scale"].numpy())
+    full, _ = oracle.fused_layer(bits, idx, *args)
+    part, etn = oracle.fused_layer(bits, idx, *args, n_active=6)
+    assert np.array_equal(part[:6], full[:6])  # tokens are independent
+    assert (part[6:] == 0).all()
+    assert etn.sum() == 6 * 2

@@ -1,0 +1,74 @@
+// Device-side helpers shared by the CAM kernels (gfx950, 64-wide wavefronts).
+#ifndef CAM_DEVICE_H_
+#define CAM_DEVICE_H_
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace cam {
+
+constexpr int kWave = 64;
+
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef int v2i __attribute__((ext_vector_type(2)));
+typedef int v16i __attribute__((ext_vector_type(16)));
+typedef float v4f __attribute__((ext_vector_type(4)));
+typedef unsigned int v4u __attribute__((ext_vector_type(4)));
+typedef unsigned int v2u __attribute__((ext_vector_type(2)));
+
+__device__ __forceinline__ float bf16_bits_to_f32(uint32_t bits16)
+{
+    return __uint_as_float(bits16 << 16);
+}
+
+// Round-to-nearest-even fp32 -> bf16 bit pattern (NaN stays a quiet NaN).
+__device__ __forceinline__ uint32_t f32_to_bf16_bits(float f)
+{
+    uint32_t u = __float_as_uint(f);
+    if ((u & 0x7fffffffu) > 0x7f800000u) {
+        return (u >> 16) | 0x0040u;
+    }
+    uint32_t lsb = (u >> 16) & 1u;
+    u += 0x7fffu + lsb;
+    return u >> 16;
+}
+
+__device__ __forceinline__ int lane_id()
+{
+    return (int)__builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u));
+}
+
+__device__ __forceinline__ float wave_max(float v)
+{
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) {
+        v = fmaxf(v, __shfl_xor(v, off, kWave));
+    }
+    return v;
+}
+
+__device__ __forceinline__ int wave_sum(int v)
+{
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) {
+        v += __shfl_xor(v, off, kWave);
+    }
+    return v;
+}
+
+// Inclusive scan across the 64 lanes of a wave.
+__device__ __forceinline__ int wave_inclusive_scan(int v, int lane)
+{
+#pragma unroll
+    for (int off = 1; off < kWave; off <<= 1) {
+        int n = __shfl_up(v, off, kWave);
+        if (lane >= off) {
+            v += n;
+        }
+    }
+    return v;
+}
+
+}  // namespace cam
+
+#endif  // CAM_DEVICE_H_

@@ -1,0 +1,125 @@
+// Host-callable launchers of the CAM HIP kernels.  Pointers are device pointers unless noted.
+// Each launcher only enqueues work on `stream`; it never allocates or synchronises.
+#ifndef CAM_KERNELS_H_
+#define CAM_KERNELS_H_
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace cam {
+
+constexpr int kMaxExperts = 512;   // E <= 512 on every CAM operator
+constexpr int kMaxRanks = 384;
+constexpr int kMaxTopk = 16;
+constexpr int kGemmTileM = 128;    // rows per GEMM tile (tile table granularity)
+constexpr int kMaxListExperts = 64;  // per-expert weight tensors that fit in the kernel arguments
+
+// ---------------------------------------------------------------------------------------------
+// Routing plan: counts, offsets, within-expert ranks, receive bookkeeping, GEMM tile table.
+struct PlanArgs {
+    const void *idx;          // [T,K] int32 or int64
+    int idx_is64;
+    const uint8_t *mask;      // optional [T] bool; the number of set entries is the active prefix
+    int T, K, E;
+    int32_t *pos;             // [T,K]  required: rank within expert, -1 where skipped
+    int32_t *dst_row;         // [T,K]  optional: off[e] + pos, -1 where skipped
+    int32_t *cnt;             // [E]    optional
+    int32_t *off;             // [E]    optional exclusive scan of cnt
+    int32_t *recv_off;        // [E]    optional (== off on one rank)
+    int32_t *recv_count;      // [E]    optional inclusive scan
+    int64_t *tokens_per_expert;  // [E] optional
+    int64_t *group_list;      // [E]    optional cumulative rows, int64
+    int64_t *total;           // [1]    optional
+    int32_t *per_rank_zero;   // [R]    optional: zeroed here so a later kernel can accumulate into it
+    int R;
+    int32_t *tiles;           // optional GEMM tile table: [0]=tile count, then int4 (expert, m0, rows, 0) from [4]
+};
+hipError_t launch_plan(const PlanArgs &a, hipStream_t stream);
+
+// isTokenInRank / numTokensPerRank (per_rank must have been zeroed on the same stream).
+struct InRankArgs {
+    const void *idx;
+    int idx_is64;
+    int T, K, E, R;
+    void *in_rank;     // [T,R] int32 or 1-byte
+    int in_rank_bytes; // 4 or 1
+    int32_t *per_rank; // [R]
+};
+hipError_t launch_in_rank(const InRankArgs &a, hipStream_t stream);
+
+// NotifyDispatch on one rank: exclusive scan + triplets.
+hipError_t launch_notify_scan(const int32_t *cnt, int E, int num_tokens, int32_t *off, int32_t *send_data,
+                              int32_t *recv_data, hipStream_t stream);
+
+// Tile table from a group list (cumulative or per-expert counts, int64).
+hipError_t launch_build_tiles(const int64_t *group_list, int cumulative, int G, int64_t max_rows, int max_tiles,
+                              int32_t *tiles, hipStream_t stream);
+
+// ---------------------------------------------------------------------------------------------
+// Permute (+ per-token int8 quantisation).
+struct DispatchArgs {
+    const uint16_t *x;   // [T,H] bf16 bits
+    const int32_t *idx;  // [T,K]
+    const int32_t *send_offset, *send_token_idx, *recv_offset, *recv_count;  // row = see cam_mi355x.h
+    const int32_t *dst_row;  // if non-null, used instead of the four arrays above
+    int T, K, H, E;
+    int64_t A;           // rows in the outputs
+    int quant;           // 0 copy, 1 = epsilon variant, 2 = no-epsilon variant
+    void *out;           // [A,H] bf16 bits or int8
+    float *scales;       // [A]   (quant only)
+    int32_t *src_info;   // [3A]  optional
+    int src_rank;
+};
+hipError_t launch_dispatch(const DispatchArgs &a, hipStream_t stream);
+
+// ---------------------------------------------------------------------------------------------
+// Combine.
+hipError_t launch_invert_src_info(const int32_t *src_info, int64_t A, int T, int K, int32_t *slot_row,
+                                  hipStream_t stream);
+struct CombineArgs {
+    const uint16_t *y;        // [A,H] bf16 bits
+    const int32_t *slot_row;  // [T,K] row of slot (t,k) (<0: skip)
+    const int32_t *src_info;  // optional: when set, slot_row entries are verified against the triples
+    const float *w;           // [T,K]
+    int T, K, H;
+    int64_t A;
+    const int32_t *t_active;  // optional device scalar: tokens >= *t_active produce zero rows
+    uint16_t *out;            // [T,H]
+};
+hipError_t launch_combine(const CombineArgs &a, hipStream_t stream);
+
+// ---------------------------------------------------------------------------------------------
+// Grouped int8 GEMM.
+struct WeightPtrs {
+    const int8_t *w[kMaxListExperts];   // used when per_expert != 0
+    const float *s[kMaxListExperts];
+};
+enum GemmEpilogue { kEpiInt32 = 0, kEpiSwiglu = 1, kEpiDequantBf16 = 2 };
+struct GemmArgs {
+    const int8_t *a;       // [A,Kd] int8
+    const float *a_scale;  // [A]
+    const int8_t *w;       // stacked packed weights [G,Kd,N] (per_expert == 0)
+    const float *w_scale;  // stacked [G,N]
+    int per_expert;        // weights given per expert through `list`
+    WeightPtrs list;
+    const int32_t *tiles;  // tile table
+    int max_tiles;         // upper bound on the number of tiles (grid size)
+    int Kd, N;             // N = logical columns of the weight
+    int gate_up;           // weight prepacked with gate/up pairing
+    int epilogue;
+    void *out;             // int32 [A,N] | fp32 [A,N/2] | bf16 bits [A,N]
+};
+hipError_t launch_gemm(const GemmArgs &a, hipStream_t stream);
+
+// fp32 SwiGLU products [rows,I] -> int8 + per-row scale.  rows_dev: optional device count of valid rows.
+hipError_t launch_requant(const float *y, int64_t max_rows, int I, const int32_t *tiles_for_rows, int8_t *q,
+                          float *scale, hipStream_t stream);
+
+hipError_t launch_prepack(const int8_t *src, int8_t *dst, int G, int Kd, int N, int gate_up, hipStream_t stream);
+
+// Small utilities.
+hipError_t launch_cast_i64_to_i32(const int64_t *src, int32_t *dst, int64_t n, hipStream_t stream);
+
+}  // namespace cam
+
+#endif  // CAM_KERNELS_H_
