@@ -81,7 +81,9 @@ def main():
     torch.cuda.set_device(dev)
     props = torch.cuda.get_device_properties(dev)
     log("device: %s, %d CUs" % (props.name, props.multi_processor_count))
-    ROT = 4  # rotating buffer sets per graph: one replay = ROT steps
+    NBUF = 4   # rotating buffer sets
+    ROT = 16   # passes per graph (buffer set = pass % NBUF): one replay = ROT steps, which amortises
+               # the ~8 us a graph launch costs
     replays = max(1, (args.steps + ROT - 1) // ROT)
     warm = max(1, (args.warmup + ROT - 1) // ROT)
 
@@ -98,23 +100,24 @@ def main():
     t_disp = t_plan = t_perm = t_comb = None
 
     if want("dispatch"):
-        xs = [synth.normal_bf16(T, H, seed=44 + i).to(dev) for i in range(ROT)]
+        xs = [synth.normal_bf16(T, H, seed=44 + i).to(dev) for i in range(NBUF)]
         i32 = dict(dtype=torch.int32, device=dev)
         plan_bufs = [dict(pos=torch.empty((T, K), **i32), cnt=torch.empty(E, **i32), off=torch.empty(E, **i32),
                           roff=torch.empty(E, **i32), rcnt=torch.empty(E, **i32),
                           tpe=torch.empty(E, dtype=torch.int64, device=dev),
-                          total=torch.empty(1, dtype=torch.int64, device=dev)) for _ in range(ROT)]
+                          total=torch.empty(1, dtype=torch.int64, device=dev),
+                          ws=torch.empty(1 << 18, dtype=torch.uint8, device=dev)) for _ in range(NBUF)]
         outs = [dict(rx=torch.empty((A, H), dtype=torch.int8, device=dev),
                      sc=torch.empty(A, dtype=torch.float32, device=dev),
-                     info=torch.empty(3 * A, **i32)) for _ in range(ROT)]
+                     info=torch.empty(3 * A, **i32)) for _ in range(NBUF)]
 
         def run_plan(i):
-            p = plan_bufs[i]
+            p = plan_bufs[i % NBUF]
             _lib.call("MoeDispatchPlan", [ids, E, 1, 0, p["pos"], p["cnt"], p["off"], p["roff"], p["rcnt"], p["tpe"],
-                                          p["total"]])
+                                          p["total"]], workspace=p["ws"])
 
         def run_permute(i):
-            p, o = plan_bufs[i], outs[i]
+            p, o, i = plan_bufs[i % NBUF], outs[i % NBUF], i % NBUF
             _lib.call("MoeDispatchNormal", [xs[i], ids, p["off"], p["pos"], p["roff"], p["rcnt"], "", 1, 0, "", 1, 0,
                                             E, 2, 0, o["rx"], o["sc"], o["info"]])
 
@@ -148,7 +151,7 @@ def main():
     if want("combine"):
         import numpy as np
         plan = cam.moe_dispatch_plan(ids, E)
-        ys = [synth.normal_bf16(A, H, seed=46 + i).to(dev) for i in range(ROT)]
+        ys = [synth.normal_bf16(A, H, seed=46 + i).to(dev) for i in range(NBUF)]
         # triples as the dispatch kernel writes them
         dummy = torch.empty((A, 1024), dtype=torch.bfloat16, device=dev)
         _, _, info = cam.moe_dispatch_normal(torch.zeros((T, 1024), dtype=torch.bfloat16, device=dev), ids,
@@ -156,13 +159,13 @@ def main():
                                              plan["recv_count"], A, E)
         del dummy
         gw = gate_w.to(dev)
-        couts = [torch.empty((T, H), dtype=torch.bfloat16, device=dev) for _ in range(ROT)]
-        wss = [torch.empty(T * K * 4 + 256, dtype=torch.uint8, device=dev) for _ in range(ROT)]
+        couts = [torch.empty((T, H), dtype=torch.bfloat16, device=dev) for _ in range(NBUF)]
+        wss = [torch.empty(T * K * 4 + 256, dtype=torch.uint8, device=dev) for _ in range(NBUF)]
 
         def comb_all():
             for i in range(ROT):
-                _lib.call("MoeCombineNormal", [ys[i], info, plan["recv_count"], gw, None, "", 1, 0, "", 1, 0, E, 0,
-                                               couts[i]], workspace=wss[i])
+                _lib.call("MoeCombineNormal", [ys[i % NBUF], info, plan["recv_count"], gw, None, "", 1, 0, "", 1, 0, E,
+                                               0, couts[i % NBUF]], workspace=wss[i % NBUF])
 
         t_comb = time_graph(graph_of(comb_all), replays, warm) / ROT
         log("combine: %.1f us -> %.0f GB/s = %.1f%% of HBM peak" % (t_comb * 1e6, comb_bytes / t_comb / 1e9,
@@ -179,14 +182,14 @@ def main():
         _, _, infod = cam.moe_dispatch_normal(torch.zeros((Td, 1024), dtype=torch.bfloat16, device=dev), idd32,
                                               pland["send_offset"], pland["send_token_idx"], pland["recv_offset"],
                                               pland["recv_count"], Td * K, E)
-        yd = [synth.normal_bf16(Td * K, H, seed=48 + i).to(dev) for i in range(ROT)]
-        od = [torch.empty((Td, H), dtype=torch.bfloat16, device=dev) for _ in range(ROT)]
+        yd = [synth.normal_bf16(Td * K, H, seed=48 + i).to(dev) for i in range(NBUF)]
+        od = [torch.empty((Td, H), dtype=torch.bfloat16, device=dev) for _ in range(NBUF)]
         gwd = gwd.to(dev)
 
         def comb_decode():
             for i in range(ROT):
-                _lib.call("MoeCombineNormal", [yd[i], infod, pland["recv_count"], gwd, None, "", 1, 0, "", 1, 0, E, 0,
-                                               od[i]], workspace=wss[i])
+                _lib.call("MoeCombineNormal", [yd[i % NBUF], infod, pland["recv_count"], gwd, None, "", 1, 0, "", 1, 0,
+                                               E, 0, od[i % NBUF]], workspace=wss[i % NBUF])
 
         t_cd = time_graph(graph_of(comb_decode), replays, warm) / ROT
         cd_bytes = synth.combine_bytes(Td, H, K)
@@ -337,7 +340,8 @@ def main():
                         "per-token int8 quant + fp32 scales; then combine: 32768 bf16 rows x 7168 -> 4096 tokens",
             "tokens": T, "hidden": H, "experts": E, "top_k": K,
             "dispatch_bytes": disp_bytes, "combine_bytes": comb_bytes,
-            "timing": "HIP graph replays bracketed by HIP events on the launch stream; %d rotating buffer sets" % ROT,
+            "timing": "HIP graph replays (%d passes each) bracketed by HIP events on the launch stream; %d rotating "
+                      "buffer sets" % (ROT, NBUF),
         },
     }
     if t_disp is not None and t_comb is not None:

@@ -162,7 +162,7 @@ CAM_API camStatus camMoeDispatchPlan(void *workspace, uint64_t workspaceSize, ca
  * (…/grouped_matmul_slice_m_per_token_dequant_swiglu_quant_multistage_workspace.h:780-818).
  * quantMode 1 (static) -> CAM_ERR_UNSUPPORTED.  epWorldSize must be 1 (reference: >= 2).
  * Limits (AK/moe_dispatch_normal/op_host/moe_dispatch_normal_tiling.cc:87-100): 1024 <= H <= 7168,
- * 0 < K <= 16, 0 < E <= 512.  H must be a multiple of 16. */
+ * 0 < K <= 16, 0 < E <= 512.  H must be a multiple of 8. */
 CAM_API camStatus camMoeDispatchNormalGetWorkspaceSize(
     const camTensor *x, const camTensor *topkIdx, const camTensor *sendOffset, const camTensor *sendTokenIdx,
     const camTensor *recvOffset, const camTensor *recvCount, char *groupEp, int64_t epWorldSize,

@@ -73,7 +73,7 @@ def test_moe_dispatch_normal_validation():
     assert _lib.phase1("MoeDispatchNormal", _dispatch_args(quant=2))[0] == CAM_OK
     assert _lib.phase1("MoeDispatchNormal", _dispatch_args(H=512))[0] == CAM_ERR_RANGE
     assert _lib.phase1("MoeDispatchNormal", _dispatch_args(H=7184))[0] == CAM_ERR_RANGE
-    assert _lib.phase1("MoeDispatchNormal", _dispatch_args(H=1032))[0] == CAM_ERR_ALIGN
+    assert _lib.phase1("MoeDispatchNormal", _dispatch_args(H=1028))[0] == CAM_ERR_ALIGN
     assert _lib.phase1("MoeDispatchNormal", _dispatch_args(K=17, E=32))[0] == CAM_ERR_RANGE
     assert _lib.phase1("MoeDispatchNormal", _dispatch_args(E=513))[0] == CAM_ERR_RANGE
     assert _lib.phase1("MoeDispatchNormal", _dispatch_args(quant=4))[0] == CAM_ERR_RANGE

@@ -114,7 +114,7 @@ def _dispatch_case(gpu, oracle, T, K, E, H, quant_mode, seed, neg=0.0, zero_rows
 
 @pytest.mark.parametrize("quant_mode", [0, 2, 3])
 @pytest.mark.parametrize("T,K,E,H", [(1, 1, 2, 1024), (37, 3, 8, 1024), (128, 2, 8, 1024), (64, 8, 32, 7168),
-                                      (50, 16, 64, 4096), (19, 4, 16, 2064)])
+                                      (50, 16, 64, 4096), (19, 4, 16, 2064), (9, 2, 4, 1032)])
 def test_dispatch_normal_bit_exact(gpu, oracle, T, K, E, H, quant_mode):
     announce("dispatch T=%d K=%d E=%d H=%d quant=%d" % (T, K, E, H, quant_mode))
     _dispatch_case(gpu, oracle, T, K, E, H, quant_mode, seed=T + H)

@@ -329,6 +329,7 @@ camStatus camDispatchLayoutGetWorkspaceSize(const camTensor *topkIdx, int64_t nu
     }
     Carver c;
     const uint64_t o_pos = c.take((uint64_t)numTokens * numTopk * 4);
+    const uint64_t o_hist = c.take(cam::plan_workspace_bytes(numTokens, numTopk, (int)numExperts));
     cam::PlanArgs p{};
     p.idx = topkIdx->data;
     p.idx_is64 = topkIdx->dtype == CAM_DT_INT64;
@@ -348,8 +349,9 @@ camStatus camDispatchLayoutGetWorkspaceSize(const camTensor *topkIdx, int64_t nu
     r.in_rank = isTokenInRank->data;
     r.in_rank_bytes = isTokenInRank->dtype == CAM_DT_INT32 ? 4 : 1;
     r.per_rank = (int32_t *)numTokensPerRank->data;
-    auto run = [p, r, o_pos](void *ws, hipStream_t s) mutable -> hipError_t {
+    auto run = [p, r, o_pos, o_hist](void *ws, hipStream_t s) mutable -> hipError_t {
         p.pos = (int32_t *)((char *)ws + o_pos);
+        p.hist_ws = (int32_t *)((char *)ws + o_hist);
         hipError_t e = cam::launch_plan(p, s);
         if (e != hipSuccess) {
             return e;
@@ -484,8 +486,12 @@ camStatus camMoeDispatchPlanGetWorkspaceSize(const camTensor *topkIdx, int64_t n
     p.recv_count = recvCount ? (int32_t *)recvCount->data : nullptr;
     p.tokens_per_expert = numRecvTokensPerExpert ? (int64_t *)numRecvTokensPerExpert->data : nullptr;
     p.total = totalRecvTokens ? (int64_t *)totalRecvTokens->data : nullptr;
-    auto run = [p](void *, hipStream_t s) -> hipError_t { return cam::launch_plan(p, s); };
-    return finish_phase1(kOpPlan, 0, run, workspaceSize, executor);
+    const uint64_t ws_bytes = align_up(cam::plan_workspace_bytes(T, K, (int)numExperts));
+    auto run = [p](void *ws, hipStream_t s) mutable -> hipError_t {
+        p.hist_ws = (int32_t *)ws;
+        return cam::launch_plan(p, s);
+    };
+    return finish_phase1(kOpPlan, ws_bytes, run, workspaceSize, executor);
 }
 
 camStatus camMoeDispatchPlan(void *workspace, uint64_t workspaceSize, camOpExecutor *executor, camStream_t stream)
@@ -541,8 +547,8 @@ camStatus camMoeDispatchNormalGetWorkspaceSize(const camTensor *x, const camTens
     if (H < 1024 || H > 7168) {
         return fail(CAM_ERR_RANGE, "hidden size %lld outside [1024, 7168]", (long long)H);
     }
-    if (H % 16 != 0) {
-        return fail(CAM_ERR_ALIGN, "hidden size %lld must be a multiple of 16", (long long)H);
+    if (H % 8 != 0) {
+        return fail(CAM_ERR_ALIGN, "hidden size %lld must be a multiple of 8", (long long)H);
     }
     if (topkIdx->sizes[0] != T) {
         return fail(CAM_ERR_SHAPE, "x and topkIdx must agree on dimension 0");
@@ -1060,6 +1066,7 @@ camStatus camFusedDeepMoeGetWorkspaceSize(const camTensor *x, const camTensor *e
     const uint64_t o_pos = c.take((uint64_t)A * 4);
     const uint64_t o_row = c.take((uint64_t)A * 4);
     const uint64_t o_tiles = c.take(tile_table_bytes(max_tiles));
+    const uint64_t o_hist = c.take(cam::plan_workspace_bytes(T, K, (int)Epr));
     const uint64_t o_x1 = c.take((uint64_t)A * H);
     const uint64_t o_x1s = c.take((uint64_t)A * 4);
     const uint64_t o_prod = c.take((uint64_t)A * I * 4);
@@ -1099,6 +1106,7 @@ camStatus camFusedDeepMoeGetWorkspaceSize(const camTensor *x, const camTensor *e
         p.dst_row = row;
         p.tokens_per_expert = etn;
         p.tiles = tiles;
+        p.hist_ws = (int32_t *)(w + o_hist);
         hipError_t e = cam::launch_plan(p, s);
         if (e != hipSuccess) return e;
 

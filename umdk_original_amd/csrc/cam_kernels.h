@@ -11,7 +11,7 @@ namespace cam {
 constexpr int kMaxExperts = 512;   // E <= 512 on every CAM operator
 constexpr int kMaxRanks = 384;
 constexpr int kMaxTopk = 16;
-constexpr int kGemmTileM = 128;    // rows per GEMM tile (tile table granularity)
+constexpr int kGemmTileM = 256;    // rows per GEMM tile (tile table granularity)
 constexpr int kMaxListExperts = 64;  // per-expert weight tensors that fit in the kernel arguments
 
 // ---------------------------------------------------------------------------------------------
@@ -33,7 +33,9 @@ struct PlanArgs {
     int32_t *per_rank_zero;   // [R]    optional: zeroed here so a later kernel can accumulate into it
     int R;
     int32_t *tiles;           // optional GEMM tile table: [0]=tile count, then int4 (expert, m0, rows, 0) from [4]
+    int32_t *hist_ws;         // required scratch of plan_workspace_bytes(T, K, E) bytes
 };
+uint64_t plan_workspace_bytes(int64_t T, int64_t K, int E);
 hipError_t launch_plan(const PlanArgs &a, hipStream_t stream);
 
 // isTokenInRank / numTokensPerRank (per_rank must have been zeroed on the same stream).

@@ -8,11 +8,12 @@
 //   receive     moe_dispatch_normal.h:486-535 (rows land at recvCount[i-1] + j; triple and scale per row)
 //
 // Design.  The reference reads a token once per top-k copy and moves every row twice (sender ->
-// window -> output).  Here one workgroup owns one token: each thread loads 16 contiguous bf16 values
-// (two 16-byte loads) exactly once, the row maximum is reduced with wave shuffles and one LDS
-// exchange, the row is quantised in registers and the 16 resulting bytes are stored with one 16-byte
-// store to each of the K destination rows.  HBM traffic is therefore the algorithmic minimum:
-// H*2 bytes read and K*H bytes written per token.
+// window -> output).  Here one wavefront owns one token: lane l loads the 16-byte chunks l, l+64, ...
+// of the row (each load instruction covers 1 KB of contiguous memory) exactly once, the row maximum
+// is reduced with wave shuffles alone (no LDS, no workgroup barrier, so waves never wait for each
+// other), the row is quantised in registers and each chunk's 8 result bytes are stored, again 512
+// contiguous bytes per instruction, to each of the K destination rows.  HBM traffic is the
+// algorithmic minimum: H*2 bytes read and K*H bytes written per token.
 #include "cam_device.h"
 #include "cam_kernels.h"
 
@@ -20,12 +21,13 @@ namespace cam {
 
 namespace {
 
-constexpr int kDispMaxWaves = 8;  // H <= 7168 -> at most 448 threads
+constexpr int kDispWaves = 4;         // tokens (waves) per workgroup
+constexpr int kDispMaxChunks = 14;    // 16-byte chunks per lane: H <= 14 * 64 * 8 = 7168
 
 // Output row of entry (t,k), or -1.
 __device__ __forceinline__ long long dispatch_row(const DispatchArgs &a, int t, int k)
 {
-    const int i = t * a.K + k;
+    const long long i = (long long)t * a.K + k;
     if (a.dst_row != nullptr) {
         return a.dst_row[i];
     }
@@ -45,50 +47,38 @@ __device__ __forceinline__ uint32_t pack4(int a, int b, int c, int d)
 }
 
 template <int QUANT>
-__global__ __launch_bounds__(kDispMaxWaves * kWave) void dispatch_kernel(DispatchArgs a)
+__global__ __launch_bounds__(kDispWaves * kWave) void dispatch_kernel(DispatchArgs a)
 {
-    __shared__ float wave_max_s[kDispMaxWaves];
-    const int t = blockIdx.x;
-    const int tid = threadIdx.x;
-    const int chunks = a.H >> 4;  // 16 elements per thread
-    const bool active = tid < chunks;
-
-    v4u lo = {0u, 0u, 0u, 0u};
-    v4u hi = {0u, 0u, 0u, 0u};
-    if (active) {
-        const v4u *src = (const v4u *)(a.x + (long long)t * a.H) + 2 * tid;
-        lo = __builtin_nontemporal_load(src);
-        hi = __builtin_nontemporal_load(src + 1);
+    const int t = blockIdx.x * kDispWaves + (threadIdx.x >> 6);
+    const int lane = threadIdx.x & (kWave - 1);
+    if (t >= a.T) {
+        return;
+    }
+    const int nch = a.H >> 3;  // 8 bf16 values per chunk
+    const v4u *src = (const v4u *)(a.x + (long long)t * a.H);
+    v4u raw[kDispMaxChunks];
+#pragma unroll
+    for (int j = 0; j < kDispMaxChunks; ++j) {
+        const int c = j * kWave + lane;
+        raw[j] = v4u{0u, 0u, 0u, 0u};
+        if (c < nch) {
+            raw[j] = __builtin_nontemporal_load(src + c);
+        }
     }
 
-    v4u q = {0u, 0u, 0u, 0u};
+    v2u q[kDispMaxChunks];
     float scale_out = 0.0f;
     if (QUANT != 0) {
-        float f[16];
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            f[2 * j] = bf16_bits_to_f32(lo[j] & 0xffffu);
-            f[2 * j + 1] = bf16_bits_to_f32(lo[j] >> 16);
-            f[8 + 2 * j] = bf16_bits_to_f32(hi[j] & 0xffffu);
-            f[8 + 2 * j + 1] = bf16_bits_to_f32(hi[j] >> 16);
-        }
         float m = 0.0f;
 #pragma unroll
-        for (int j = 0; j < 16; ++j) {
-            m = fmaxf(m, fabsf(f[j]));
+        for (int j = 0; j < kDispMaxChunks; ++j) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                m = fmaxf(m, fabsf(bf16_bits_to_f32(raw[j][i] & 0xffffu)));
+                m = fmaxf(m, fabsf(bf16_bits_to_f32(raw[j][i] >> 16)));
+            }
         }
         m = wave_max(m);
-        const int nw = (blockDim.x + kWave - 1) / kWave;
-        if (nw > 1) {
-            if ((tid & (kWave - 1)) == 0) {
-                wave_max_s[tid >> 6] = m;
-            }
-            __syncthreads();
-            m = wave_max_s[0];
-            for (int w = 1; w < nw; ++w) {
-                m = fmaxf(m, wave_max_s[w]);
-            }
-        }
         float s;
         bool zero_row = false;
         if (QUANT == 1) {
@@ -98,15 +88,16 @@ __global__ __launch_bounds__(kDispMaxWaves * kWave) void dispatch_kernel(Dispatc
             s = zero_row ? 0.0f : __fdiv_rn(127.0f, m);
         }
         scale_out = zero_row ? 0.0f : __fdiv_rn(1.0f, s);
-        int qi[16];
 #pragma unroll
-        for (int j = 0; j < 16; ++j) {
-            qi[j] = (int)rintf(__fmul_rn(f[j], s));
+        for (int j = 0; j < kDispMaxChunks; ++j) {
+            int v[8];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                v[2 * i] = (int)rintf(__fmul_rn(bf16_bits_to_f32(raw[j][i] & 0xffffu), s));
+                v[2 * i + 1] = (int)rintf(__fmul_rn(bf16_bits_to_f32(raw[j][i] >> 16), s));
+            }
+            q[j] = v2u{pack4(v[0], v[1], v[2], v[3]), pack4(v[4], v[5], v[6], v[7])};
         }
-        q[0] = pack4(qi[0], qi[1], qi[2], qi[3]);
-        q[1] = pack4(qi[4], qi[5], qi[6], qi[7]);
-        q[2] = pack4(qi[8], qi[9], qi[10], qi[11]);
-        q[3] = pack4(qi[12], qi[13], qi[14], qi[15]);
     }
 
     for (int k = 0; k < a.K; ++k) {
@@ -114,17 +105,26 @@ __global__ __launch_bounds__(kDispMaxWaves * kWave) void dispatch_kernel(Dispatc
         if (row < 0 || row >= a.A) {
             continue;
         }
-        if (active) {
-            if (QUANT != 0) {
-                v4u *dst = (v4u *)((int8_t *)a.out + row * a.H) + tid;
-                __builtin_nontemporal_store(q, dst);
-            } else {
-                v4u *dst = (v4u *)((uint16_t *)a.out + row * a.H) + 2 * tid;
-                __builtin_nontemporal_store(lo, dst);
-                __builtin_nontemporal_store(hi, dst + 1);
+        if (QUANT != 0) {
+            v2u *dst = (v2u *)((int8_t *)a.out + row * a.H);
+#pragma unroll
+            for (int j = 0; j < kDispMaxChunks; ++j) {
+                const int c = j * kWave + lane;
+                if (c < nch) {
+                    __builtin_nontemporal_store(q[j], dst + c);
+                }
+            }
+        } else {
+            v4u *dst = (v4u *)((uint16_t *)a.out + row * a.H);
+#pragma unroll
+            for (int j = 0; j < kDispMaxChunks; ++j) {
+                const int c = j * kWave + lane;
+                if (c < nch) {
+                    __builtin_nontemporal_store(raw[j], dst + c);
+                }
             }
         }
-        if (tid == 0) {
+        if (lane == 0) {
             if (QUANT != 0) {
                 a.scales[row] = scale_out;
             }
@@ -144,12 +144,10 @@ hipError_t launch_dispatch(const DispatchArgs &a, hipStream_t stream)
     if (a.T <= 0) {
         return hipSuccess;
     }
-    const int chunks = a.H / 16;
-    const int threads = ((chunks + kWave - 1) / kWave) * kWave;
-    if (a.H % 16 != 0 || threads > kDispMaxWaves * kWave) {
+    if (a.H % 8 != 0 || a.H / 8 > kDispMaxChunks * kWave) {
         return hipErrorInvalidValue;
     }
-    dim3 grid(a.T), block(threads);
+    dim3 grid((a.T + kDispWaves - 1) / kDispWaves), block(kDispWaves * kWave);
     if (a.quant == 0) {
         hipLaunchKernelGGL(dispatch_kernel<0>, grid, block, 0, stream, a);
     } else if (a.quant == 1) {

@@ -9,11 +9,13 @@
 //   GMM2 epilogue   FDM/epilogue/block/block_epilogue_per_token_dequant.hpp:665-684
 //
 // Design (not a translation of the cube/vector split above).
-//   * One workgroup = 4 waves = a tile of up to 128 rows of ONE expert x 256 packed weight columns.
-//     Every wave covers all 128 rows and its own 64 columns, so a weight byte is needed by exactly
-//     one wave: weights go straight from HBM to registers in the lane order the MFMA wants (they
-//     were laid out that way once by the prepack kernel), 16 bytes per lane, 1 KB contiguous per
-//     wave and load, double-buffered in registers one 128-deep K step ahead.  No LDS for weights.
+//   * One workgroup = 4 waves = a tile of up to 256 rows of ONE expert x 256 packed weight columns.
+//     Every wave covers all rows of the tile and its own 64 columns, so a weight byte is needed by
+//     exactly one wave: weights go straight from HBM to registers in the lane order the MFMA wants
+//     (they were laid out that way once by the prepack kernel), 16 bytes per lane, 1 KB contiguous
+//     per wave and load, through a register ring two 128-deep K steps ahead.  No LDS for weights.
+//     The grouped shape is bound by streaming the weights, so the tile is as tall as the register
+//     file allows (256 int32 accumulators per lane): every weight byte fetched feeds up to 256 rows.
 //   * Activations (shared by the 4 waves) are staged through LDS, double-buffered, with an XOR
 //     swizzle of the 16-byte chunks so that both the cooperative stores and the ds_read_b128
 //     fragment loads are bank-conflict free.
@@ -34,8 +36,8 @@ namespace cam {
 
 namespace {
 
-constexpr int kBM = kGemmTileM;  // 128 rows
-constexpr int kMF = kBM / 32;    // 4 row fragments
+constexpr int kBM = kGemmTileM;  // rows per tile
+constexpr int kMF = kBM / 32;    // row fragments per tile
 constexpr int kNF = 2;           // 2 column fragments per wave (64 columns)
 constexpr int kBK = 128;         // K bytes per main-loop step
 constexpr int kKK = kBK / 32;    // MFMA steps per main-loop step
@@ -43,6 +45,7 @@ constexpr int kThreads = 256;
 constexpr int kWaveCols = 64;
 constexpr int kBlockCols = 4 * kWaveCols;
 constexpr int kNumXcd = 8;
+constexpr int kBDepth = 3;       // weight register ring: steps in flight
 
 // LDS offset (bytes) of the 16-byte chunk `c` (0..7) of row `r` in one A stage.
 __device__ __forceinline__ int a_lds_offset(int r, int c)
@@ -62,84 +65,62 @@ __device__ __forceinline__ void load_b(BRegs &b, const v4i *__restrict__ wp, int
     for (int kk = 0; kk < kKK; ++kk) {
 #pragma unroll
         for (int nf = 0; nf < kNF; ++nf) {
-            b.v[kk][nf] = __builtin_nontemporal_load(p + (kk * kNF + nf) * kWave);
+            b.v[kk][nf] = p[(kk * kNF + nf) * kWave];
         }
     }
 }
 
+// Activation loads of one step for a tile of MF 32-row fragments: MF 16-byte loads per thread.
+// Rows inside the last fragment but beyond the tile repeat its last row (their results are dropped in
+// the epilogue).
+template <int MF>
 struct ARegs {
-    v4i v[4];
+    v4i v[MF];
 };
 
-__device__ __forceinline__ void load_a(ARegs &r, const int8_t *__restrict__ a_tile, int Kd, int rows, int kt, int tid)
+template <int MF>
+__device__ __forceinline__ void load_a(ARegs<MF> &r, const int8_t *__restrict__ a_tile, int Kd, int rows, int kt,
+                                       int tid)
 {
     const int c = tid & 7;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        int row = (tid >> 3) + 32 * i;
-        row = min(row, rows - 1);  // rows beyond the tile repeat its last row; their results are dropped
+    for (int i = 0; i < MF; ++i) {
+        const int row = min((tid >> 3) + 32 * i, rows - 1);
         r.v[i] = *(const v4i *)(a_tile + (long long)row * Kd + kt * kBK + c * 16);
     }
 }
 
-__device__ __forceinline__ void store_a(const ARegs &r, int8_t *stage, int tid)
+template <int MF>
+__device__ __forceinline__ void store_a(const ARegs<MF> &r, int8_t *stage, int tid)
 {
     const int c = tid & 7;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
+    for (int i = 0; i < MF; ++i) {
         const int row = (tid >> 3) + 32 * i;
         *(v4i *)(stage + a_lds_offset(row, c)) = r.v[i];
     }
 }
 
-template <int EPI>
-__global__ __launch_bounds__(kThreads, 1) void gemm_kernel(GemmArgs a)
-{
-    __shared__ __attribute__((aligned(16))) int8_t a_s[2][kBM * kBK];
-    __shared__ float row_scale_s[kBM];
+struct TileCtx {
+    const int8_t *a_tile;   // first activation row of the tile
+    const v4i *wp;          // this wave's weight stream (+ lane)
+    const float *sg;        // this expert's per-channel scales
+    int m0, rows, nw, Kd, N;
+    bool wave_live;
+};
 
+// The whole tile for a compile-time number of row fragments, so that the main loop is branch-free.
+template <int EPI, int MF>
+__device__ __forceinline__ void gemm_tile(const GemmArgs &a, const TileCtx &t, int8_t (*a_s)[kBM * kBK],
+                                          const float *row_scale_s)
+{
     const int tid = threadIdx.x;
     const int lane = tid & (kWave - 1);
-    const int wave = tid >> 6;
+    const int KT = t.Kd / kBK;
 
-    // ---- which tile, which column block
-    const int num_tiles = min(a.tiles[0], a.max_tiles);
-    const int nblocks = (a.N + kBlockCols - 1) / kBlockCols;
-    const long long total_work = (long long)num_tiles * nblocks;
-    const long long chunk = (total_work + kNumXcd - 1) / kNumXcd;
-    const long long slot = blockIdx.x / kNumXcd;
-    const long long wid = (long long)(blockIdx.x % kNumXcd) * chunk + slot;
-    if (slot >= chunk || wid >= total_work) {
-        return;
-    }
-    const int tile = (int)(wid / nblocks);
-    const int nb = (int)(wid - (long long)tile * nblocks);
-    const int32_t *te = a.tiles + 4 + 4 * tile;
-    const int g = te[0];
-    const int m0 = te[1];
-    const int rows = te[2];
-    if (rows <= 0) {
-        return;
-    }
-    const int mfrags = (rows + 31) >> 5;
-
-    const int Kd = a.Kd;
-    const int N = a.N;
-    const int nw = nb * 4 + wave;             // this wave's 64-column group
-    const bool wave_live = nw * kWaveCols < N;
-    const int8_t *wg = a.per_expert ? a.list.w[g] : a.w + (long long)g * Kd * N;
-    const float *sg = a.per_expert ? a.list.s[g] : a.w_scale + (long long)g * N;
-    const v4i *wp = (const v4i *)(wg + (long long)(wave_live ? nw : 0) * Kd * kWaveCols) + lane;
-    const int8_t *a_tile = a.a + (long long)m0 * Kd;
-    const int KT = Kd / kBK;
-
-    if (EPI != kEpiInt32 && tid < kBM) {
-        row_scale_s[tid] = a.a_scale[m0 + min(tid, rows - 1)];
-    }
-
-    v16i acc[kMF][kNF];
+    v16i acc[MF][kNF];
 #pragma unroll
-    for (int mf = 0; mf < kMF; ++mf) {
+    for (int mf = 0; mf < MF; ++mf) {
 #pragma unroll
         for (int nf = 0; nf < kNF; ++nf) {
 #pragma unroll
@@ -149,66 +130,88 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_kernel(GemmArgs a)
         }
     }
 
-    BRegs b0, b1;
-    ARegs ar;
-    load_a(ar, a_tile, Kd, rows, 0, tid);
-    load_b(b0, wp, 0);
-    store_a(ar, a_s[0], tid);
+    // Software pipeline: weights for steps kt+1 and kt+2 are in flight (register ring of three steps)
+    // while step kt is multiplied; activations for step kt+1 travel global -> registers -> LDS.
+    // Every load in the loop is unconditional (step indices are clamped to the last step, which is
+    // then simply fetched again), so the loop body has no control flow and nothing forces a wait on
+    // a load before its data is needed.
+    BRegs bring[kBDepth];
+    ARegs<MF> ar;
+    const int last = KT - 1;
+    load_b(bring[0], t.wp, 0);
+    load_a<MF>(ar, t.a_tile, t.Kd, t.rows, 0, tid);
+    load_b(bring[1], t.wp, min(1, last));
+    store_a<MF>(ar, a_s[0], tid);
     __syncthreads();
 
     const int a_row = lane & 31;
     const int a_half = lane >> 5;
 
+    // A fragments are double-buffered in registers across the four MFMA sub-steps of a step.
+    auto load_frags = [&](v4i *af, const int8_t *stage, int kk) {
+#pragma unroll
+        for (int mf = 0; mf < MF; ++mf) {
+            af[mf] = *(const v4i *)(stage + a_lds_offset(mf * 32 + a_row, kk * 2 + a_half));
+        }
+    };
     auto compute = [&](const int8_t *stage, const BRegs &b) {
+        v4i af[2][MF];
+        load_frags(af[0], stage, 0);
 #pragma unroll
         for (int kk = 0; kk < kKK; ++kk) {
+            if (kk + 1 < kKK) {
+                load_frags(af[(kk + 1) & 1], stage, kk + 1);
+            }
+            // Keep the LDS reads of the next sub-step ahead of this sub-step's MFMAs: the scheduler
+            // would otherwise sink them to just before their first use and expose the LDS latency.
+            __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-            for (int mf = 0; mf < kMF; ++mf) {
-                if (mf < mfrags) {
-                    const v4i af = *(const v4i *)(stage + a_lds_offset(mf * 32 + a_row, kk * 2 + a_half));
+            for (int mf = 0; mf < MF; ++mf) {
 #pragma unroll
-                    for (int nf = 0; nf < kNF; ++nf) {
-                        acc[mf][nf] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af, b.v[kk][nf], acc[mf][nf], 0, 0, 0);
-                    }
+                for (int nf = 0; nf < kNF; ++nf) {
+                    acc[mf][nf] =
+                        __builtin_amdgcn_mfma_i32_32x32x32_i8(af[kk & 1][mf], b.v[kk][nf], acc[mf][nf], 0, 0, 0);
                 }
             }
+            __builtin_amdgcn_sched_barrier(0);
         }
     };
 
-    for (int kt = 0; kt < KT; kt += 2) {
-        // even step: compute stage 0 / b0 while fetching step kt+1 into stage 1 / b1
-        const bool more1 = kt + 1 < KT;
-        if (more1) {
-            load_a(ar, a_tile, Kd, rows, kt + 1, tid);
-            load_b(b1, wp, kt + 1);
-        }
-        compute(a_s[0], b0);
-        if (more1) {
-            store_a(ar, a_s[1], tid);
-        }
-        __syncthreads();
-        if (!more1) {
-            break;
-        }
-        // odd step
-        const bool more2 = kt + 2 < KT;
-        if (more2) {
-            load_a(ar, a_tile, Kd, rows, kt + 2, tid);
-            load_b(b0, wp, kt + 2);
-        }
-        compute(a_s[1], b1);
-        if (more2) {
-            store_a(ar, a_s[0], tid);
-        }
-        __syncthreads();
+    // One step with static ring indices: fetch step KT_+2 into ring[(CUR+2)%3], multiply ring[CUR].
+#define CAM_GEMM_STEP(CUR, KT_)                                               \
+    {                                                                         \
+        const int kt_ = (KT_);                                                \
+        load_b(bring[((CUR) + 2) % kBDepth], t.wp, min(kt_ + 2, last));       \
+        load_a<MF>(ar, t.a_tile, t.Kd, t.rows, min(kt_ + 1, last), tid);      \
+        compute(a_s[kt_ & 1], bring[(CUR)]);                                  \
+        store_a<MF>(ar, a_s[(kt_ + 1) & 1], tid);                             \
+        __syncthreads();                                                      \
     }
 
-    if (!wave_live) {
+    int kt = 0;
+    for (; kt + kBDepth <= KT; kt += kBDepth) {
+        CAM_GEMM_STEP(0, kt)
+        CAM_GEMM_STEP(1, kt + 1)
+        CAM_GEMM_STEP(2, kt + 2)
+    }
+    if (kt < KT) {
+        CAM_GEMM_STEP(0, kt)
+    }
+    if (kt + 1 < KT) {
+        CAM_GEMM_STEP(1, kt + 1)
+    }
+#undef CAM_GEMM_STEP
+
+    if (!t.wave_live) {
         return;
     }
 
     // ---- epilogue, accumulators in registers.
     // Lane l holds column (l & 31) of each 32x32 fragment; register i holds row 8*(i/4) + 4*(l/32) + i%4.
+    const int rows = t.rows;
+    const int m0 = t.m0;
+    const int N = t.N;
+    const int nw = t.nw;
     const int col_in = lane & 31;
     const int row_half = (lane >> 5) * 4;
     if (EPI == kEpiInt32) {
@@ -217,7 +220,7 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_kernel(GemmArgs a)
         for (int nf = 0; nf < kNF; ++nf) {
             const int col = a.gate_up ? (nf * (N / 2) + nw * 32 + col_in) : (nw * kWaveCols + nf * 32 + col_in);
 #pragma unroll
-            for (int mf = 0; mf < kMF; ++mf) {
+            for (int mf = 0; mf < MF; ++mf) {
 #pragma unroll
                 for (int i = 0; i < 16; ++i) {
                     const int row = mf * 32 + 8 * (i >> 2) + row_half + (i & 3);
@@ -232,10 +235,10 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_kernel(GemmArgs a)
         float *out = (float *)a.out;
         const int I = N / 2;
         const int c = nw * 32 + col_in;
-        const float sg_gate = sg[c];
-        const float sg_up = sg[I + c];
+        const float sg_gate = t.sg[c];
+        const float sg_up = t.sg[I + c];
 #pragma unroll
-        for (int mf = 0; mf < kMF; ++mf) {
+        for (int mf = 0; mf < MF; ++mf) {
 #pragma unroll
             for (int i = 0; i < 16; ++i) {
                 const int row = mf * 32 + 8 * (i >> 2) + row_half + (i & 3);
@@ -252,9 +255,9 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_kernel(GemmArgs a)
 #pragma unroll
         for (int nf = 0; nf < kNF; ++nf) {
             const int col = nw * kWaveCols + nf * 32 + col_in;
-            const float ws = sg[col];
+            const float ws = t.sg[col];
 #pragma unroll
-            for (int mf = 0; mf < kMF; ++mf) {
+            for (int mf = 0; mf < MF; ++mf) {
 #pragma unroll
                 for (int i = 0; i < 16; ++i) {
                     const int row = mf * 32 + 8 * (i >> 2) + row_half + (i & 3);
@@ -265,6 +268,65 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_kernel(GemmArgs a)
                 }
             }
         }
+    }
+}
+
+template <int EPI>
+__global__ __launch_bounds__(kThreads, 1) void gemm_kernel(GemmArgs a)
+{
+    __shared__ __attribute__((aligned(16))) int8_t a_s[2][kBM * kBK];
+    __shared__ float row_scale_s[kBM];
+
+    const int tid = threadIdx.x;
+    const int lane = tid & (kWave - 1);
+    const int wave = tid >> 6;
+
+    // ---- which tile, which column block.  Work ids run (tile, column block) with the column block
+    // fastest; each XCD takes one contiguous run of ids, so the workgroups that share a tile's
+    // activation rows, and neighbouring tiles of one expert that share weight panels, meet in one L2.
+    const int num_tiles = min(a.tiles[0], a.max_tiles);
+    const int nblocks = (a.N + kBlockCols - 1) / kBlockCols;
+    const long long total_work = (long long)num_tiles * nblocks;
+    const long long chunk = (total_work + kNumXcd - 1) / kNumXcd;
+    const long long slot = blockIdx.x / kNumXcd;
+    const long long wid = (long long)(blockIdx.x % kNumXcd) * chunk + slot;
+    if (slot >= chunk || wid >= total_work) {
+        return;
+    }
+    const int tile = (int)(wid / nblocks);
+    const int nb = (int)(wid - (long long)tile * nblocks);
+    const int32_t *te = a.tiles + 4 + 4 * tile;
+    const int g = te[0];
+    TileCtx t;
+    t.m0 = te[1];
+    t.rows = te[2];
+    if (t.rows <= 0) {
+        return;
+    }
+    t.Kd = a.Kd;
+    t.N = a.N;
+    t.nw = nb * 4 + wave;  // this wave's 64-column group
+    t.wave_live = t.nw * kWaveCols < t.N;
+    const int8_t *wg = a.per_expert ? a.list.w[g] : a.w + (long long)g * t.Kd * t.N;
+    t.sg = a.per_expert ? a.list.s[g] : a.w_scale + (long long)g * t.N;
+    t.wp = (const v4i *)(wg + (long long)(t.wave_live ? t.nw : 0) * t.Kd * kWaveCols) + lane;
+    t.a_tile = a.a + (long long)t.m0 * t.Kd;
+
+    if (EPI != kEpiInt32) {
+        for (int r = tid; r < kBM; r += kThreads) {
+            row_scale_s[r] = a.a_scale[t.m0 + min(r, t.rows - 1)];
+        }
+    }
+
+    const int mfrags = (t.rows + 31) >> 5;
+    if (mfrags <= 1) {
+        gemm_tile<EPI, 1>(a, t, a_s, row_scale_s);
+    } else if (mfrags <= 2) {
+        gemm_tile<EPI, 2>(a, t, a_s, row_scale_s);
+    } else if (mfrags <= 4) {
+        gemm_tile<EPI, 4>(a, t, a_s, row_scale_s);
+    } else {
+        gemm_tile<EPI, 8>(a, t, a_s, row_scale_s);
     }
 }
 

@@ -8,12 +8,13 @@
 //   recv cumsum   src/cam/comm_operator/pybind/moe_dispatch_prefill.cpp:126-145
 //
 // Design.  The rank of an entry is its position among earlier flat (t,k) entries with the same
-// expert id, i.e. a stable counting sort; atomics would make the order depend on scheduling.  All
-// integer work of one call is a few hundred KB, so one 1024-thread workgroup does it in a single
-// launch: each of the 16 waves owns a contiguous slice of the flat id sequence and ranks 64 ids at a
-// time with wave ballots (lanes holding the same id find each other bit by bit), keeping a private
-// running histogram in LDS; a scan across the 16 histograms then turns wave-local ranks into global
-// ones.  No inter-workgroup synchronisation, no atomics, fully deterministic.
+// expert id, i.e. a stable counting sort; atomics would make the order depend on scheduling.  Two
+// short launches, no atomics on results, no spinning, fully deterministic:
+//   1. every workgroup ranks its own contiguous chunk of the flat id sequence (wave ballots + per-wave
+//      LDS histograms) and publishes the chunk's per-expert histogram;
+//   2. every workgroup sums the histograms of the chunks before it (its base), scans the per-expert
+//      totals into offsets, and finishes its chunk.  The reference does this part on the CPU after a
+//      device-to-host copy.
 #include "cam_device.h"
 #include "cam_kernels.h"
 
@@ -21,19 +22,21 @@ namespace cam {
 
 namespace {
 
-constexpr int kPlanThreads = 1024;
-constexpr int kPlanWaves = kPlanThreads / kWave;
-constexpr int kUnroll = 4;
+constexpr int kScanThreads = 1024;  // single-workgroup scan kernels (notify, tile table)
+constexpr int kLocalThreads = 256;  // phase 1: 4 waves per workgroup
+constexpr int kLocalWaves = kLocalThreads / kWave;
+constexpr int kGlobalThreads = 512; // phase 2: one thread per expert column
 
 template <typename IdT>
-__device__ __forceinline__ int load_id(const IdT *p, int i, int E)
+__device__ __forceinline__ int load_id(const IdT *p, long long i, int E)
 {
     long long v = (long long)p[i];
     return (v < 0 || v >= (long long)E) ? -1 : (int)v;
 }
 
-// Exclusive scan of one value per thread for tid < 512 (others pass 0); returns the exclusive prefix
-// and leaves the grand total in *total_out (LDS).  Uses `scratch` (>= 16 ints of LDS).
+// Exclusive scan of one value per thread across a workgroup of NWAVES waves; returns the exclusive
+// prefix and leaves the grand total in *total_out (LDS).  Uses `scratch` (>= NWAVES ints of LDS).
+template <int NWAVES>
 __device__ __forceinline__ int block_exclusive_scan(int v, int tid, int *scratch, int *total_out)
 {
     int lane = tid & (kWave - 1);
@@ -44,12 +47,12 @@ __device__ __forceinline__ int block_exclusive_scan(int v, int tid, int *scratch
     }
     __syncthreads();
     if (w == 0) {
-        int t = lane < kPlanWaves ? scratch[lane] : 0;
+        int t = lane < NWAVES ? scratch[lane] : 0;
         int ti = wave_inclusive_scan(t, lane);
-        if (lane < kPlanWaves) {
+        if (lane < NWAVES) {
             scratch[lane] = ti - t;
         }
-        if (lane == kPlanWaves - 1) {
+        if (lane == NWAVES - 1) {
             *total_out = ti;
         }
     }
@@ -59,51 +62,53 @@ __device__ __forceinline__ int block_exclusive_scan(int v, int tid, int *scratch
     return r;
 }
 
-template <typename IdT>
-__global__ __launch_bounds__(kPlanThreads) void plan_kernel(PlanArgs a)
+__device__ __forceinline__ int count_active(const uint8_t *mask, int T, int tid, int nthreads, int *slot)
 {
-    __shared__ int hist[kPlanWaves * kMaxExperts];  // 32 KB: running per-wave histograms
-    __shared__ int off_s[kMaxExperts];
-    __shared__ int scan_s[kPlanWaves];
-    __shared__ int total_s;
-    __shared__ int active_s;
+    if (mask == nullptr) {
+        return T;
+    }
+    int c = 0;
+    for (int t = tid; t < T; t += nthreads) {
+        c += mask[t] != 0 ? 1 : 0;
+    }
+    c = wave_sum(c);
+    if (tid == 0) {
+        *slot = 0;
+    }
+    __syncthreads();
+    if ((tid & (kWave - 1)) == 0 && c != 0) {
+        atomicAdd(slot, c);
+    }
+    __syncthreads();
+    return *slot;
+}
 
+// Phase 1.  Workgroup b owns the flat entries [b*chunk, (b+1)*chunk), chunk = IT*256; wave w of it the
+// IT*64 entries from b*chunk + w*IT*64.  Each lane keeps its IT ids in registers.  64 ids at a time,
+// lanes holding the same id find each other with one ballot per id bit; the rank inside the wave is the
+// wave's running count of that id (LDS) plus the number of lower lanes in the group, and the group's
+// highest lane publishes the new count.  A scan over the 4 waves' histograms turns wave-local ranks
+// into workgroup-local ones; the workgroup's histogram goes to hist_out[b][*].
+template <typename IdT, int IT>
+__global__ __launch_bounds__(kLocalThreads) void plan_local_kernel(PlanArgs a, int32_t *hist_out)
+{
+    __shared__ int hist[kLocalWaves * kMaxExperts];
+    __shared__ int active_s;
     const int tid = threadIdx.x;
     const int lane = tid & (kWave - 1);
     const int w = tid >> 6;
+    const int b = blockIdx.x;
     const int E = a.E;
     const IdT *__restrict__ idx = (const IdT *)a.idx;
-    int32_t *__restrict__ pos = a.pos;
 
-    for (int i = tid; i < kPlanWaves * kMaxExperts; i += kPlanThreads) {
+    for (int i = tid; i < kLocalWaves * kMaxExperts; i += kLocalThreads) {
         hist[i] = 0;
     }
-    // Active prefix length: number of set mask entries (all tokens when there is no mask).
-    int t_active = a.T;
-    if (a.mask != nullptr) {
-        int c = 0;
-        for (int t = tid; t < a.T; t += kPlanThreads) {
-            c += a.mask[t] != 0 ? 1 : 0;
-        }
-        c = wave_sum(c);
-        if (tid == 0) {
-            active_s = 0;
-        }
-        __syncthreads();
-        if (lane == 0) {
-            atomicAdd(&active_s, c);
-        }
-        __syncthreads();
-        t_active = active_s;
-    }
+    const int t_active = count_active(a.mask, a.T, tid, kLocalThreads, &active_s);
     __syncthreads();
-
-    const int n = t_active * a.K;
-    const int n_all = a.T * a.K;
-    int per_wave = (n + kPlanWaves - 1) / kPlanWaves;
-    per_wave = (per_wave + kWave - 1) & ~(kWave - 1);
-    const int beg = min(n, w * per_wave);
-    const int end = min(n, beg + per_wave);
+    const long long n = (long long)t_active * a.K;
+    const long long n_all = (long long)a.T * a.K;
+    const long long base = (long long)b * (IT * kLocalThreads) + (long long)w * (IT * kWave);
     int nbits = 0;
     while ((1 << nbits) < E) {
         ++nbits;
@@ -111,82 +116,123 @@ __global__ __launch_bounds__(kPlanThreads) void plan_kernel(PlanArgs a)
     int *my_hist = hist + w * kMaxExperts;
     const unsigned long long lt_mask = (1ull << lane) - 1ull;
 
-    // Pass 1: wave-local stable ranks.
-    for (int base = beg; base < end; base += kWave * kUnroll) {
-        int e[kUnroll];
+    int e[IT], r[IT];
 #pragma unroll
-        for (int u = 0; u < kUnroll; ++u) {
-            int i = base + u * kWave + lane;
-            e[u] = i < end ? load_id(idx, i, E) : -1;
-        }
+    for (int it = 0; it < IT; ++it) {
+        const long long i = base + it * kWave + lane;
+        e[it] = i < n ? load_id(idx, i, E) : -1;
+    }
 #pragma unroll
-        for (int u = 0; u < kUnroll; ++u) {
-            int i = base + u * kWave + lane;
-            bool act = e[u] >= 0;
-            unsigned long long peers = __ballot(act);
-            for (int b = 0; b < nbits; ++b) {
-                bool bit = act && ((e[u] >> b) & 1);
-                unsigned long long bal = __ballot(bit);
-                peers &= bit ? bal : ~bal;
-            }
-            int r = -1;
-            int prior = 0;
-            if (act) {
-                prior = my_hist[e[u]];
-                r = prior + __popcll(peers & lt_mask);
-            }
-            __builtin_amdgcn_wave_barrier();
-            if (act && (peers >> lane) == 1ull) {  // highest lane of the group publishes the new count
-                my_hist[e[u]] = prior + __popcll(peers);
-            }
-            __builtin_amdgcn_wave_barrier();
-            if (i < end) {
-                pos[i] = r;
-            }
+    for (int it = 0; it < IT; ++it) {
+        const bool act = e[it] >= 0;
+        unsigned long long peers = __ballot(act);
+        for (int bit_i = 0; bit_i < nbits; ++bit_i) {
+            const bool bit = act && ((e[it] >> bit_i) & 1);
+            const unsigned long long bal = __ballot(bit);
+            peers &= bit ? bal : ~bal;
         }
+        int prior = 0;
+        r[it] = -1;
+        if (act) {
+            prior = my_hist[e[it]];
+            r[it] = prior + __popcll(peers & lt_mask);
+        }
+        __builtin_amdgcn_wave_barrier();
+        if (act && (peers >> lane) == 1ull) {
+            my_hist[e[it]] = prior + __popcll(peers);
+        }
+        __builtin_amdgcn_wave_barrier();
     }
     __syncthreads();
-
-    // Per expert: exclusive scan across the waves' histograms, total count.
-    int cnt = 0;
-    if (tid < E) {
+    for (int ee = tid; ee < E; ee += kLocalThreads) {
         int run = 0;
 #pragma unroll
-        for (int ww = 0; ww < kPlanWaves; ++ww) {
-            int t = hist[ww * kMaxExperts + tid];
-            hist[ww * kMaxExperts + tid] = run;
+        for (int ww = 0; ww < kLocalWaves; ++ww) {
+            const int t = hist[ww * kMaxExperts + ee];
+            hist[ww * kMaxExperts + ee] = run;
             run += t;
         }
-        cnt = run;
+        hist_out[(long long)b * E + ee] = run;
     }
-    int off = block_exclusive_scan(tid < E ? cnt : 0, tid, scan_s, &total_s);
-    if (tid < E) {
-        off_s[tid] = off;
+    if (b == 0 && tid == 0) {
+        hist_out[(long long)gridDim.x * E] = t_active;
     }
     __syncthreads();
-    const int total = total_s;
+#pragma unroll
+    for (int it = 0; it < IT; ++it) {
+        const long long i = base + it * kWave + lane;
+        if (i < n_all) {
+            a.pos[i] = e[it] >= 0 ? r[it] + my_hist[e[it]] : -1;
+        }
+    }
+}
 
-    // Pass 2: global ranks and destination rows.
-    for (int i = beg + lane; i < end; i += kWave) {
-        int e = load_id(idx, i, E);
-        int r = pos[i];
+// Phase 2.  Every workgroup sums the histogram columns (all rows for the per-expert count, the rows
+// before its own for its base), scans the counts into offsets, and finishes its own chunk:
+// pos += base[e], dst_row = off[e] + pos.  Workgroup 0 also writes the per-expert outputs and the
+// GEMM tile table.
+template <typename IdT>
+__global__ __launch_bounds__(kGlobalThreads) void plan_global_kernel(PlanArgs a, int chunk, const int32_t *hist_in)
+{
+    constexpr int NW = kGlobalThreads / kWave;
+    __shared__ int base_s[kMaxExperts];
+    __shared__ int off_s[kMaxExperts];
+    __shared__ int scan_s[NW];
+    __shared__ int total_s;
+    const int tid = threadIdx.x;
+    const int b = blockIdx.x;
+    const int nb = gridDim.x;
+    const int E = a.E;
+    const IdT *__restrict__ idx = (const IdT *)a.idx;
+
+    int cnt = 0, base = 0;
+    if (tid < E) {
+        const int32_t *col = hist_in + tid;
+        int bb = 0;
+        for (; bb + 8 <= nb; bb += 8) {
+            int v[8];
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                v[j] = col[(long long)(bb + j) * E];
+            }
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                cnt += v[j];
+                base += (bb + j) < b ? v[j] : 0;
+            }
+        }
+        for (; bb < nb; ++bb) {
+            const int v = col[(long long)bb * E];
+            cnt += v;
+            base += bb < b ? v : 0;
+        }
+    }
+    const int off = block_exclusive_scan<NW>(cnt, tid, scan_s, &total_s);
+    const int total = total_s;
+    base_s[tid] = base;
+    off_s[tid] = off;
+    __syncthreads();
+
+    const int t_active = hist_in[(long long)nb * E];
+    const long long n = (long long)t_active * a.K;
+    const long long n_all = (long long)a.T * a.K;
+    const long long lo = (long long)b * chunk;
+    const long long hi = min(n_all, lo + chunk);
+    for (long long i = lo + tid; i < hi; i += kGlobalThreads) {
+        const int e = i < n ? load_id(idx, i, E) : -1;
         int row = -1;
         if (e >= 0) {
-            r += my_hist[e];
-            row = off_s[e] + r;
-            pos[i] = r;
+            const int p = a.pos[i] + base_s[e];
+            a.pos[i] = p;
+            row = off_s[e] + p;
         }
         if (a.dst_row != nullptr) {
             a.dst_row[i] = row;
         }
     }
-    for (int i = n + tid; i < n_all; i += kPlanThreads) {  // masked-out tokens
-        pos[i] = -1;
-        if (a.dst_row != nullptr) {
-            a.dst_row[i] = -1;
-        }
+    if (b != 0) {
+        return;
     }
-
     if (tid < E) {
         if (a.cnt) a.cnt[tid] = cnt;
         if (a.off) a.off[tid] = off;
@@ -198,14 +244,15 @@ __global__ __launch_bounds__(kPlanThreads) void plan_kernel(PlanArgs a)
     if (tid == 0 && a.total) {
         a.total[0] = total;
     }
-    if (a.per_rank_zero != nullptr && tid < a.R) {
-        a.per_rank_zero[tid] = 0;
+    if (a.per_rank_zero != nullptr) {
+        for (int r = tid; r < a.R; r += kGlobalThreads) {
+            a.per_rank_zero[r] = 0;
+        }
     }
-
     // GEMM tile table: expert e owns ceil(cnt/kGemmTileM) tiles, in expert order.
     if (a.tiles != nullptr) {
-        int nt = tid < E ? (cnt + kGemmTileM - 1) / kGemmTileM : 0;
-        int tbase = block_exclusive_scan(nt, tid, scan_s, &total_s);
+        const int nt = tid < E ? (cnt + kGemmTileM - 1) / kGemmTileM : 0;
+        const int tbase = block_exclusive_scan<NW>(nt, tid, scan_s, &total_s);
         if (tid < E) {
             for (int j = 0; j < nt; ++j) {
                 int32_t *t = a.tiles + 4 + 4 * (tbase + j);
@@ -267,15 +314,15 @@ __global__ __launch_bounds__(256) void in_rank_kernel(InRankArgs a)
     }
 }
 
-__global__ __launch_bounds__(kPlanThreads) void notify_scan_kernel(const int32_t *cnt, int E, int num_tokens,
+__global__ __launch_bounds__(kScanThreads) void notify_scan_kernel(const int32_t *cnt, int E, int num_tokens,
                                                                   int32_t *off, int32_t *send_data,
                                                                   int32_t *recv_data)
 {
-    __shared__ int scan_s[kPlanWaves];
+    __shared__ int scan_s[kScanThreads / kWave];
     __shared__ int total_s;
     const int tid = threadIdx.x;
     int c = tid < E ? cnt[tid] : 0;
-    int o = block_exclusive_scan(c, tid, scan_s, &total_s);
+    int o = block_exclusive_scan<kScanThreads / kWave>(c, tid, scan_s, &total_s);
     if (tid < E) {
         if (off) off[tid] = o;
         if (send_data) {
@@ -291,11 +338,11 @@ __global__ __launch_bounds__(kPlanThreads) void notify_scan_kernel(const int32_t
     }
 }
 
-__global__ __launch_bounds__(kPlanThreads) void build_tiles_kernel(const int64_t *group_list, int cumulative,
+__global__ __launch_bounds__(kScanThreads) void build_tiles_kernel(const int64_t *group_list, int cumulative,
                                                                   int G, long long max_rows, int max_tiles,
                                                                   int32_t *tiles)
 {
-    __shared__ int scan_s[kPlanWaves];
+    __shared__ int scan_s[kScanThreads / kWave];
     __shared__ int total_s;
     const int tid = threadIdx.x;
     long long m0 = 0, m1 = 0;
@@ -309,7 +356,7 @@ __global__ __launch_bounds__(kPlanThreads) void build_tiles_kernel(const int64_t
     }
     if (!cumulative) {
         int c = tid < G ? (int)min(max(m1, 0ll), max_rows) : 0;
-        int o = block_exclusive_scan(c, tid, scan_s, &total_s);
+        int o = block_exclusive_scan<kScanThreads / kWave>(c, tid, scan_s, &total_s);
         m0 = o;
         m1 = (long long)o + c;
     }
@@ -318,7 +365,7 @@ __global__ __launch_bounds__(kPlanThreads) void build_tiles_kernel(const int64_t
     m1 = min(max(m1, m0), max_rows);
     int cnt = tid < G ? (int)(m1 - m0) : 0;
     int nt = (cnt + kGemmTileM - 1) / kGemmTileM;
-    int tbase = block_exclusive_scan(nt, tid, scan_s, &total_s);
+    int tbase = block_exclusive_scan<kScanThreads / kWave>(nt, tid, scan_s, &total_s);
     int num_tiles = min(total_s, max_tiles);
     if (tid < G) {
         for (int j = 0; j < nt && tbase + j < max_tiles; ++j) {  // a corrupt list cannot overrun the table
@@ -330,7 +377,7 @@ __global__ __launch_bounds__(kPlanThreads) void build_tiles_kernel(const int64_t
         }
     }
     __syncthreads();
-    int rows_total = block_exclusive_scan(cnt, tid, scan_s, &total_s);
+    int rows_total = block_exclusive_scan<kScanThreads / kWave>(cnt, tid, scan_s, &total_s);
     (void)rows_total;
     if (tid == 0) {
         tiles[0] = num_tiles;
@@ -349,16 +396,56 @@ __global__ void cast_i64_to_i32_kernel(const int64_t *src, int32_t *dst, long lo
     }
 }
 
+void plan_geometry(long long n_all, int *it_out, int *nb_out)
+{
+    int it = 1;
+    while (it < 8 && (n_all + (long long)it * kLocalThreads - 1) / ((long long)it * kLocalThreads) > 64) {
+        it *= 2;
+    }
+    long long nb = (n_all + (long long)it * kLocalThreads - 1) / ((long long)it * kLocalThreads);
+    *it_out = it;
+    *nb_out = (int)(nb < 1 ? 1 : nb);
+}
+
+template <typename IdT>
+hipError_t launch_plan_t(const PlanArgs &a, int it, int nb, int32_t *hist, hipStream_t stream)
+{
+    dim3 grid(nb), blk(kLocalThreads);
+    switch (it) {
+        case 1: hipLaunchKernelGGL((plan_local_kernel<IdT, 1>), grid, blk, 0, stream, a, hist); break;
+        case 2: hipLaunchKernelGGL((plan_local_kernel<IdT, 2>), grid, blk, 0, stream, a, hist); break;
+        case 4: hipLaunchKernelGGL((plan_local_kernel<IdT, 4>), grid, blk, 0, stream, a, hist); break;
+        default: hipLaunchKernelGGL((plan_local_kernel<IdT, 8>), grid, blk, 0, stream, a, hist); break;
+    }
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) {
+        return e;
+    }
+    hipLaunchKernelGGL(plan_global_kernel<IdT>, grid, dim3(kGlobalThreads), 0, stream, a, it * kLocalThreads,
+                       (const int32_t *)hist);
+    return hipGetLastError();
+}
+
 }  // namespace
+
+uint64_t plan_workspace_bytes(int64_t T, int64_t K, int E)
+{
+    int it, nb;
+    plan_geometry(T * K, &it, &nb);
+    return ((uint64_t)nb * (uint64_t)E + 4) * sizeof(int32_t);
+}
 
 hipError_t launch_plan(const PlanArgs &a, hipStream_t stream)
 {
-    if (a.idx_is64) {
-        hipLaunchKernelGGL(plan_kernel<int64_t>, dim3(1), dim3(kPlanThreads), 0, stream, a);
-    } else {
-        hipLaunchKernelGGL(plan_kernel<int32_t>, dim3(1), dim3(kPlanThreads), 0, stream, a);
+    if (a.hist_ws == nullptr) {
+        return hipErrorInvalidValue;
     }
-    return hipGetLastError();
+    int it, nb;
+    plan_geometry((long long)a.T * a.K, &it, &nb);
+    if (a.idx_is64) {
+        return launch_plan_t<int64_t>(a, it, nb, a.hist_ws, stream);
+    }
+    return launch_plan_t<int32_t>(a, it, nb, a.hist_ws, stream);
 }
 
 hipError_t launch_in_rank(const InRankArgs &a, hipStream_t stream)
@@ -386,7 +473,7 @@ hipError_t launch_in_rank(const InRankArgs &a, hipStream_t stream)
 hipError_t launch_notify_scan(const int32_t *cnt, int E, int num_tokens, int32_t *off, int32_t *send_data,
                               int32_t *recv_data, hipStream_t stream)
 {
-    hipLaunchKernelGGL(notify_scan_kernel, dim3(1), dim3(kPlanThreads), 0, stream, cnt, E, num_tokens, off,
+    hipLaunchKernelGGL(notify_scan_kernel, dim3(1), dim3(kScanThreads), 0, stream, cnt, E, num_tokens, off,
                        send_data, recv_data);
     return hipGetLastError();
 }
@@ -394,7 +481,7 @@ hipError_t launch_notify_scan(const int32_t *cnt, int E, int num_tokens, int32_t
 hipError_t launch_build_tiles(const int64_t *group_list, int cumulative, int G, int64_t max_rows, int max_tiles,
                               int32_t *tiles, hipStream_t stream)
 {
-    hipLaunchKernelGGL(build_tiles_kernel, dim3(1), dim3(kPlanThreads), 0, stream, group_list, cumulative, G,
+    hipLaunchKernelGGL(build_tiles_kernel, dim3(1), dim3(kScanThreads), 0, stream, group_list, cumulative, G,
                        (long long)max_rows, max_tiles, tiles);
     return hipGetLastError();
 }
