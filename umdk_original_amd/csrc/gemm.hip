@@ -10,15 +10,18 @@
 //
 // Design (not a translation of the cube/vector split above).
 //   * One workgroup = 4 waves = a tile of up to 256 rows of ONE expert x 256 packed weight columns.
-//     Every wave covers all rows of the tile and its own 64 columns, so a weight byte is needed by
-//     exactly one wave: weights go straight from HBM to registers in the lane order the MFMA wants
-//     (they were laid out that way once by the prepack kernel), 16 bytes per lane, 1 KB contiguous
-//     per wave and load, through a register ring two 128-deep K steps ahead.  No LDS for weights.
-//     The grouped shape is bound by streaming the weights, so the tile is as tall as the register
-//     file allows (256 int32 accumulators per lane): every weight byte fetched feeds up to 256 rows.
-//   * Activations (shared by the 4 waves) are staged through LDS, double-buffered, with an XOR
-//     swizzle of the 16-byte chunks so that both the cooperative stores and the ds_read_b128
-//     fragment loads are bank-conflict free.
+//     Every wave covers all rows of the tile and its own 64 columns (256 int32 accumulators per lane,
+//     the most the register file allows): the grouped shape is bound by streaming the weights, and a
+//     tile this tall makes every weight byte fetched feed up to 256 rows.
+//   * Both operands travel global -> LDS with direct-to-LDS loads (16 bytes per lane, no registers),
+//     four stages deep, three 64-deep K steps ahead of the MFMAs.  Weights were laid out once by the
+//     prepack kernel in the lane order the MFMA wants, so a wave's weight load is 1 KB of contiguous
+//     memory that lands in LDS already in fragment order.  Activation rows are placed with an XOR
+//     swizzle of their 16-byte chunks (chosen on the global side, since a direct-to-LDS load writes
+//     lane i at base + 16*i), which makes the ds_read_b128 fragment reads bank-conflict free.
+//   * The loads are issued from inline assembly and the pipeline's waits are written out by hand.
+//     Left to itself the compiler drains every outstanding load at each workgroup barrier and before
+//     LDS reads it cannot prove independent, which serialises the pipeline.
 //   * The int32 accumulators stay in registers through the epilogue: dequantisation, SiLU and the
 //     gate*up product are applied in place; the int32 tile never goes to memory.
 //     For GMM1 the prepack pairs gate column c with up column I+c inside one wave.
@@ -37,86 +40,69 @@ namespace cam {
 namespace {
 
 constexpr int kBM = kGemmTileM;  // rows per tile
-constexpr int kMF = kBM / 32;    // row fragments per tile
 constexpr int kNF = 2;           // 2 column fragments per wave (64 columns)
-constexpr int kBK = 128;         // K bytes per main-loop step
-constexpr int kKK = kBK / 32;    // MFMA steps per main-loop step
+constexpr int kBK = 64;          // K bytes per pipeline step
+constexpr int kKK = kBK / 32;    // MFMA sub-steps per step
 constexpr int kThreads = 256;
 constexpr int kWaveCols = 64;
 constexpr int kBlockCols = 4 * kWaveCols;
 constexpr int kNumXcd = 8;
-constexpr int kBDepth = 3;       // weight register ring: steps in flight
+constexpr int kStages = 4;
+constexpr int kStageA = kBM * kBK;                    // 16 KB of activations per stage
+constexpr int kStageB = 4 * kWaveCols * kBK;          // 16 KB of weights per stage (4 KB per wave)
+constexpr int kStageBytes = kStageA + kStageB;
+constexpr int kBLoads = kKK * kNF;                    // weight loads per wave and step
+constexpr int kEpiRowBytes = 144;                     // epilogue staging: 128 data bytes + 16 of padding per row
+constexpr int kLdsBytes = kStages * kStageBytes > 4 * kBM * kEpiRowBytes ? kStages * kStageBytes
+                                                                         : 4 * kBM * kEpiRowBytes;
 
-// LDS offset (bytes) of the 16-byte chunk `c` (0..7) of row `r` in one A stage.
+// LDS offset (bytes) inside a stage of the 16-byte chunk `c` (0..3) of activation row `r`.
 __device__ __forceinline__ int a_lds_offset(int r, int c)
 {
-    return r * kBK + ((c ^ ((r >> 1) & 7)) << 4);
+    return r * kBK + ((c ^ ((r >> 2) & 3)) << 4);
 }
 
-struct BRegs {
-    v4i v[kKK][kNF];
-};
-
-__device__ __forceinline__ void load_b(BRegs &b, const v4i *__restrict__ wp, int kt)
+// One direct-to-LDS load: lane i of the wave fetches 16 bytes at its own global address `g` and the
+// data lands at LDS byte address lds_base + 16*i.
+__device__ __forceinline__ void dma16(const void *g, unsigned lds_base)
 {
-    // wave-contiguous: [(kt*4 + kk)*2 + nf][lane] 16-byte pieces
-    const v4i *p = wp + (long long)kt * (kKK * kNF * kWave);
-#pragma unroll
-    for (int kk = 0; kk < kKK; ++kk) {
-#pragma unroll
-        for (int nf = 0; nf < kNF; ++nf) {
-            b.v[kk][nf] = p[(kk * kNF + nf) * kWave];
-        }
-    }
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(lds_base), "v"(g) : "memory");
 }
 
-// Activation loads of one step for a tile of MF 32-row fragments: MF 16-byte loads per thread.
-// Rows inside the last fragment but beyond the tile repeat its last row (their results are dropped in
-// the epilogue).
-template <int MF>
-struct ARegs {
-    v4i v[MF];
-};
-
-template <int MF>
-__device__ __forceinline__ void load_a(ARegs<MF> &r, const int8_t *__restrict__ a_tile, int Kd, int rows, int kt,
-                                       int tid)
+template <int N>
+__device__ __forceinline__ void wait_loads_outstanding()
 {
-    const int c = tid & 7;
-#pragma unroll
-    for (int i = 0; i < MF; ++i) {
-        const int row = min((tid >> 3) + 32 * i, rows - 1);
-        r.v[i] = *(const v4i *)(a_tile + (long long)row * Kd + kt * kBK + c * 16);
-    }
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
 }
 
-template <int MF>
-__device__ __forceinline__ void store_a(const ARegs<MF> &r, int8_t *stage, int tid)
+// Workgroup barrier without the memory fence of __syncthreads(); the waits are explicit (above).
+__device__ __forceinline__ void barrier_no_fence()
 {
-    const int c = tid & 7;
-#pragma unroll
-    for (int i = 0; i < MF; ++i) {
-        const int row = (tid >> 3) + 32 * i;
-        *(v4i *)(stage + a_lds_offset(row, c)) = r.v[i];
-    }
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
 }
 
 struct TileCtx {
     const int8_t *a_tile;   // first activation row of the tile
-    const v4i *wp;          // this wave's weight stream (+ lane)
+    const int8_t *wp;       // this wave's weight stream (+ 16 * lane)
     const float *sg;        // this expert's per-channel scales
     int m0, rows, nw, Kd, N;
     bool wave_live;
 };
 
-// The whole tile for a compile-time number of row fragments, so that the main loop is branch-free.
+// The whole tile for a compile-time number of 32-row fragments, so that the main loop is branch-free.
 template <int EPI, int MF>
-__device__ __forceinline__ void gemm_tile(const GemmArgs &a, const TileCtx &t, int8_t (*a_s)[kBM * kBK],
-                                          const float *row_scale_s)
+__device__ __forceinline__ void gemm_tile(const GemmArgs &a, const TileCtx &t, int8_t *lds, const float *row_scale_s)
 {
+    constexpr int AI = MF >= 2 ? MF / 2 : 1;   // activation loads per wave and step (1 KB each)
+    constexpr int PER_STEP = AI + kBLoads;     // loads per wave and step
     const int tid = threadIdx.x;
     const int lane = tid & (kWave - 1);
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int KT = t.Kd / kBK;
+    const int last = KT - 1;
+    const unsigned lds0 = (unsigned)(unsigned long long)(__attribute__((address_space(3))) int8_t *)lds;
 
     v16i acc[MF][kNF];
 #pragma unroll
@@ -130,109 +116,147 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs &a, const TileCtx &t, i
         }
     }
 
-    // Software pipeline: weights for steps kt+1 and kt+2 are in flight (register ring of three steps)
-    // while step kt is multiplied; activations for step kt+1 travel global -> registers -> LDS.
-    // Every load in the loop is unconditional (step indices are clamped to the last step, which is
-    // then simply fetched again), so the loop body has no control flow and nothing forces a wait on
-    // a load before its data is needed.
-    BRegs bring[kBDepth];
-    ARegs<MF> ar;
-    const int last = KT - 1;
-    load_b(bring[0], t.wp, 0);
-    load_a<MF>(ar, t.a_tile, t.Kd, t.rows, 0, tid);
-    load_b(bring[1], t.wp, min(1, last));
-    store_a<MF>(ar, a_s[0], tid);
-    __syncthreads();
+    // Per-lane source addresses of the activation loads (they advance by kBK per step).
+    // Load j of wave w fills the 64-byte LDS rows 16q .. 16q+15 with q = 4j + w (q = w & 1 for a
+    // single-fragment tile, where waves 2 and 3 repeat the loads of waves 0 and 1); lane i brings row
+    // 16q + i/4, and the chunk whose swizzled slot is i%4.  Rows inside the last fragment but beyond
+    // the tile repeat its last row (their results are dropped in the epilogue).
+    const int8_t *a_src[AI];
+    unsigned a_dst[AI];
+#pragma unroll
+    for (int j = 0; j < AI; ++j) {
+        const int q = MF >= 2 ? j * 4 + wave : (wave & 1);
+        const int r = 16 * q + (lane >> 2);
+        const int c = (lane & 3) ^ ((r >> 2) & 3);
+        a_src[j] = t.a_tile + (long long)min(r, t.rows - 1) * t.Kd + c * 16;
+        a_dst[j] = (unsigned)(q * 1024);
+    }
+    const unsigned b_dst = (unsigned)(kStageA + wave * (kWaveCols * kBK));
+
+    auto issue = [&](int step, int stage) {
+        const unsigned sbase = lds0 + (unsigned)(stage * kStageBytes);
+#pragma unroll
+        for (int j = 0; j < AI; ++j) {
+            dma16(a_src[j] + (long long)step * kBK, sbase + a_dst[j]);
+        }
+        const int8_t *bp = t.wp + (long long)step * (kBLoads * kWave * 16);
+#pragma unroll
+        for (int i = 0; i < kBLoads; ++i) {
+            dma16(bp + i * (kWave * 16), sbase + b_dst + (unsigned)(i * 1024));
+        }
+    };
 
     const int a_row = lane & 31;
     const int a_half = lane >> 5;
+    constexpr int HF = MF >= 4 ? MF / 2 : MF;   // fragments per half
+    constexpr int NH = MF / HF;                 // halves per sub-step
 
-    // A fragments are double-buffered in registers across the four MFMA sub-steps of a step.
-    auto load_frags = [&](v4i *af, const int8_t *stage, int kk) {
+    // Multiplies one stage.  Fragment reads run one half sub-step ahead of the MFMAs that use them.
+    auto compute = [&](const int8_t *stage) {
+        const int8_t *sa = stage;
+        const int8_t *sb = stage + kStageA + wave * (kWaveCols * kBK) + lane * 16;
+        v4i af[2][HF];
+        v4i bf[kKK][kNF];
+        auto load_frags = [&](v4i *dst, int kk, int half) {
 #pragma unroll
-        for (int mf = 0; mf < MF; ++mf) {
-            af[mf] = *(const v4i *)(stage + a_lds_offset(mf * 32 + a_row, kk * 2 + a_half));
-        }
-    };
-    auto compute = [&](const int8_t *stage, const BRegs &b) {
-        v4i af[2][MF];
-        load_frags(af[0], stage, 0);
+            for (int f = 0; f < HF; ++f) {
+                dst[f] = *(const v4i *)(sa + a_lds_offset((half * HF + f) * 32 + a_row, kk * 2 + a_half));
+            }
+        };
 #pragma unroll
         for (int kk = 0; kk < kKK; ++kk) {
-            if (kk + 1 < kKK) {
-                load_frags(af[(kk + 1) & 1], stage, kk + 1);
+#pragma unroll
+            for (int nf = 0; nf < kNF; ++nf) {
+                bf[kk][nf] = *(const v4i *)(sb + (kk * kNF + nf) * 1024);
             }
-            // Keep the LDS reads of the next sub-step ahead of this sub-step's MFMAs: the scheduler
-            // would otherwise sink them to just before their first use and expose the LDS latency.
+        }
+        load_frags(af[0], 0, 0);
+#pragma unroll
+        for (int q = 0; q < kKK * NH; ++q) {
+            const int kk = q / NH;
+            const int half = q % NH;
+            if (q + 1 < kKK * NH) {
+                load_frags(af[(q + 1) & 1], (q + 1) / NH, (q + 1) % NH);
+            }
+            // Keep the LDS reads of the next half ahead of this half's MFMAs: the scheduler would
+            // otherwise sink them to just before their first use and expose the LDS latency.
             __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-            for (int mf = 0; mf < MF; ++mf) {
+            for (int f = 0; f < HF; ++f) {
 #pragma unroll
                 for (int nf = 0; nf < kNF; ++nf) {
-                    acc[mf][nf] =
-                        __builtin_amdgcn_mfma_i32_32x32x32_i8(af[kk & 1][mf], b.v[kk][nf], acc[mf][nf], 0, 0, 0);
+                    acc[half * HF + f][nf] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[q & 1][f], bf[kk][nf],
+                                                                                   acc[half * HF + f][nf], 0, 0, 0);
                 }
             }
             __builtin_amdgcn_sched_barrier(0);
         }
     };
 
-    // One step with static ring indices: fetch step KT_+2 into ring[(CUR+2)%3], multiply ring[CUR].
-#define CAM_GEMM_STEP(CUR, KT_)                                               \
-    {                                                                         \
-        const int kt_ = (KT_);                                                \
-        load_b(bring[((CUR) + 2) % kBDepth], t.wp, min(kt_ + 2, last));       \
-        load_a<MF>(ar, t.a_tile, t.Kd, t.rows, min(kt_ + 1, last), tid);      \
-        compute(a_s[kt_ & 1], bring[(CUR)]);                                  \
-        store_a<MF>(ar, a_s[(kt_ + 1) & 1], tid);                             \
-        __syncthreads();                                                      \
+    // Pipeline.  Every step issues exactly PER_STEP loads per wave and loads retire in order, so "at
+    // most (kStages-2)*PER_STEP outstanding" means that this wave's part of the current step has
+    // landed; the barrier then makes every wave's part visible and also guarantees that all waves
+    // are done reading the previous stage, which the loads issued next overwrite.  Step indices past
+    // the end are clamped (the last step is fetched again), so the loop body has no control flow.
+#pragma unroll
+    for (int p = 0; p < kStages - 1; ++p) {
+        issue(min(p, last), p);
     }
-
-    int kt = 0;
-    for (; kt + kBDepth <= KT; kt += kBDepth) {
-        CAM_GEMM_STEP(0, kt)
-        CAM_GEMM_STEP(1, kt + 1)
-        CAM_GEMM_STEP(2, kt + 2)
+    for (int kt = 0; kt < KT; ++kt) {
+        wait_loads_outstanding<(kStages - 2) * PER_STEP>();
+        barrier_no_fence();
+        issue(min(kt + kStages - 1, last), (kt + kStages - 1) & (kStages - 1));
+        compute(lds + (kt & (kStages - 1)) * kStageBytes);
     }
-    if (kt < KT) {
-        CAM_GEMM_STEP(0, kt)
-    }
-    if (kt + 1 < KT) {
-        CAM_GEMM_STEP(1, kt + 1)
-    }
-#undef CAM_GEMM_STEP
-
-    if (!t.wave_live) {
-        return;
-    }
+    wait_loads_outstanding<0>();
 
     // ---- epilogue, accumulators in registers.
     // Lane l holds column (l & 31) of each 32x32 fragment; register i holds row 8*(i/4) + 4*(l/32) + i%4.
+    // Storing from that layout would write 2- or 4-byte pieces; instead every wave transposes its
+    // results through its own slice of LDS (the pipeline stages are free by now) and writes 16 bytes
+    // per lane: 128 contiguous bytes per output row, 8 rows per store instruction.
+    barrier_no_fence();  // all waves are done with the pipeline stages
+    if (!t.wave_live) {
+        return;
+    }
     const int rows = t.rows;
     const int m0 = t.m0;
     const int N = t.N;
     const int nw = t.nw;
     const int col_in = lane & 31;
     const int row_half = (lane >> 5) * 4;
+    int8_t *slice = lds + wave * (kBM * kEpiRowBytes);
+
+    // Copies the wave's staged rows (128 bytes each) to `dst` + row * row_pitch_bytes.
+    auto flush_rows = [&](int8_t *dst, long long row_pitch_bytes) {
+        const int sub = lane >> 3;    // row inside a group of 8
+        const int piece = lane & 7;   // 16-byte piece of the 128-byte row
+#pragma unroll
+        for (int it = 0; it < MF * 4; ++it) {
+            const int row = it * 8 + sub;
+            const v4u v = *(const v4u *)(slice + row * kEpiRowBytes + piece * 16);
+            if (row < rows) {
+                *(v4u *)(dst + (long long)(m0 + row) * row_pitch_bytes + piece * 16) = v;
+            }
+        }
+    };
+
     if (EPI == kEpiInt32) {
-        int32_t *out = (int32_t *)a.out;
 #pragma unroll
         for (int nf = 0; nf < kNF; ++nf) {
-            const int col = a.gate_up ? (nf * (N / 2) + nw * 32 + col_in) : (nw * kWaveCols + nf * 32 + col_in);
+            const int col0 = a.gate_up ? (nf * (N / 2) + nw * 32) : (nw * kWaveCols + nf * 32);
 #pragma unroll
             for (int mf = 0; mf < MF; ++mf) {
 #pragma unroll
                 for (int i = 0; i < 16; ++i) {
                     const int row = mf * 32 + 8 * (i >> 2) + row_half + (i & 3);
-                    if (row < rows) {
-                        out[(long long)(m0 + row) * N + col] = acc[mf][nf][i];
-                    }
+                    *(int32_t *)(slice + row * kEpiRowBytes + col_in * 4) = acc[mf][nf][i];
                 }
             }
+            flush_rows((int8_t *)a.out + (long long)col0 * 4, (long long)N * 4);
         }
     } else if (EPI == kEpiSwiglu) {
         // t = (float(C) * w_scale[n]) * x_scale[m]; y = silu(t_gate) * t_up
-        float *out = (float *)a.out;
         const int I = N / 2;
         const int c = nw * 32 + col_in;
         const float sg_gate = t.sg[c];
@@ -242,39 +266,35 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs &a, const TileCtx &t, i
 #pragma unroll
             for (int i = 0; i < 16; ++i) {
                 const int row = mf * 32 + 8 * (i >> 2) + row_half + (i & 3);
-                if (row < rows) {
-                    const float xs = row_scale_s[row];
-                    const float tg = __fmul_rn(__fmul_rn((float)acc[mf][0][i], sg_gate), xs);
-                    const float tu = __fmul_rn(__fmul_rn((float)acc[mf][1][i], sg_up), xs);
-                    out[(long long)(m0 + row) * I + c] = __fmul_rn(cam_silu_spec(tg), tu);
-                }
+                const float xs = row_scale_s[row];
+                const float tg = __fmul_rn(__fmul_rn((float)acc[mf][0][i], sg_gate), xs);
+                const float tu = __fmul_rn(__fmul_rn((float)acc[mf][1][i], sg_up), xs);
+                *(float *)(slice + row * kEpiRowBytes + col_in * 4) = __fmul_rn(cam_silu_spec(tg), tu);
             }
         }
+        flush_rows((int8_t *)a.out + (long long)(nw * 32) * 4, (long long)I * 4);
     } else {
-        uint16_t *out = (uint16_t *)a.out;
 #pragma unroll
         for (int nf = 0; nf < kNF; ++nf) {
-            const int col = nw * kWaveCols + nf * 32 + col_in;
-            const float ws = t.sg[col];
+            const float ws = t.sg[nw * kWaveCols + nf * 32 + col_in];
 #pragma unroll
             for (int mf = 0; mf < MF; ++mf) {
 #pragma unroll
                 for (int i = 0; i < 16; ++i) {
                     const int row = mf * 32 + 8 * (i >> 2) + row_half + (i & 3);
-                    if (row < rows) {
-                        const float v = __fmul_rn(__fmul_rn((float)acc[mf][nf][i], ws), row_scale_s[row]);
-                        out[(long long)(m0 + row) * N + col] = (uint16_t)f32_to_bf16_bits(v);
-                    }
+                    const float v = __fmul_rn(__fmul_rn((float)acc[mf][nf][i], ws), row_scale_s[row]);
+                    *(uint16_t *)(slice + row * kEpiRowBytes + (nf * 32 + col_in) * 2) = (uint16_t)f32_to_bf16_bits(v);
                 }
             }
         }
+        flush_rows((int8_t *)a.out + (long long)(nw * kWaveCols) * 2, (long long)N * 2);
     }
 }
 
 template <int EPI>
 __global__ __launch_bounds__(kThreads, 1) void gemm_kernel(GemmArgs a)
 {
-    __shared__ __attribute__((aligned(16))) int8_t a_s[2][kBM * kBK];
+    __shared__ __attribute__((aligned(1024))) int8_t lds[kLdsBytes];
     __shared__ float row_scale_s[kBM];
 
     const int tid = threadIdx.x;
@@ -309,7 +329,7 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_kernel(GemmArgs a)
     t.wave_live = t.nw * kWaveCols < t.N;
     const int8_t *wg = a.per_expert ? a.list.w[g] : a.w + (long long)g * t.Kd * t.N;
     t.sg = a.per_expert ? a.list.s[g] : a.w_scale + (long long)g * t.N;
-    t.wp = (const v4i *)(wg + (long long)(t.wave_live ? t.nw : 0) * t.Kd * kWaveCols) + lane;
+    t.wp = wg + (long long)(t.wave_live ? t.nw : 0) * t.Kd * kWaveCols + lane * 16;
     t.a_tile = a.a + (long long)t.m0 * t.Kd;
 
     if (EPI != kEpiInt32) {
@@ -320,13 +340,13 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_kernel(GemmArgs a)
 
     const int mfrags = (t.rows + 31) >> 5;
     if (mfrags <= 1) {
-        gemm_tile<EPI, 1>(a, t, a_s, row_scale_s);
+        gemm_tile<EPI, 1>(a, t, lds, row_scale_s);
     } else if (mfrags <= 2) {
-        gemm_tile<EPI, 2>(a, t, a_s, row_scale_s);
+        gemm_tile<EPI, 2>(a, t, lds, row_scale_s);
     } else if (mfrags <= 4) {
-        gemm_tile<EPI, 4>(a, t, a_s, row_scale_s);
+        gemm_tile<EPI, 4>(a, t, lds, row_scale_s);
     } else {
-        gemm_tile<EPI, 8>(a, t, a_s, row_scale_s);
+        gemm_tile<EPI, 8>(a, t, lds, row_scale_s);
     }
 }
 
@@ -425,7 +445,7 @@ hipError_t launch_gemm(const GemmArgs &a, hipStream_t stream)
     if (a.max_tiles <= 0) {
         return hipSuccess;
     }
-    if (a.Kd % kBK != 0 || a.N % kWaveCols != 0 || (a.gate_up && a.N % (2 * kWaveCols) != 0)) {
+    if (a.Kd % 128 != 0 || a.N % kWaveCols != 0 || (a.gate_up && a.N % (2 * kWaveCols) != 0)) {
         return hipErrorInvalidValue;
     }
     const int nblocks = (a.N + kBlockCols - 1) / kBlockCols;
