@@ -90,6 +90,18 @@ def main():
     result = {}
     kernels = {}
 
+    # ------------------------------------------------------------------ counter calibration (on request)
+    if "copy" in only:
+        # A plain device-to-device copy of known size: 256 MiB read + 256 MiB written per launch.  Profiling
+        # runs include it so that FETCH_SIZE / WRITE_SIZE readings can be scaled by what they show here.
+        src = torch.empty(256 << 20, dtype=torch.uint8, device=dev).fill_(1)
+        dst = torch.empty_like(src)
+        for _ in range(5):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        log("copy calibration: 5 launches, 268435456 B read + 268435456 B written each")
+        del src, dst
+
     # ------------------------------------------------------------------ dispatch (config 2)
     T, H, E, K = 4096, 7168, 256, 8
     A = T * K
@@ -168,12 +180,28 @@ def main():
                                                0, couts[i % NBUF]], workspace=wss[i % NBUF])
 
         t_comb = time_graph(graph_of(comb_all), replays, warm) / ROT
-        log("combine: %.1f us -> %.0f GB/s = %.1f%% of HBM peak" % (t_comb * 1e6, comb_bytes / t_comb / 1e9,
-                                                                   100 * comb_bytes / t_comb / HBM_PEAK))
-        kernels["combine_gather"] = dict(bound="hbm", us=t_comb * 1e6, bytes=comb_bytes,
-                                         achieved=comb_bytes / t_comb / 1e9, peak=HBM_PEAK / 1e9, unit="GB/s",
-                                         frac=comb_bytes / t_comb / HBM_PEAK,
-                                         note="operator time: inverse-map kernel (32768 threads) + gather kernel")
+        # The operator is two kernels (inverse map, then gather); the two halves exist as operators of their
+        # own, which lets the gather kernel be timed alone.
+        slots = [torch.empty((T, K), dtype=torch.int32, device=dev) for _ in range(NBUF)]
+
+        def index_only():
+            for i in range(ROT):
+                _lib.call("MoeCombineIndex", [info, A, slots[i % NBUF]])
+
+        def gather_only():
+            for i in range(ROT):
+                _lib.call("MoeCombineGather", [ys[i % NBUF], info, slots[i % NBUF], gw, couts[i % NBUF]])
+
+        t_index = time_graph(graph_of(index_only), replays, warm) / ROT
+        t_gather = time_graph(graph_of(gather_only), replays, warm) / ROT
+        log("combine: %.1f us (inverse-map kernel %.1f us, gather kernel %.1f us) -> %.0f GB/s = %.1f%% of HBM peak"
+            % (t_comb * 1e6, t_index * 1e6, t_gather * 1e6, comb_bytes / t_comb / 1e9,
+               100 * comb_bytes / t_comb / HBM_PEAK))
+        gather_bytes = A * H * 2 + A * 4 + A * 4 + T * H * 2  # rows, weights, map, output
+        kernels["combine_gather"] = dict(bound="hbm", us=t_gather * 1e6, bytes=gather_bytes,
+                                         achieved=gather_bytes / t_gather / 1e9, peak=HBM_PEAK / 1e9, unit="GB/s",
+                                         frac=gather_bytes / t_gather / HBM_PEAK)
+        kernels["combine_index"] = dict(bound="latency", us=t_index * 1e6)
         # decode-shaped variant
         Td = 128
         idd, gwd = synth.sigmoid_zipf_routing(Td, E, K, seed=47)
@@ -350,7 +378,8 @@ def main():
         line["ms_per_step"] = total_t * 1e3
         line["dispatch"] = dict(us=t_disp * 1e6, gb_per_s=disp_bytes / t_disp / 1e9, frac_hbm_peak=disp_bytes / t_disp / HBM_PEAK)
         line["combine"] = dict(us=t_comb * 1e6, gb_per_s=comb_bytes / t_comb / 1e9, frac_hbm_peak=comb_bytes / t_comb / HBM_PEAK)
-        dom = "combine_gather" if t_comb >= t_perm else "dispatch_permute_quant"
+        dom = "combine_gather" if kernels["combine_gather"]["us"] >= kernels["dispatch_permute_quant"]["us"] \
+            else "dispatch_permute_quant"
         k = kernels[dom]
         line["roofline"] = {"kernel": dom, "bound": "hbm", "achieved": k["achieved"], "peak": HBM_PEAK / 1e9,
                             "unit": "GB/s", "frac": k["frac"], "traffic": None, "us": k["us"], "bytes": k["bytes"]}

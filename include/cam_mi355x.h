@@ -189,6 +189,27 @@ CAM_API camStatus camMoeCombineNormal(void *workspace, uint64_t workspaceSize, c
                                       camStream_t stream);
 
 /* ------------------------------------------------------------------------------------------------
+ * MoeCombineIndex / MoeCombineGather -- the two halves of MoeCombineNormal as operators of their own, for
+ * callers that combine more than one tensor with the same routing and want to build the (token, k) -> row
+ * map once.  No counterpart in the reference, which scatters rows instead of gathering them
+ * (AK/moe_combine_normal/op_kernel/moe_combine_normal.h:210-275).
+ * MoeCombineIndex:  tokenSrcInfo int32 [3A] -> slotRow int32 [T,K] (entries no row names are left untouched).
+ * MoeCombineGather: recvX bf16 [A,H], tokenSrcInfo int32 [3A], slotRow int32 [T,K], recvTopkWeights fp32
+ * [T,K] -> out bf16 [T,H]; a slotRow entry counts only if the triple of the row it names points back at
+ * that slot, so slotRow needs no initialisation.  Same arithmetic and limits as MoeCombineNormal. */
+CAM_API camStatus camMoeCombineIndexGetWorkspaceSize(const camTensor *tokenSrcInfo, int64_t numRows,
+                                                     const camTensor *slotRow, uint64_t *workspaceSize,
+                                                     camOpExecutor **executor);
+CAM_API camStatus camMoeCombineIndex(void *workspace, uint64_t workspaceSize, camOpExecutor *executor,
+                                     camStream_t stream);
+CAM_API camStatus camMoeCombineGatherGetWorkspaceSize(const camTensor *recvX, const camTensor *tokenSrcInfo,
+                                                      const camTensor *slotRow, const camTensor *recvTopkWeights,
+                                                      const camTensor *out, uint64_t *workspaceSize,
+                                                      camOpExecutor **executor);
+CAM_API camStatus camMoeCombineGather(void *workspace, uint64_t workspaceSize, camOpExecutor *executor,
+                                      camStream_t stream);
+
+/* ------------------------------------------------------------------------------------------------
  * PrepackWeight -- one-time weight layout conversion, off the timed path; the counterpart of
  * torch_npu.npu_format_cast(w, FRACTAL_NZ) (test/cam/ut/fused_deep_moe/test_fused_deep_moe.py:243-246).
  * src int8 [G,Kd,N] or [Kd,N], row-major -> dst int8, same extents, CAM_FORMAT_MFMA_B.

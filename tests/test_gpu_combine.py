@@ -68,3 +68,21 @@ def test_combine_identity_and_linearity(gpu, oracle):
     assert torch.equal(back, x)  # K = 1, weight 1: combine undoes dispatch exactly
     half = cam.moe_combine_normal(rx, assist, plan["recv_count"], ones * 0.5)
     assert torch.equal(half.float(), (x.float() * 0.5).bfloat16().float())
+
+
+def test_combine_index_then_gather_equals_normal(gpu, oracle):
+    announce("combine index + gather")
+    T, K, E, H = 200, 8, 64, 2048
+    ids, w = synth.sigmoid_zipf_routing(T, E, K, seed=21)
+    cnt, off, pos, _ = plan_oracle(oracle, ids.numpy(), E)
+    A = T * K
+    _, _, src = oracle.dispatch(np.zeros((T, 8), np.uint16), ids.numpy(), off, pos, E, 0, A)
+    src_d = torch.from_numpy(src).to(gpu)
+    recv_count = torch.from_numpy((off + cnt).astype(np.int32)).to(gpu)
+    slot = cam.moe_combine_index(src_d, A, T, K)
+    assert_bits_equal(to_np(slot), oracle.rows_from_src_info(src, A, T, K), "slot_row")
+    for seed in (1, 2):  # one index, several gathers
+        y = synth.normal_bf16(A, H, seed=seed).to(gpu)
+        got = cam.moe_combine_gather(y, src_d, slot, w.to(gpu))
+        want = cam.moe_combine_normal(y, src_d, recv_count, w.to(gpu))
+        assert torch.equal(got, want)

@@ -94,6 +94,8 @@ SIGNATURES = {
     "MoeDispatchNormal": [_TP, _TP, _TP, _TP, _TP, _TP, _STR, _I64, _I64, _STR, _I64, _I64, _I64, _I64, _I64,
                           _TP, _TP, _TP],
     "MoeCombineNormal": [_TP, _TP, _TP, _TP, _TP, _STR, _I64, _I64, _STR, _I64, _I64, _I64, _I64, _TP],
+    "MoeCombineIndex": [_TP, _I64, _TP],
+    "MoeCombineGather": [_TP, _TP, _TP, _TP, _TP],
     "PrepackWeight": [_TP, _I64, _TP],
     "GroupedMatmulSwigluQuant": [_TP, _TP, _LP, _LP, _TP, _I64, _TP, _TP],
     "GroupedMatmulDequant": [_TP, _TP, _LP, _LP, _TP, _I64, _TP],

@@ -42,6 +42,8 @@ enum OpTag {
     kOpPlan = 0x504c414e,
     kOpDispatch = 0x44495350,
     kOpCombine = 0x434f4d42,
+    kOpCombIndex = 0x43494458,
+    kOpCombGather = 0x43475448,
     kOpPrepack = 0x5052454b,
     kOpGmm1 = 0x474d4d31,
     kOpGmm2 = 0x474d4d32,
@@ -708,6 +710,87 @@ camStatus camMoeCombineNormalGetWorkspaceSize(const camTensor *recvX, const camT
 camStatus camMoeCombineNormal(void *workspace, uint64_t workspaceSize, camOpExecutor *executor, camStream_t stream)
 {
     return run_phase2(kOpCombine, "camMoeCombineNormal", workspace, workspaceSize, executor, stream);
+}
+
+// ------------------------------------------------------------------------------------------------
+camStatus camMoeCombineIndexGetWorkspaceSize(const camTensor *tokenSrcInfo, int64_t numRows, const camTensor *slotRow,
+                                             uint64_t *workspaceSize, camOpExecutor **executor)
+{
+    CAM_TRY(check_tensor(tokenSrcInfo, "tokenSrcInfo", 1, CAM_DT_INT32));
+    CAM_TRY(check_tensor(slotRow, "slotRow", 2, CAM_DT_INT32));
+    if (numRows < 0 || numRows > 0x7fffffffll || tokenSrcInfo->sizes[0] < 3 * numRows) {
+        return fail(CAM_ERR_SHAPE, "tokenSrcInfo must hold 3 values for each of the %lld rows", (long long)numRows);
+    }
+    const int64_t T = slotRow->sizes[0], K = slotRow->sizes[1];
+    if (K <= 0 || K > cam::kMaxTopk || T * K > 0x7fffffffll) {
+        return fail(CAM_ERR_RANGE, "slotRow must be [T,K] with 0 < K <= %d", cam::kMaxTopk);
+    }
+    const int32_t *src = (const int32_t *)tokenSrcInfo->data;
+    int32_t *slot = (int32_t *)slotRow->data;
+    const int iT = (int)T, iK = (int)K;
+    auto run = [=](void *, hipStream_t s) -> hipError_t {
+        return cam::launch_invert_src_info(src, numRows, iT, iK, slot, s);
+    };
+    return finish_phase1(kOpCombIndex, 0, run, workspaceSize, executor);
+}
+
+camStatus camMoeCombineIndex(void *workspace, uint64_t workspaceSize, camOpExecutor *executor, camStream_t stream)
+{
+    return run_phase2(kOpCombIndex, "camMoeCombineIndex", workspace, workspaceSize, executor, stream);
+}
+
+camStatus camMoeCombineGatherGetWorkspaceSize(const camTensor *recvX, const camTensor *tokenSrcInfo,
+                                              const camTensor *slotRow, const camTensor *recvTopkWeights,
+                                              const camTensor *out, uint64_t *workspaceSize,
+                                              camOpExecutor **executor)
+{
+    CAM_TRY(check_tensor(recvX, "recvX", 2, CAM_DT_BF16));
+    CAM_TRY(check_tensor(tokenSrcInfo, "tokenSrcInfo", 1, CAM_DT_INT32));
+    CAM_TRY(check_tensor(slotRow, "slotRow", 2, CAM_DT_INT32));
+    CAM_TRY(check_tensor(recvTopkWeights, "recvTopkWeights", 2, CAM_DT_FLOAT));
+    CAM_TRY(check_tensor(out, "out", 2, CAM_DT_BF16));
+    const int64_t A = recvX->sizes[0], H = recvX->sizes[1];
+    const int64_t T = recvTopkWeights->sizes[0], K = recvTopkWeights->sizes[1];
+    if (H < 1024 || H > 7168) {
+        return fail(CAM_ERR_RANGE, "hidden size %lld outside [1024, 7168]", (long long)H);
+    }
+    if (H % 8 != 0) {
+        return fail(CAM_ERR_ALIGN, "hidden size %lld must be a multiple of 8", (long long)H);
+    }
+    if (K <= 0 || K > cam::kMaxTopk || T < 1) {
+        return fail(CAM_ERR_RANGE, "recvTopkWeights must be [T,K] with T >= 1 and 0 < K <= %d", cam::kMaxTopk);
+    }
+    if (slotRow->sizes[0] != T || slotRow->sizes[1] != K) {
+        return fail(CAM_ERR_SHAPE, "slotRow must be [T,K]");
+    }
+    if (out->sizes[0] != T || out->sizes[1] != H) {
+        return fail(CAM_ERR_SHAPE, "out must be [T,H]");
+    }
+    if (tokenSrcInfo->sizes[0] < 3 * A) {
+        return fail(CAM_ERR_SHAPE, "tokenSrcInfo must hold 3 values per recvX row");
+    }
+    if (T * K > 0x7fffffffll || A > 0x7fffffffll) {
+        return fail(CAM_ERR_RANGE, "row counts do not fit 32 bits");
+    }
+    CAM_TRY(check_aligned(recvX, "recvX", 16));
+    CAM_TRY(check_aligned(out, "out", 16));
+    cam::CombineArgs g{};
+    g.y = (const uint16_t *)recvX->data;
+    g.slot_row = (const int32_t *)slotRow->data;
+    g.src_info = (const int32_t *)tokenSrcInfo->data;
+    g.w = (const float *)recvTopkWeights->data;
+    g.T = (int)T;
+    g.K = (int)K;
+    g.H = (int)H;
+    g.A = A;
+    g.out = (uint16_t *)out->data;
+    auto run = [g](void *, hipStream_t s) -> hipError_t { return cam::launch_combine(g, s); };
+    return finish_phase1(kOpCombGather, 0, run, workspaceSize, executor);
+}
+
+camStatus camMoeCombineGather(void *workspace, uint64_t workspaceSize, camOpExecutor *executor, camStream_t stream)
+{
+    return run_phase2(kOpCombGather, "camMoeCombineGather", workspace, workspaceSize, executor, stream);
 }
 
 // ------------------------------------------------------------------------------------------------

@@ -189,14 +189,14 @@ __global__ __launch_bounds__(kGlobalThreads) void plan_global_kernel(PlanArgs a,
     if (tid < E) {
         const int32_t *col = hist_in + tid;
         int bb = 0;
-        for (; bb + 8 <= nb; bb += 8) {
-            int v[8];
+        for (; bb + 16 <= nb; bb += 16) {  // 16 independent loads in flight per thread
+            int v[16];
 #pragma unroll
-            for (int j = 0; j < 8; ++j) {
+            for (int j = 0; j < 16; ++j) {
                 v[j] = col[(long long)(bb + j) * E];
             }
 #pragma unroll
-            for (int j = 0; j < 8; ++j) {
+            for (int j = 0; j < 16; ++j) {
                 cnt += v[j];
                 base += (bb + j) < b ? v[j] : 0;
             }

@@ -26,7 +26,7 @@ from ._lib import CamError, CAM_FORMAT_MFMA_B
 
 __all__ = [
     "CamError", "get_dispatch_layout", "moe_dispatch_plan", "moe_dispatch_prefill", "moe_dispatch_normal",
-    "moe_combine_prefill", "moe_combine_normal", "notify_dispatch", "prepack_weight",
+    "moe_combine_prefill", "moe_combine_normal", "moe_combine_index", "moe_combine_gather", "notify_dispatch", "prepack_weight",
     "grouped_matmul_swiglu_quant", "grouped_matmul_dequant", "grouped_matmul_int32", "fused_deep_moe",
 ]
 
@@ -171,6 +171,23 @@ def moe_combine_normal(recv_x, token_src_info, ep_recv_counts, topk_weights, gro
     out = torch.empty((T, recv_x.size(1)), dtype=recv_x.dtype, device=recv_x.device)
     _lib.call("MoeCombineNormal", [recv_x, token_src_info, ep_recv_counts, topk_weights, None, group_ep, num_ranks,
                                    rank, group_ep, 1, 0, ep_recv_counts.size(0), global_bs, out])
+    return out
+
+
+def moe_combine_index(token_src_info, num_rows, num_tokens, top_k):
+    """(token, k) -> row map from the (srcRank, token, k) triples; build once, reuse for several gathers."""
+    _require_gpu(token_src_info, "token_src_info")
+    slot_row = torch.empty((num_tokens, top_k), dtype=torch.int32, device=token_src_info.device)
+    _lib.call("MoeCombineIndex", [token_src_info, num_rows, slot_row])
+    return slot_row
+
+
+def moe_combine_gather(recv_x, token_src_info, slot_row, topk_weights, out=None):
+    """Weighted gather-reduce with a prebuilt map: -> combined bf16 [T,H]."""
+    _require_gpu(recv_x, "recv_x")
+    if out is None:
+        out = torch.empty((topk_weights.size(0), recv_x.size(1)), dtype=recv_x.dtype, device=recv_x.device)
+    _lib.call("MoeCombineGather", [recv_x, token_src_info, slot_row, topk_weights, out])
     return out
 
 
