@@ -11,7 +11,7 @@ namespace cam {
 constexpr int kMaxExperts = 512;   // E <= 512 on every CAM operator
 constexpr int kMaxRanks = 384;
 constexpr int kMaxTopk = 16;
-constexpr int kGemmTileM = 256;    // rows per GEMM tile (tile table granularity)
+constexpr int kGemmTileM = 128;    // rows per GEMM tile (tile table granularity)
 constexpr int kMaxListExperts = 64;  // per-expert weight tensors that fit in the kernel arguments
 
 // ---------------------------------------------------------------------------------------------

@@ -47,7 +47,7 @@ constexpr int kThreads = 256;
 constexpr int kWaveCols = 64;
 constexpr int kBlockCols = 4 * kWaveCols;
 constexpr int kNumXcd = 8;
-constexpr int kStages = 4;
+constexpr int kStages = 3;
 constexpr int kStageA = kBM * kBK;                    // 16 KB of activations per stage
 constexpr int kStageB = 4 * kWaveCols * kBK;          // 16 KB of weights per stage (4 KB per wave)
 constexpr int kStageBytes = kStageA + kStageB;
@@ -88,6 +88,7 @@ struct TileCtx {
     const int8_t *wp;       // this wave's weight stream (+ 16 * lane)
     const float *sg;        // this expert's per-channel scales
     int m0, rows, nw, Kd, N;
+    int k_start;            // first K step of this workgroup (the K loop wraps around)
     bool wave_live;
 };
 
@@ -95,7 +96,7 @@ struct TileCtx {
 template <int EPI, int MF>
 __device__ __forceinline__ void gemm_tile(const GemmArgs &a, const TileCtx &t, int8_t *lds, const float *row_scale_s)
 {
-    constexpr int AI = MF >= 2 ? MF / 2 : 1;   // activation loads per wave and step (1 KB each)
+    constexpr int AI = (MF + 1) / 2;           // activation loads per wave and step (1 KB each)
     constexpr int PER_STEP = AI + kBLoads;     // loads per wave and step
     const int tid = threadIdx.x;
     const int lane = tid & (kWave - 1);
@@ -125,7 +126,7 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs &a, const TileCtx &t, i
     unsigned a_dst[AI];
 #pragma unroll
     for (int j = 0; j < AI; ++j) {
-        const int q = MF >= 2 ? j * 4 + wave : (wave & 1);
+        const int q = MF >= 2 ? j * 4 + wave : (wave & 1);  // MF == 3: loads 6, 7 bring rows of a fourth, unused fragment
         const int r = 16 * q + (lane >> 2);
         const int c = (lane & 3) ^ ((r >> 2) & 3);
         a_src[j] = t.a_tile + (long long)min(r, t.rows - 1) * t.Kd + c * 16;
@@ -133,7 +134,12 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs &a, const TileCtx &t, i
     }
     const unsigned b_dst = (unsigned)(kStageA + wave * (kWaveCols * kBK));
 
-    auto issue = [&](int step, int stage) {
+    // Step s of the pipeline reads K step (k_start + s) mod KT: an integer dot product does not care
+    // about the order, and workgroups that start at different depths do not all pull on the same
+    // memory channels at the same moment (their weight streams lie a fixed stride apart).
+    auto issue = [&](int s_idx, int stage) {
+        int step = t.k_start + s_idx;
+        step = step >= KT ? step - KT : step;
         const unsigned sbase = lds0 + (unsigned)(stage * kStageBytes);
 #pragma unroll
         for (int j = 0; j < AI; ++j) {
@@ -148,7 +154,7 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs &a, const TileCtx &t, i
 
     const int a_row = lane & 31;
     const int a_half = lane >> 5;
-    constexpr int HF = MF >= 4 ? MF / 2 : MF;   // fragments per half
+    constexpr int HF = MF == 4 ? 2 : MF;        // fragments per half
     constexpr int NH = MF / HF;                 // halves per sub-step
 
     // Multiplies one stage.  Fragment reads run one half sub-step ahead of the MFMAs that use them.
@@ -205,8 +211,8 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs &a, const TileCtx &t, i
     for (int kt = 0; kt < KT; ++kt) {
         wait_loads_outstanding<(kStages - 2) * PER_STEP>();
         barrier_no_fence();
-        issue(min(kt + kStages - 1, last), (kt + kStages - 1) & (kStages - 1));
-        compute(lds + (kt & (kStages - 1)) * kStageBytes);
+        issue(min(kt + kStages - 1, last), (kt + kStages - 1) % kStages);
+        compute(lds + (kt % kStages) * kStageBytes);
     }
     wait_loads_outstanding<0>();
 
@@ -292,7 +298,7 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs &a, const TileCtx &t, i
 }
 
 template <int EPI>
-__global__ __launch_bounds__(kThreads, 1) void gemm_kernel(GemmArgs a)
+__global__ __launch_bounds__(kThreads, 2) void gemm_kernel(GemmArgs a)
 {
     __shared__ __attribute__((aligned(1024))) int8_t lds[kLdsBytes];
     __shared__ float row_scale_s[kBM];
@@ -331,6 +337,9 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_kernel(GemmArgs a)
     t.sg = a.per_expert ? a.list.s[g] : a.w_scale + (long long)g * t.N;
     t.wp = wg + (long long)(t.wave_live ? t.nw : 0) * t.Kd * kWaveCols + lane * 16;
     t.a_tile = a.a + (long long)t.m0 * t.Kd;
+    // The start depth depends on the expert and the column block only, so that the row tiles of one
+    // expert, which stream the same weight panel, stay in step and find each other's lines in L2.
+    t.k_start = (int)((((long long)g * nblocks + nb) * 37) % (t.Kd / kBK));
 
     if (EPI != kEpiInt32) {
         for (int r = tid; r < kBM; r += kThreads) {
@@ -343,10 +352,10 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_kernel(GemmArgs a)
         gemm_tile<EPI, 1>(a, t, lds, row_scale_s);
     } else if (mfrags <= 2) {
         gemm_tile<EPI, 2>(a, t, lds, row_scale_s);
-    } else if (mfrags <= 4) {
-        gemm_tile<EPI, 4>(a, t, lds, row_scale_s);
+    } else if (mfrags <= 3) {
+        gemm_tile<EPI, 3>(a, t, lds, row_scale_s);
     } else {
-        gemm_tile<EPI, 8>(a, t, lds, row_scale_s);
+        gemm_tile<EPI, 4>(a, t, lds, row_scale_s);
     }
 }
 
