@@ -279,7 +279,10 @@ camStatus check_gemm_dims(const char *op, int64_t Kd, int64_t N, bool gate_up)
 }
 
 int max_tiles_for(int64_t rows, int64_t G) { return (int)(rows / cam::kGemmTileM + G); }
-uint64_t tile_table_bytes(int max_tiles) { return (uint64_t)(4 + 4 * (int64_t)max_tiles) * 4; }
+uint64_t tile_table_bytes(int max_tiles)
+{
+    return (uint64_t)(cam::kTileHeader + cam::kTileRecord * (int64_t)max_tiles) * 4;
+}
 
 }  // namespace
 

@@ -13,6 +13,11 @@ constexpr int kMaxRanks = 384;
 constexpr int kMaxTopk = 16;
 constexpr int kGemmTileM = 128;    // rows per GEMM tile (tile table granularity)
 constexpr int kMaxListExperts = 64;  // per-expert weight tensors that fit in the kernel arguments
+// GEMM tile table: kTileHeader ints {tile count, total rows, active tokens, 0}, then one record of
+// kTileRecord ints per tile: {expert, first row, rows, first tile of the expert, tiles of the expert, 0, 0, 0}.
+// Tiles are listed in expert order; the rows of an expert are split evenly over its tiles.
+constexpr int kTileHeader = 4;
+constexpr int kTileRecord = 8;
 
 // ---------------------------------------------------------------------------------------------
 // Routing plan: counts, offsets, within-expert ranks, receive bookkeeping, GEMM tile table.
@@ -32,7 +37,7 @@ struct PlanArgs {
     int64_t *total;           // [1]    optional
     int32_t *per_rank_zero;   // [R]    optional: zeroed here so a later kernel can accumulate into it
     int R;
-    int32_t *tiles;           // optional GEMM tile table: [0]=tile count, then int4 (expert, m0, rows, 0) from [4]
+    int32_t *tiles;           // optional GEMM tile table (layout: kTileHeader / kTileRecord below)
     int32_t *hist_ws;         // required scratch of plan_workspace_bytes(T, K, E) bytes
 };
 uint64_t plan_workspace_bytes(int64_t T, int64_t K, int E);

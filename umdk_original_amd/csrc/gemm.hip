@@ -307,9 +307,12 @@ __global__ __launch_bounds__(kThreads, 2) void gemm_kernel(GemmArgs a)
     const int lane = tid & (kWave - 1);
     const int wave = tid >> 6;
 
-    // ---- which tile, which column block.  Work ids run (tile, column block) with the column block
-    // fastest; each XCD takes one contiguous run of ids, so the workgroups that share a tile's
-    // activation rows, and neighbouring tiles of one expert that share weight panels, meet in one L2.
+    // ---- which tile, which column block.
+    // Each XCD takes one contiguous run of work ids (workgroup i runs on XCD i % 8).  Inside an expert
+    // with n tiles the ids run: a group of column blocks, and inside the group the column block, and
+    // inside the column block the expert's n tiles.  The workgroups that are resident together on an
+    // XCD (64) then are all the row tiles of an expert for a few column blocks: they stream the same
+    // weight panels at the same depth and find each other's lines in L2, so a panel is fetched once.
     const int num_tiles = min(a.tiles[0], a.max_tiles);
     const int nblocks = (a.N + kBlockCols - 1) / kBlockCols;
     const long long total_work = (long long)num_tiles * nblocks;
@@ -319,9 +322,13 @@ __global__ __launch_bounds__(kThreads, 2) void gemm_kernel(GemmArgs a)
     if (slot >= chunk || wid >= total_work) {
         return;
     }
-    const int tile = (int)(wid / nblocks);
-    const int nb = (int)(wid - (long long)tile * nblocks);
-    const int32_t *te = a.tiles + 4 + 4 * tile;
+    const int32_t *probe = a.tiles + kTileHeader + kTileRecord * (int)(wid / nblocks);
+    const int first = probe[3];
+    const int ntile = max(probe[4], 1);
+    const int local = (int)(wid - (long long)first * nblocks);  // id inside the expert
+    const int tile = first + local % ntile;
+    const int nb = local / ntile;
+    const int32_t *te = a.tiles + kTileHeader + kTileRecord * tile;
     const int g = te[0];
     TileCtx t;
     t.m0 = te[1];

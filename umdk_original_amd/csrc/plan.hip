@@ -83,6 +83,25 @@ __device__ __forceinline__ int count_active(const uint8_t *mask, int T, int tid,
     return *slot;
 }
 
+// Tile records of one expert: its `cnt` rows from row `off` on, split evenly over `nt` tiles (equal
+// tiles keep the workgroups that stream the same weight panel in step with each other).
+__device__ __forceinline__ void write_tile_records(int32_t *tiles, int expert, int off, int cnt, int tbase, int nt,
+                                                   int max_tiles)
+{
+    const int q = nt > 0 ? (cnt + nt - 1) / nt : 0;
+    for (int j = 0; j < nt && tbase + j < max_tiles; ++j) {
+        int32_t *t = tiles + kTileHeader + kTileRecord * (tbase + j);
+        t[0] = expert;
+        t[1] = off + j * q;
+        t[2] = min(q, cnt - j * q);
+        t[3] = tbase;
+        t[4] = nt;
+        t[5] = 0;
+        t[6] = 0;
+        t[7] = 0;
+    }
+}
+
 // Phase 1.  Workgroup b owns the flat entries [b*chunk, (b+1)*chunk), chunk = IT*256; wave w of it the
 // IT*64 entries from b*chunk + w*IT*64.  Each lane keeps its IT ids in registers.  64 ids at a time,
 // lanes holding the same id find each other with one ballot per id bit; the rank inside the wave is the
@@ -254,13 +273,7 @@ __global__ __launch_bounds__(kGlobalThreads) void plan_global_kernel(PlanArgs a,
         const int nt = tid < E ? (cnt + kGemmTileM - 1) / kGemmTileM : 0;
         const int tbase = block_exclusive_scan<NW>(nt, tid, scan_s, &total_s);
         if (tid < E) {
-            for (int j = 0; j < nt; ++j) {
-                int32_t *t = a.tiles + 4 + 4 * (tbase + j);
-                t[0] = tid;
-                t[1] = off + j * kGemmTileM;
-                t[2] = min(kGemmTileM, cnt - j * kGemmTileM);
-                t[3] = 0;
-            }
+            write_tile_records(a.tiles, tid, off, cnt, tbase, nt, 0x7fffffff);
         }
         if (tid == 0) {
             a.tiles[0] = total_s;
@@ -368,13 +381,7 @@ __global__ __launch_bounds__(kScanThreads) void build_tiles_kernel(const int64_t
     int tbase = block_exclusive_scan<kScanThreads / kWave>(nt, tid, scan_s, &total_s);
     int num_tiles = min(total_s, max_tiles);
     if (tid < G) {
-        for (int j = 0; j < nt && tbase + j < max_tiles; ++j) {  // a corrupt list cannot overrun the table
-            int32_t *t = tiles + 4 + 4 * (tbase + j);
-            t[0] = tid;
-            t[1] = (int)m0 + j * kGemmTileM;
-            t[2] = min(kGemmTileM, cnt - j * kGemmTileM);
-            t[3] = 0;
-        }
+        write_tile_records(tiles, tid, (int)m0, cnt, tbase, nt, max_tiles);  // a corrupt list cannot overrun the table
     }
     __syncthreads();
     int rows_total = block_exclusive_scan<kScanThreads / kWave>(cnt, tid, scan_s, &total_s);
