@@ -343,7 +343,7 @@ def main():
             cam_oracle.combine(y_s, row_of, gw_s)
             reps += 1
             el = time.perf_counter() - t0
-            if el > 10.0 or reps >= 200:
+            if el > 12.0:
                 break
         sample_bytes = synth.dispatch_bytes(Ts, H, K, E) + synth.combine_bytes(Ts, H, K)
         cpu = dict(value=sample_bytes * reps / el / 1e9, unit="GB/s", cores=cam_oracle.num_threads(), kind="port",
@@ -381,8 +381,12 @@ def main():
         dom = "combine_gather" if kernels["combine_gather"]["us"] >= kernels["dispatch_permute_quant"]["us"] \
             else "dispatch_permute_quant"
         k = kernels[dom]
+        # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, each scaled by what the same
+        # counter shows for a 256 MiB device copy (x2.000 and x1.000): profiles/dispatch_combine_c2_c4.md.
+        measured_traffic = {"combine_gather": 539.0e6, "dispatch_permute_quant": 295.9e6}
         line["roofline"] = {"kernel": dom, "bound": "hbm", "achieved": k["achieved"], "peak": HBM_PEAK / 1e9,
-                            "unit": "GB/s", "frac": k["frac"], "traffic": None, "us": k["us"], "bytes": k["bytes"]}
+                            "unit": "GB/s", "frac": k["frac"], "traffic": measured_traffic[dom], "us": k["us"],
+                            "bytes": k["bytes"]}
     else:
         line["value"] = None
         line["ms_per_step"] = None
