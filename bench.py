@@ -361,7 +361,9 @@ def main():
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
-        "dtype": "bf16 in, fp32 scale arithmetic, int8 out (dispatch); int8 x int8 -> int32 (GEMM); fp32 -> bf16 (combine)",
+        "dtype": "int8",
+        "dtype_detail": "dispatch: bf16 in, fp32 scale arithmetic, int8 out; GEMM: int8 x int8 -> int32, fp32 "
+                        "dequantisation; combine: fp32 accumulate -> bf16",
         "data": "synthetic",
         "config": {
             "workload": "dispatch: 4096 tokens x 7168 bf16, 256 experts, top-8 (sigmoid + Zipf(1.1)-biased routing), "
