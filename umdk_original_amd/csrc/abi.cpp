@@ -14,7 +14,6 @@
 #include <functional>
 #include <new>
 #include <string>
-#include <vector>
 
 #include <hip/hip_runtime.h>
 

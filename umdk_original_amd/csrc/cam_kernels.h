@@ -124,9 +124,6 @@ hipError_t launch_requant(const float *y, int64_t max_rows, int I, const int32_t
 
 hipError_t launch_prepack(const int8_t *src, int8_t *dst, int G, int Kd, int N, int gate_up, hipStream_t stream);
 
-// Small utilities.
-hipError_t launch_cast_i64_to_i32(const int64_t *src, int32_t *dst, int64_t n, hipStream_t stream);
-
 }  // namespace cam
 
 #endif  // CAM_KERNELS_H_

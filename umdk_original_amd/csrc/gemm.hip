@@ -9,12 +9,14 @@
 //   GMM2 epilogue   FDM/epilogue/block/block_epilogue_per_token_dequant.hpp:665-684
 //
 // Design (not a translation of the cube/vector split above).
-//   * One workgroup = 4 waves = a tile of up to 256 rows of ONE expert x 256 packed weight columns.
-//     Every wave covers all rows of the tile and its own 64 columns (256 int32 accumulators per lane,
-//     the most the register file allows): the grouped shape is bound by streaming the weights, and a
-//     tile this tall makes every weight byte fetched feed up to 256 rows.
+//   * One workgroup = 4 waves = a tile of up to 128 rows of ONE expert x 256 packed weight columns.
+//     Every wave covers all rows of the tile and its own 64 columns (128 int32 accumulators per lane),
+//     and two workgroups share a CU so that one runs MFMAs while the other waits on memory or
+//     writes its epilogue.  The grouped shape is bound by streaming the weights: a tall tile makes
+//     every weight byte fetched feed up to 128 rows, and sibling tiles of one expert are scheduled
+//     next to each other so that they find the same weight panel in L2.
 //   * Both operands travel global -> LDS with direct-to-LDS loads (16 bytes per lane, no registers),
-//     four stages deep, three 64-deep K steps ahead of the MFMAs.  Weights were laid out once by the
+//     three stages deep, two 64-deep K steps ahead of the MFMAs.  Weights were laid out once by the
 //     prepack kernel in the lane order the MFMA wants, so a wave's weight load is 1 KB of contiguous
 //     memory that lands in LDS already in fragment order.  Activation rows are placed with an XOR
 //     swizzle of their 16-byte chunks (chosen on the global side, since a direct-to-LDS load writes
@@ -25,10 +27,13 @@
 //   * The int32 accumulators stay in registers through the epilogue: dequantisation, SiLU and the
 //     gate*up product are applied in place; the int32 tile never goes to memory.
 //     For GMM1 the prepack pairs gate column c with up column I+c inside one wave.
-//   * Variable rows per expert: a device-built tile table lists (expert, first row, rows); empty
-//     experts own no tile.  The grid is sized for the worst case and surplus workgroups exit at once.
-//     Work ids are dealt to the 8 XCDs in contiguous runs so that workgroups sharing activation rows
-//     (same tile, neighbouring column blocks) run on one XCD and share its L2.
+//   * Variable rows per expert: a device-built tile table lists, per tile, (expert, first row, rows,
+//     first tile of the expert, tiles of the expert); an expert's rows are split evenly over its
+//     tiles and empty experts own no tile.  The grid is sized for the worst case and surplus
+//     workgroups exit at once.  Work ids are dealt to the 8 XCDs in contiguous runs, tile index
+//     fastest inside an expert, so that the workgroups reading one weight panel run together on one
+//     XCD and share its L2; each (expert, column block) starts its K loop at a different step so
+//     that concurrent panels do not hit the same memory channels in lockstep.
 //   * The K order inside a 32-deep MFMA step is whatever the two operands agree on (an integer dot
 //     product does not care), which is what lets both be loaded as plain 16-byte pieces.
 #include "cam_device.h"
@@ -48,7 +53,7 @@ constexpr int kWaveCols = 64;
 constexpr int kBlockCols = 4 * kWaveCols;
 constexpr int kNumXcd = 8;
 constexpr int kStages = 3;
-constexpr int kStageA = kBM * kBK;                    // 16 KB of activations per stage
+constexpr int kStageA = kBM * kBK;                    // 8 KB of activations per stage
 constexpr int kStageB = 4 * kWaveCols * kBK;          // 16 KB of weights per stage (4 KB per wave)
 constexpr int kStageBytes = kStageA + kStageB;
 constexpr int kBLoads = kKK * kNF;                    // weight loads per wave and step

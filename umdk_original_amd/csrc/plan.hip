@@ -394,15 +394,6 @@ __global__ __launch_bounds__(kScanThreads) void build_tiles_kernel(const int64_t
     }
 }
 
-__global__ void cast_i64_to_i32_kernel(const int64_t *src, int32_t *dst, long long n)
-{
-    long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
-    if (i < n) {
-        long long v = src[i];
-        dst[i] = v < -2147483647ll ? -1 : (v > 2147483647ll ? 2147483647 : (int32_t)v);
-    }
-}
-
 void plan_geometry(long long n_all, int *it_out, int *nb_out)
 {
     int it = 1;
@@ -490,16 +481,6 @@ hipError_t launch_build_tiles(const int64_t *group_list, int cumulative, int G, 
 {
     hipLaunchKernelGGL(build_tiles_kernel, dim3(1), dim3(kScanThreads), 0, stream, group_list, cumulative, G,
                        (long long)max_rows, max_tiles, tiles);
-    return hipGetLastError();
-}
-
-hipError_t launch_cast_i64_to_i32(const int64_t *src, int32_t *dst, int64_t n, hipStream_t stream)
-{
-    if (n <= 0) {
-        return hipSuccess;
-    }
-    hipLaunchKernelGGL(cast_i64_to_i32_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, stream, src, dst,
-                       (long long)n);
     return hipGetLastError();
 }
 
