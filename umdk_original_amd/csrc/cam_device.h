@@ -24,13 +24,10 @@ __device__ __forceinline__ float bf16_bits_to_f32(uint32_t bits16)
 // Round-to-nearest-even fp32 -> bf16 bit pattern (NaN stays a quiet NaN).
 __device__ __forceinline__ uint32_t f32_to_bf16_bits(float f)
 {
-    uint32_t u = __float_as_uint(f);
-    if ((u & 0x7fffffffu) > 0x7f800000u) {
-        return (u >> 16) | 0x0040u;
-    }
-    uint32_t lsb = (u >> 16) & 1u;
-    u += 0x7fffu + lsb;
-    return u >> 16;
+    const uint32_t u = __float_as_uint(f);
+    const uint32_t rounded = (u + 0x7fffu + ((u >> 16) & 1u)) >> 16;
+    const uint32_t quiet = (u >> 16) | 0x0040u;
+    return (u & 0x7fffffffu) > 0x7f800000u ? quiet : rounded;  // both sides computed: a select, no branch
 }
 
 __device__ __forceinline__ int lane_id()

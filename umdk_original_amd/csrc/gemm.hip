@@ -25,15 +25,18 @@
 //     Left to itself the compiler drains every outstanding load at each workgroup barrier and before
 //     LDS reads it cannot prove independent, which serialises the pipeline.
 //   * The int32 accumulators stay in registers through the epilogue: dequantisation, SiLU and the
-//     gate*up product are applied in place; the int32 tile never goes to memory.
+//     gate*up product are applied in place; the int32 tile never goes to memory.  The MFMAs take the
+//     weights as their first operand, so a lane ends up with ONE activation row and runs of four
+//     consecutive weight columns: one row scale per lane, column scales as 16-byte vectors, 8- or
+//     16-byte pieces into the LDS staging from which whole 128-byte lines are stored.
 //     For GMM1 the prepack pairs gate column c with up column I+c inside one wave.
 //   * Variable rows per expert: a device-built tile table lists, per tile, (expert, first row, rows,
 //     first tile of the expert, tiles of the expert); an expert's rows are split evenly over its
 //     tiles and empty experts own no tile.  The grid is sized for the worst case and surplus
 //     workgroups exit at once.  Work ids are dealt to the 8 XCDs in contiguous runs, tile index
 //     fastest inside an expert, so that the workgroups reading one weight panel run together on one
-//     XCD and share its L2; each (expert, column block) starts its K loop at a different step so
-//     that concurrent panels do not hit the same memory channels in lockstep.
+//     XCD and share its L2; all workgroups of an expert start their K loop at the same step (which
+//     differs from expert to expert), so that they also find each other's activation rows there.
 //   * The K order inside a 32-deep MFMA step is whatever the two operands agree on (an integer dot
 //     product does not care), which is what lets both be loaded as plain 16-byte pieces.
 #include "cam_device.h"
@@ -196,7 +199,9 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs &a, const TileCtx &t, i
             for (int f = 0; f < HF; ++f) {
 #pragma unroll
                 for (int nf = 0; nf < kNF; ++nf) {
-                    acc[half * HF + f][nf] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[q & 1][f], bf[kk][nf],
+                    // Weights as the first operand: the result tile comes out transposed, i.e. a lane
+                    // holds ONE activation row and 4 consecutive weight columns per register quad.
+                    acc[half * HF + f][nf] = __builtin_amdgcn_mfma_i32_32x32x32_i8(bf[kk][nf], af[q & 1][f],
                                                                                    acc[half * HF + f][nf], 0, 0, 0);
                 }
             }
@@ -222,10 +227,11 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs &a, const TileCtx &t, i
     wait_loads_outstanding<0>();
 
     // ---- epilogue, accumulators in registers.
-    // Lane l holds column (l & 31) of each 32x32 fragment; register i holds row 8*(i/4) + 4*(l/32) + i%4.
-    // Storing from that layout would write 2- or 4-byte pieces; instead every wave transposes its
-    // results through its own slice of LDS (the pipeline stages are free by now) and writes 16 bytes
-    // per lane: 128 contiguous bytes per output row, 8 rows per store instruction.
+    // Lane l holds activation row (l & 31) of each 32x32 fragment; registers 4j .. 4j+3 hold the four
+    // consecutive weight columns 8j + 4*(l/32) + 0..3.  Dequantisation runs on that layout with one
+    // row scale per lane and fragment and the column scales fetched as 16-byte vectors.  To store
+    // whole 128-byte lines, every wave passes its results through its own slice of LDS (the pipeline
+    // stages are free by now): 128 staged bytes per row, then 16 bytes per lane and 8 rows per store.
     barrier_no_fence();  // all waves are done with the pipeline stages
     if (!t.wave_live) {
         return;
@@ -234,8 +240,8 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs &a, const TileCtx &t, i
     const int m0 = t.m0;
     const int N = t.N;
     const int nw = t.nw;
-    const int col_in = lane & 31;
-    const int row_half = (lane >> 5) * 4;
+    const int row_in = lane & 31;
+    const int col_half = (lane >> 5) * 4;
     int8_t *slice = lds + wave * (kBM * kEpiRowBytes);
 
     // Copies the wave's staged rows (128 bytes each) to `dst` + row * row_pitch_bytes.
@@ -259,9 +265,10 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs &a, const TileCtx &t, i
 #pragma unroll
             for (int mf = 0; mf < MF; ++mf) {
 #pragma unroll
-                for (int i = 0; i < 16; ++i) {
-                    const int row = mf * 32 + 8 * (i >> 2) + row_half + (i & 3);
-                    *(int32_t *)(slice + row * kEpiRowBytes + col_in * 4) = acc[mf][nf][i];
+                for (int j = 0; j < 4; ++j) {
+                    const v4i v = {acc[mf][nf][4 * j], acc[mf][nf][4 * j + 1], acc[mf][nf][4 * j + 2],
+                                   acc[mf][nf][4 * j + 3]};
+                    *(v4i *)(slice + (mf * 32 + row_in) * kEpiRowBytes + (8 * j + col_half) * 4) = v;
                 }
             }
             flush_rows((int8_t *)a.out + (long long)col0 * 4, (long long)N * 4);
@@ -269,32 +276,48 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs &a, const TileCtx &t, i
     } else if (EPI == kEpiSwiglu) {
         // t = (float(C) * w_scale[n]) * x_scale[m]; y = silu(t_gate) * t_up
         const int I = N / 2;
-        const int c = nw * 32 + col_in;
-        const float sg_gate = t.sg[c];
-        const float sg_up = t.sg[I + c];
+        v4f sg_gate[4], sg_up[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            sg_gate[j] = *(const v4f *)(t.sg + nw * 32 + 8 * j + col_half);
+            sg_up[j] = *(const v4f *)(t.sg + I + nw * 32 + 8 * j + col_half);
+        }
 #pragma unroll
         for (int mf = 0; mf < MF; ++mf) {
+            const float xs = row_scale_s[mf * 32 + row_in];
 #pragma unroll
-            for (int i = 0; i < 16; ++i) {
-                const int row = mf * 32 + 8 * (i >> 2) + row_half + (i & 3);
-                const float xs = row_scale_s[row];
-                const float tg = __fmul_rn(__fmul_rn((float)acc[mf][0][i], sg_gate), xs);
-                const float tu = __fmul_rn(__fmul_rn((float)acc[mf][1][i], sg_up), xs);
-                *(float *)(slice + row * kEpiRowBytes + col_in * 4) = __fmul_rn(cam_silu_spec(tg), tu);
+            for (int j = 0; j < 4; ++j) {
+                v4f y;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    const float tg = __fmul_rn(__fmul_rn((float)acc[mf][0][4 * j + e], sg_gate[j][e]), xs);
+                    const float tu = __fmul_rn(__fmul_rn((float)acc[mf][1][4 * j + e], sg_up[j][e]), xs);
+                    y[e] = __fmul_rn(cam_silu_spec(tg), tu);
+                }
+                *(v4f *)(slice + (mf * 32 + row_in) * kEpiRowBytes + (8 * j + col_half) * 4) = y;
             }
         }
         flush_rows((int8_t *)a.out + (long long)(nw * 32) * 4, (long long)I * 4);
     } else {
 #pragma unroll
         for (int nf = 0; nf < kNF; ++nf) {
-            const float ws = t.sg[nw * kWaveCols + nf * 32 + col_in];
+            v4f ws[4];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                ws[j] = *(const v4f *)(t.sg + nw * kWaveCols + nf * 32 + 8 * j + col_half);
+            }
 #pragma unroll
             for (int mf = 0; mf < MF; ++mf) {
+                const float xs = row_scale_s[mf * 32 + row_in];
 #pragma unroll
-                for (int i = 0; i < 16; ++i) {
-                    const int row = mf * 32 + 8 * (i >> 2) + row_half + (i & 3);
-                    const float v = __fmul_rn(__fmul_rn((float)acc[mf][nf][i], ws), row_scale_s[row]);
-                    *(uint16_t *)(slice + row * kEpiRowBytes + (nf * 32 + col_in) * 2) = (uint16_t)f32_to_bf16_bits(v);
+                for (int j = 0; j < 4; ++j) {
+                    uint32_t b[4];
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        b[e] = f32_to_bf16_bits(__fmul_rn(__fmul_rn((float)acc[mf][nf][4 * j + e], ws[j][e]), xs));
+                    }
+                    const v2u v = {b[0] | (b[1] << 16), b[2] | (b[3] << 16)};
+                    *(v2u *)(slice + (mf * 32 + row_in) * kEpiRowBytes + (nf * 32 + 8 * j + col_half) * 2) = v;
                 }
             }
         }
@@ -349,9 +372,9 @@ __global__ __launch_bounds__(kThreads, 2) void gemm_kernel(GemmArgs a)
     t.sg = a.per_expert ? a.list.s[g] : a.w_scale + (long long)g * t.N;
     t.wp = wg + (long long)(t.wave_live ? t.nw : 0) * t.Kd * kWaveCols + lane * 16;
     t.a_tile = a.a + (long long)t.m0 * t.Kd;
-    // The start depth depends on the expert and the column block only, so that the row tiles of one
-    // expert, which stream the same weight panel, stay in step and find each other's lines in L2.
-    t.k_start = (int)((((long long)g * nblocks + nb) * 37) % (t.Kd / kBK));
+    // The start depth depends on the expert only, so that all workgroups of an expert, which share
+    // activation rows or weight panels, stay in step and find each other's lines in L2.
+    t.k_start = (int)(((long long)g * 37) % (t.Kd / kBK));
 
     if (EPI != kEpiInt32) {
         for (int r = tid; r < kBM; r += kThreads) {
