@@ -25,6 +25,8 @@ def _inputs(sizes, Kd, N, seed, wrange=127):
     ([1, 0, 33, 128, 129, 0, 7], 256, 256),
     ([300, 2, 0, 64], 384, 640),
     ([17, 40], 1024, 1152),
+    ([700, 5, 0, 385], 128, 384),    # several row tiles per expert, shortest K loop, ragged column block
+    ([257], 2048, 128),              # three uneven tiles, long K loop that wraps around its start depth
 ])
 def test_int32_accumulators_bit_exact(gpu, oracle, sizes, Kd, N, gate_up):
     announce("gemm int32 sizes=%s Kd=%d N=%d gate_up=%s" % (sizes, Kd, N, gate_up))
