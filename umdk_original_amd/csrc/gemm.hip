@@ -145,20 +145,27 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs &a, const TileCtx &t, i
     // Step s of the pipeline reads K step (k_start + s) mod KT: an integer dot product does not care
     // about the order, and workgroups that start at different depths do not all pull on the same
     // memory channels at the same moment (their weight streams lie a fixed stride apart).
-    auto issue = [&](int s_idx, int stage) {
+    // Issues the loads of pipeline step s_idx whose index i (activation loads first, then the weight
+    // loads) satisfies i % nparts == part.
+    auto issue_part = [&](int s_idx, int stage, int part, int nparts) {
         int step = t.k_start + s_idx;
         step = step >= KT ? step - KT : step;
         const unsigned sbase = lds0 + (unsigned)(stage * kStageBytes);
 #pragma unroll
         for (int j = 0; j < AI; ++j) {
-            dma16(a_src[j] + (long long)step * kBK, sbase + a_dst[j]);
+            if (j % nparts == part) {
+                dma16(a_src[j] + (long long)step * kBK, sbase + a_dst[j]);
+            }
         }
         const int8_t *bp = t.wp + (long long)step * (kBLoads * kWave * 16);
 #pragma unroll
         for (int i = 0; i < kBLoads; ++i) {
-            dma16(bp + i * (kWave * 16), sbase + b_dst + (unsigned)(i * 1024));
+            if ((AI + i) % nparts == part) {
+                dma16(bp + i * (kWave * 16), sbase + b_dst + (unsigned)(i * 1024));
+            }
         }
     };
+    auto issue = [&](int s_idx, int stage) { issue_part(s_idx, stage, 0, 1); };
 
     const int a_row = lane & 31;
     const int a_half = lane >> 5;
@@ -166,7 +173,10 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs &a, const TileCtx &t, i
     constexpr int NH = MF / HF;                 // halves per sub-step
 
     // Multiplies one stage.  Fragment reads run one half sub-step ahead of the MFMAs that use them.
-    auto compute = [&](const int8_t *stage) {
+    // The loads of the step two ahead are issued from inside the phases, a few at a time between the
+    // MFMA groups: a wave that issued them all at once would sit at the memory pipe's input while it
+    // drains, with its MFMAs waiting behind the loads in program order.
+    auto compute = [&](const int8_t *stage, int next_idx, int next_stage) {
         const int8_t *sa = stage;
         const int8_t *sb = stage + kStageA + wave * (kWaveCols * kBK) + lane * 16;
         v4i af[2][HF];
@@ -195,6 +205,8 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs &a, const TileCtx &t, i
             // Keep the LDS reads of the next half ahead of this half's MFMAs: the scheduler would
             // otherwise sink them to just before their first use and expose the LDS latency.
             __builtin_amdgcn_sched_barrier(0);
+            issue_part(next_idx, next_stage, q, kKK * NH);
+            __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
             for (int f = 0; f < HF; ++f) {
 #pragma unroll
@@ -221,8 +233,7 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs &a, const TileCtx &t, i
     for (int kt = 0; kt < KT; ++kt) {
         wait_loads_outstanding<(kStages - 2) * PER_STEP>();
         barrier_no_fence();
-        issue(min(kt + kStages - 1, last), (kt + kStages - 1) % kStages);
-        compute(lds + (kt % kStages) * kStageBytes);
+        compute(lds + (kt % kStages) * kStageBytes, min(kt + kStages - 1, last), (kt + kStages - 1) % kStages);
     }
     wait_loads_outstanding<0>();
 
