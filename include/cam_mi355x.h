@@ -98,8 +98,10 @@ CAM_API const char *camGetVersion(void);
 /* ------------------------------------------------------------------------------------------------
  * DispatchLayout -- replaces aclnnDispatchLayout (AUTOGEN/aclnn_dispatch_layout.h:32-54).
  * topkIdx int64 [T,K] (int32 also accepted) -> numTokensPerRank int32 [R], numTokensPerExpert
- * int32 [E], isTokenInRank int32 [T,R] (bool/uint8 also accepted).  Ids < 0 are skipped; ids >= E are
- * ignored and counted nowhere.  Outputs need not be zeroed by the caller.
+ * int32 [E], isTokenInRank int32 [T,R] (bool/uint8 also accepted).  Ids < 0 are skipped
+ * (src/cam/comm_operator/pybind/moe_dispatch_prefill.cpp:106); ids >= E, which the reference kernel does not
+ * guard against (AK/dispatch_layout/op_kernel/dispatch_layout.h:113-118) and which would index past its
+ * count table, are skipped the same way and counted nowhere.  Outputs need not be zeroed by the caller.
  * Limits (AK/dispatch_layout/op_host/dispatch_layout_tiling.cc:43-50): 0 < R <= 384, 0 < K <= 16;
  * E <= 512 here (reference: 384). */
 CAM_API camStatus camDispatchLayoutGetWorkspaceSize(const camTensor *topkIdx, int64_t numTokens,
@@ -135,8 +137,12 @@ CAM_API camStatus camNotifyDispatch(void *workspace, uint64_t workspaceSize, cam
  *   sendTokenIdx int32 [T,K]   rank of (t,k) among earlier flat entries with the same id (-1 if id<0)
  *   numTokensPerExpert int32 [E], sendOffset int32 [E] (exclusive scan), recvOffset int32 [E],
  *   recvCount int32 [E] (inclusive cumsum in (local expert, source rank) order),
- *   numRecvTokensPerExpert int64 [E/R], totalRecvTokens int64 [1].  Any output except sendTokenIdx
- *   may be NULL.  numRanks must be 1. */
+ *   numRecvTokensPerExpert int64 [E/R], totalRecvTokens int64 [1],
+ *   slotRowOptional int32 [T,K]  output row of (t,k) = offset of its expert + its rank, -1 if the entry is
+ *                                skipped: the (token, k) -> row map MoeCombineGather consumes.
+ *   Any output except sendTokenIdx may be NULL.  numRanks must be 1.  Ids outside [0, E) are skipped:
+ *   negative ones are the reference's marker for a dropped entry (moe_dispatch_prefill.cpp:106); ids >= E,
+ *   which the reference does not guard against, would index past every per-expert table. */
 CAM_API camStatus camMoeDispatchPlanGetWorkspaceSize(const camTensor *topkIdx, int64_t numExperts,
                                                      int64_t numRanks, int64_t rankId,
                                                      const camTensor *sendTokenIdx,
@@ -145,13 +151,14 @@ CAM_API camStatus camMoeDispatchPlanGetWorkspaceSize(const camTensor *topkIdx, i
                                                      const camTensor *recvCount,
                                                      const camTensor *numRecvTokensPerExpert,
                                                      const camTensor *totalRecvTokens,
+                                                     const camTensor *slotRowOptional,
                                                      uint64_t *workspaceSize, camOpExecutor **executor);
 CAM_API camStatus camMoeDispatchPlan(void *workspace, uint64_t workspaceSize, camOpExecutor *executor,
                                      camStream_t stream);
 
 /* ------------------------------------------------------------------------------------------------
  * MoeDispatchNormal -- replaces aclnnMoeDispatchNormal (AUTOGEN/aclnn_moe_dispatch_normal.h:17-25).
- * x bf16 [T,H]; topkIdx int32 [T,K]; sendOffset, recvOffset, recvCount int32 [E]; sendTokenIdx
+ * x bf16 or fp16 [T,H]; topkIdx int32 [T,K]; sendOffset, recvOffset, recvCount int32 [E]; sendTokenIdx
  * int32 [T,K] -> recvX [A,H] (int8 when quantMode == 2, else x's dtype), recvXScales fp32 [A],
  * assistInfoForCombine int32 [3A] = (srcRank, token, k) per row.
  * Row of (t,k) with e = topkIdx[t,k] >= 0 (AK/moe_dispatch_normal/op_kernel/moe_dispatch_normal.h:
@@ -173,11 +180,36 @@ CAM_API camStatus camMoeDispatchNormal(void *workspace, uint64_t workspaceSize, 
                                        camStream_t stream);
 
 /* ------------------------------------------------------------------------------------------------
+ * MoeDispatchPrefill -- the whole body of the reference's binding-level operator moe_dispatch_prefill
+ * (src/cam/comm_operator/pybind/moe_dispatch_prefill.cpp:96-192: the CPU ranking loop, the CPU loop over the
+ * exchanged counts, two device-to-host copies and the aclnnMoeDispatchNormal call) as ONE kernel launch for
+ * one rank: MoeDispatchPlan and MoeDispatchNormal fused, with the plan running underneath the first row
+ * loads.  x bf16/fp16 [T,H]; topkIdx int64/int32 [T,K] -> recvX [A,H] (int8 when quantMode is 2 or 3, else
+ * x's dtype), recvXScalesOptional fp32 [A] (required when quantising), expandIdx int32 [3A] = (srcRank,
+ * token, k) per row, sendTokenIdx int32 [T,K]; optional slotRow int32 [T,K], numTokensPerExpert int32 [E],
+ * sendOffset int32 [E], recvCount int32 [E], numRecvTokensPerExpert int64 [E], totalRecvTokens int64 [1],
+ * all exactly as MoeDispatchPlan / MoeDispatchNormal produce them.  Rows outside [0,A) are dropped, so A
+ * may be a worst-case bound (T*K) and the true total read later from totalRecvTokens.
+ * The workspace may hold anything on first use; a launch leaves it ready for the next one.  Launches
+ * that share a workspace must not overlap.  Up to 524288 (token, k) entries take the single launch; above
+ * that the operator falls back to the two launches of MoeDispatchPlan + MoeDispatchNormal. */
+CAM_API camStatus camMoeDispatchPrefillGetWorkspaceSize(
+    const camTensor *x, const camTensor *topkIdx, int64_t numExperts, int64_t numRanks, int64_t rankId,
+    int64_t quantMode, const camTensor *recvX, const camTensor *recvXScalesOptional, const camTensor *expandIdx,
+    const camTensor *sendTokenIdx, const camTensor *slotRowOptional, const camTensor *numTokensPerExpertOptional,
+    const camTensor *sendOffsetOptional, const camTensor *recvCountOptional,
+    const camTensor *numRecvTokensPerExpertOptional, const camTensor *totalRecvTokensOptional,
+    uint64_t *workspaceSize, camOpExecutor **executor);
+CAM_API camStatus camMoeDispatchPrefill(void *workspace, uint64_t workspaceSize, camOpExecutor *executor,
+                                        camStream_t stream);
+
+/* ------------------------------------------------------------------------------------------------
  * MoeCombineNormal -- replaces aclnnMoeCombineNormal (AUTOGEN/aclnn_moe_combine_normal.h:37-65).
  * recvX bf16 [A,H]; tokenSrcInfo int32 [3A]; epRecvCounts int32 [E]; recvTopkWeights fp32 [T,K]
  * -> out bf16 [T,H].  out[t] = bf16(sum over k ascending of float(recvX[row(t,k)]) * w[t,k]), multiply
  * and add rounded separately (AK/moe_combine_normal/op_kernel/moe_combine_normal.h:303-338); row(t,k) is
- * the row whose triple names (t,k) (:232-238).  Slots no row names contribute nothing.
+ * the row whose triple names (t,k) (:232-238).  Slots no row names contribute nothing.  Only the first
+ * epRecvCounts[E-1] rows are looked at (:206-207): rows past the receive total were never written.
  * Workspace: T*K int32 (the inverse map). */
 CAM_API camStatus camMoeCombineNormalGetWorkspaceSize(
     const camTensor *recvX, const camTensor *tokenSrcInfo, const camTensor *epRecvCounts,
@@ -190,22 +222,25 @@ CAM_API camStatus camMoeCombineNormal(void *workspace, uint64_t workspaceSize, c
 
 /* ------------------------------------------------------------------------------------------------
  * MoeCombineIndex / MoeCombineGather -- the two halves of MoeCombineNormal as operators of their own, for
- * callers that combine more than one tensor with the same routing and want to build the (token, k) -> row
- * map once.  No counterpart in the reference, which scatters rows instead of gathering them
- * (AK/moe_combine_normal/op_kernel/moe_combine_normal.h:210-275).
+ * callers that already hold the (token, k) -> row map (slotRow of MoeDispatchPlan / MoeDispatchPrefill) or
+ * that combine more than one tensor with the same routing.  No counterpart in the reference, which scatters
+ * rows instead of gathering them (AK/moe_combine_normal/op_kernel/moe_combine_normal.h:210-275).
  * MoeCombineIndex:  tokenSrcInfo int32 [3A] -> slotRow int32 [T,K] (entries no row names are left untouched).
- * MoeCombineGather: recvX bf16 [A,H], tokenSrcInfo int32 [3A], slotRow int32 [T,K], recvTopkWeights fp32
- * [T,K] -> out bf16 [T,H]; a slotRow entry counts only if the triple of the row it names points back at
- * that slot, so slotRow needs no initialisation.  Same arithmetic and limits as MoeCombineNormal. */
+ * MoeCombineGather: recvX bf16 [A,H], slotRow int32 [T,K], recvTopkWeights fp32 [T,K] -> out bf16 [T,H].
+ *   tokenSrcInfoOptional int32 [3A]: when given, a slotRow entry counts only if the triple of the row it
+ *   names points back at that slot, so a slotRow built by MoeCombineIndex needs no initialisation; when NULL,
+ *   slotRow is trusted (entries < 0 are skipped), which is what the dispatch operators' slotRow output is for.
+ *   epRecvCountsOptional int32 [E]: when given, rows at or past its last element are never read.
+ *   Same arithmetic and limits as MoeCombineNormal. */
 CAM_API camStatus camMoeCombineIndexGetWorkspaceSize(const camTensor *tokenSrcInfo, int64_t numRows,
                                                      const camTensor *slotRow, uint64_t *workspaceSize,
                                                      camOpExecutor **executor);
 CAM_API camStatus camMoeCombineIndex(void *workspace, uint64_t workspaceSize, camOpExecutor *executor,
                                      camStream_t stream);
-CAM_API camStatus camMoeCombineGatherGetWorkspaceSize(const camTensor *recvX, const camTensor *tokenSrcInfo,
-                                                      const camTensor *slotRow, const camTensor *recvTopkWeights,
-                                                      const camTensor *out, uint64_t *workspaceSize,
-                                                      camOpExecutor **executor);
+CAM_API camStatus camMoeCombineGatherGetWorkspaceSize(const camTensor *recvX, const camTensor *tokenSrcInfoOptional,
+                                                      const camTensor *slotRow, const camTensor *epRecvCountsOptional,
+                                                      const camTensor *recvTopkWeights, const camTensor *out,
+                                                      uint64_t *workspaceSize, camOpExecutor **executor);
 CAM_API camStatus camMoeCombineGather(void *workspace, uint64_t workspaceSize, camOpExecutor *executor,
                                       camStream_t stream);
 

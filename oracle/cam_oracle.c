@@ -57,6 +57,37 @@ static inline uint16_t f32_to_bf16(float f)
     return (uint16_t)(u >> 16);
 }
 
+/* IEEE binary16 -> binary32, exact (the reference's dispatch accepts fp16 activations as well as bf16:
+ * AK/moe_dispatch_normal/op_host/moe_dispatch_normal.cpp:17-22; its Cast to float is exact either way). */
+static inline float fp16_to_f32(uint16_t v)
+{
+    uint32_t sign = (uint32_t)(v & 0x8000u) << 16;
+    uint32_t exp = (v >> 10) & 0x1fu;
+    uint32_t man = v & 0x3ffu;
+    uint32_t u;
+    if (exp == 0) {
+        if (man == 0) {
+            u = sign;
+        } else { /* subnormal: value = man * 2^-24 */
+            float f = (float)man * 5.9604644775390625e-8f;
+            memcpy(&u, &f, 4);
+            u |= sign;
+        }
+    } else if (exp == 31) {
+        u = sign | 0x7f800000u | (man << 13);
+    } else {
+        u = sign | ((exp + 112u) << 23) | (man << 13);
+    }
+    float f;
+    memcpy(&f, &u, 4);
+    return f;
+}
+
+/* act: 0 = bf16 bits, 1 = fp16 bits */
+static inline float act_to_f32(uint16_t v, int act) { return act ? fp16_to_f32(v) : bf16_to_f32(v); }
+
+ORACLE_API float cam_oracle_fp16_to_f32(uint16_t v) { return fp16_to_f32(v); }
+
 ORACLE_API int cam_oracle_num_threads(void)
 {
 #ifdef _OPENMP
@@ -73,9 +104,11 @@ ORACLE_API uint16_t cam_oracle_f32_to_bf16(float x) { return f32_to_bf16(x); }
 /* ---------------------------------------------------------------- A.1 layout
  * AK/dispatch_layout/op_kernel/dispatch_layout.h:83-134 (counts, rank = e / (E/R), first-seen flag
  * per token and rank); negative ids are skipped as in PB/moe_dispatch_prefill.cpp:106.
- * Returns -1 if an id >= E is met. */
+ * The reference kernel indexes its count table with the id unguarded (dispatch_layout.h:113-118), so an
+ * id >= E has no defined result there.  skip_out_of_range == 0: such an id is an error (returns -1);
+ * != 0: it is skipped like a negative one, which is what the HIP kernels are specified to do. */
 ORACLE_API int cam_oracle_layout(const int64_t *idx, int64_t T, int64_t K, int64_t E, int64_t R,
-                                 int32_t *cnt, int32_t *per_rank, uint8_t *in_rank)
+                                 int skip_out_of_range, int32_t *cnt, int32_t *per_rank, uint8_t *in_rank)
 {
     int64_t epr = E / R;
     memset(cnt, 0, sizeof(int32_t) * (size_t)E);
@@ -88,6 +121,9 @@ ORACLE_API int cam_oracle_layout(const int64_t *idx, int64_t T, int64_t K, int64
                 continue;
             }
             if (e >= E) {
+                if (skip_out_of_range) {
+                    continue;
+                }
                 return -1;
             }
             cnt[e] += 1;
@@ -178,11 +214,11 @@ ORACLE_API int64_t cam_oracle_recv_bookkeeping(const int32_t *recv_data, int64_t
  *     s = 127.0f / (max|x| + 1e-12f); q = int8(rint(x * s)); scale_out = 1.0f / s
  * variant 2 ("Q2"): FDM/gemm/kernel/…swiglu_quant_multistage_workspace.h:780-818
  *     s = 127.0f / max|x| (no epsilon); an all-zero row is defined as q = 0, scale_out = 0. */
-static void quant_token(const uint16_t *x, int64_t H, int variant, int8_t *q, float *scale_out)
+static void quant_token(const uint16_t *x, int64_t H, int variant, int act, int8_t *q, float *scale_out)
 {
     float m = 0.0f;
     for (int64_t h = 0; h < H; ++h) {
-        float a = fabsf(bf16_to_f32(x[h]));
+        float a = fabsf(act_to_f32(x[h], act));
         if (a > m) {
             m = a;
         }
@@ -199,18 +235,19 @@ static void quant_token(const uint16_t *x, int64_t H, int variant, int8_t *q, fl
         s = 127.0f / m;
     }
     for (int64_t h = 0; h < H; ++h) {
-        float v = bf16_to_f32(x[h]) * s;
+        float v = act_to_f32(x[h], act) * s;
         q[h] = (int8_t)(int32_t)nearbyintf(v);
     }
     *scale_out = 1.0f / s;
 }
 
+/* variant: 1 / 2 as above, + 16 when x holds fp16 bits instead of bf16 bits. */
 ORACLE_API void cam_oracle_quant_rows(const uint16_t *x, int64_t rows, int64_t H, int variant,
                                       int8_t *q, float *scales)
 {
 #pragma omp parallel for schedule(static)
     for (int64_t r = 0; r < rows; ++r) {
-        quant_token(x + r * H, H, variant, q + r * H, scales + r);
+        quant_token(x + r * H, H, variant & 15, variant >> 4, q + r * H, scales + r);
     }
 }
 
@@ -218,7 +255,7 @@ ORACLE_API void cam_oracle_quant_rows(const uint16_t *x, int64_t rows, int64_t H
  * moe_dispatch_normal.h:330-396 (send side: row = send_offset[e] + send_token_idx, source row
  * tokenIndex / K, triple (srcRank, token, k) :318-328) and :486-535 (receive side: rows land at
  * recv_count[i-1] + j).  With one rank the window row equals the output row.
- * quant: 0 = copy bf16 rows, 1 = Q1, 2 = Q2.  out is bf16 [A,H] or int8 [A,H]. */
+ * quant: 0 = copy the 16-bit rows, 1 = Q1, 2 = Q2 (+ 16: x holds fp16 bits).  out is 16-bit [A,H] or int8 [A,H]. */
 ORACLE_API void cam_oracle_dispatch(const uint16_t *x, const int64_t *idx, const int32_t *off,
                                     const int32_t *pos, int64_t T, int64_t K, int64_t H, int64_t E,
                                     int quant, int32_t src_rank, void *out, float *scales,
@@ -232,10 +269,10 @@ ORACLE_API void cam_oracle_dispatch(const uint16_t *x, const int64_t *idx, const
         }
         int64_t t = i / K;
         int64_t row = (int64_t)off[e] + pos[i];
-        if (quant == 0) {
+        if ((quant & 15) == 0) {
             memcpy((uint16_t *)out + row * H, x + t * H, (size_t)H * 2);
         } else {
-            quant_token(x + t * H, H, quant, (int8_t *)out + row * H, scales + row);
+            quant_token(x + t * H, H, quant & 15, quant >> 4, (int8_t *)out + row * H, scales + row);
         }
         if (src_info) {
             src_info[3 * row + 0] = src_rank;
@@ -427,7 +464,7 @@ ORACLE_API int cam_oracle_fused_layer(const uint16_t *x, const int64_t *idx, con
     int32_t *off = (int32_t *)calloc((size_t)E, 4);
     int32_t per_rank = 0;
     uint8_t *in_rank = (uint8_t *)calloc((size_t)(Ta > 0 ? Ta : 1), 1);
-    if (cam_oracle_layout(idx, Ta, K, E, 1, cnt, &per_rank, in_rank) != 0) {
+    if (cam_oracle_layout(idx, Ta, K, E, 1, 0, cnt, &per_rank, in_rank) != 0) {
         free(cnt);
         free(off);
         free(in_rank);

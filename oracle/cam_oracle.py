@@ -76,14 +76,15 @@ def bf16_bits_to_f32(a):
     return (np.ascontiguousarray(a, dtype=np.uint16).astype(np.uint32) << 16).view(np.float32)
 
 
-def layout(idx, E, R):
+def layout(idx, E, R, skip_out_of_range=False):
+    """Counts per expert / per rank and the token-in-rank flags.  Ids >= E raise unless skip_out_of_range."""
     idx = _c(idx, np.int64)
     T, K = idx.shape
     cnt = np.empty(E, np.int32)
     per_rank = np.empty(R, np.int32)
     in_rank = np.empty((T, R), np.uint8)
-    rc = lib().cam_oracle_layout(_p(idx), _i64(T), _i64(K), _i64(E), _i64(R), _p(cnt), _p(per_rank),
-                                 _p(in_rank))
+    rc = lib().cam_oracle_layout(_p(idx), _i64(T), _i64(K), _i64(E), _i64(R),
+                                 ctypes.c_int(1 if skip_out_of_range else 0), _p(cnt), _p(per_rank), _p(in_rank))
     if rc != 0:
         raise ValueError("expert id out of range")
     return per_rank, cnt, in_rank.astype(bool)
@@ -117,7 +118,18 @@ def recv_bookkeeping(recv_data, R, epr):
     return int(total), rc, ro, tpe, int(mx.value)
 
 
-def quant_rows(x_bits, variant):
+def fp16_bits_to_f32(a):
+    """IEEE fp16 bit patterns -> float32 through the C code's own conversion (one call per element)."""
+    a = np.ascontiguousarray(a, dtype=np.uint16)
+    f = lib().cam_oracle_fp16_to_f32
+    f.restype = ctypes.c_float
+    f.argtypes = [ctypes.c_uint16]
+    return np.array([f(int(v)) for v in a.reshape(-1)], np.float32).reshape(a.shape)
+
+
+def quant_rows(x_bits, variant, fp16=False):
+    """variant 1: with epsilon (dispatch), 2: without (fused kernel).  fp16: x_bits are fp16, not bf16, patterns."""
+    variant = int(variant) + (16 if fp16 else 0)
     x_bits = _c(x_bits, np.uint16)
     rows, H = x_bits.shape
     q = np.empty((rows, H), np.int8)
@@ -126,7 +138,8 @@ def quant_rows(x_bits, variant):
     return q, s
 
 
-def dispatch(x_bits, idx, off, pos, E, quant, total_rows, src_rank=0):
+def dispatch(x_bits, idx, off, pos, E, quant, total_rows, src_rank=0, fp16=False):
+    quant = int(quant) + (16 if (fp16 and quant) else 0)
     x_bits = _c(x_bits, np.uint16)
     idx = _c(idx, np.int64)
     off = _c(off, np.int32)
@@ -134,7 +147,7 @@ def dispatch(x_bits, idx, off, pos, E, quant, total_rows, src_rank=0):
     T, H = x_bits.shape
     K = idx.shape[1]
     A = max(int(total_rows), 1)
-    out = np.zeros((A, H), np.uint16 if quant == 0 else np.int8)
+    out = np.zeros((A, H), np.uint16 if (quant & 15) == 0 else np.int8)
     scales = np.zeros(A, np.float32)
     src = np.zeros(3 * A, np.int32)
     lib().cam_oracle_dispatch(_p(x_bits), _p(idx), _p(off), _p(pos), _i64(T), _i64(K), _i64(H), _i64(E),

@@ -16,9 +16,9 @@ def to_np(t):
     return t.cpu().numpy()
 
 
-def plan_oracle(oracle, idx_np, E):
+def plan_oracle(oracle, idx_np, E, skip_out_of_range=False):
     T = idx_np.shape[0]
-    _, cnt, _ = oracle.layout(np.where(idx_np >= E, -1, idx_np), E, 1)
+    _, cnt, _ = oracle.layout(idx_np, E, 1, skip_out_of_range=skip_out_of_range)
     off, trip = oracle.offsets(cnt, T)
     pos = oracle.send_token_idx(idx_np, E)
     return cnt, off, pos, trip

@@ -22,7 +22,7 @@ def _header_symbols():
 
 def test_library_exports_every_declared_symbol():
     names = _header_symbols()
-    assert len(names) == 27, names
+    assert len(names) == len(_lib.EXPORTS) >= 29, names
     handle = ctypes.CDLL(_lib.LIB_PATH)
     for n in names:
         assert hasattr(handle, n), n
@@ -116,6 +116,53 @@ def test_moe_combine_normal_validation():
     a = _combine_args()
     a[0] = _t((8, 1024), torch.float32)
     assert _lib.phase1("MoeCombineNormal", a)[0] == CAM_ERR_DTYPE
+
+
+def _prefill_args(T=4, K=2, E=8, H=1024, quant=0, R=1, x_dtype=torch.bfloat16, idx_dtype=torch.int64):
+    A = T * K
+    i32 = torch.int32
+    return [_t((T, H), x_dtype), _t((T, K), idx_dtype), E, R, 0, quant,
+            _t((A, H), torch.int8 if quant else x_dtype), _t((A,), torch.float32), _t((3 * A,), i32), _t((T, K), i32),
+            _t((T, K), i32), _t((E,), i32), _t((E,), i32), _t((E,), i32), _t((E,), torch.int64), _t((1,), torch.int64)]
+
+
+def test_moe_dispatch_prefill_validation():
+    st, ws, _ = _lib.phase1("MoeDispatchPrefill", _prefill_args())
+    assert st == CAM_OK and ws > 0
+    assert _lib.phase1("MoeDispatchPrefill", _prefill_args(quant=2, x_dtype=torch.float16))[0] == CAM_OK
+    assert _lib.phase1("MoeDispatchPrefill", _prefill_args(idx_dtype=torch.int32, quant=3))[0] == CAM_OK
+    assert _lib.phase1("MoeDispatchPrefill", _prefill_args(quant=1))[0] == CAM_ERR_UNSUPPORTED
+    assert _lib.phase1("MoeDispatchPrefill", _prefill_args(quant=5))[0] == CAM_ERR_RANGE
+    assert _lib.phase1("MoeDispatchPrefill", _prefill_args(R=2))[0] == CAM_ERR_UNSUPPORTED
+    assert _lib.phase1("MoeDispatchPrefill", _prefill_args(H=512))[0] == CAM_ERR_RANGE
+    assert _lib.phase1("MoeDispatchPrefill", _prefill_args(K=17, E=32))[0] == CAM_ERR_RANGE
+    a = _prefill_args(quant=2)
+    a[7] = None  # scales are required when quantising
+    assert _lib.phase1("MoeDispatchPrefill", a)[0] == CAM_ERR_NULL
+    a = _prefill_args()
+    a[9] = _t((4, 3), torch.int32)
+    assert _lib.phase1("MoeDispatchPrefill", a)[0] == CAM_ERR_SHAPE
+    a = _prefill_args()
+    for i in (10, 11, 12, 13, 14, 15):  # every optional output may be absent
+        a[i] = None
+    assert _lib.phase1("MoeDispatchPrefill", a)[0] == CAM_OK
+    # more (token, k) entries than the single launch is built for still validates (two-launch fallback)
+    assert _lib.phase1("MoeDispatchPrefill", _prefill_args(T=40000, K=16, E=32))[0] == CAM_OK
+
+
+def test_combine_gather_validation():
+    T, K, H, A, E = 4, 2, 1024, 8, 8
+    ok = [_t((A, H), torch.bfloat16), None, _t((T, K), torch.int32), None, _t((T, K), torch.float32),
+          _t((T, H), torch.bfloat16)]
+    assert _lib.phase1("MoeCombineGather", ok)[0] == CAM_OK
+    a = list(ok)
+    a[1], a[3] = _t((3 * A,), torch.int32), _t((E,), torch.int32)
+    assert _lib.phase1("MoeCombineGather", a)[0] == CAM_OK
+    a[1] = _t((3 * A - 1,), torch.int32)
+    assert _lib.phase1("MoeCombineGather", a)[0] == CAM_ERR_SHAPE
+    a = list(ok)
+    a[2] = _t((T, K + 1), torch.int32)
+    assert _lib.phase1("MoeCombineGather", a)[0] == CAM_ERR_SHAPE
 
 
 def _packed(shape):

@@ -86,3 +86,67 @@ def test_combine_index_then_gather_equals_normal(gpu, oracle):
         got = cam.moe_combine_gather(y, src_d, slot, w.to(gpu))
         want = cam.moe_combine_normal(y, src_d, recv_count, w.to(gpu))
         assert torch.equal(got, want)
+        # the map the dispatch operators hand out, trusted as it stands (no triples)
+        plan = cam.moe_dispatch_plan(ids.to(gpu), E)
+        got2 = cam.moe_combine_gather(y, None, plan["slot_row"], w.to(gpu), ep_recv_counts=recv_count)
+        assert torch.equal(got2, want)
+
+
+def test_combine_ignores_rows_past_the_receive_total(gpu, oracle):
+    """Buffers sized for a worst case: rows at or past epRecvCounts[E-1] hold triples of an earlier routing that
+    name valid slots; they must not be read (moe_combine_normal.h:206-207 stops at the receive total)."""
+    announce("combine with a stale tail")
+    T, K, E, H = 64, 4, 16, 1024
+    ids, w = synth.sigmoid_zipf_routing(T, E, K, seed=71)
+    ids[::3, 1] = -1  # fewer than T*K rows this time
+    idx_np = ids.numpy()
+    cnt, off, pos, _ = plan_oracle(oracle, idx_np, E)
+    total = int(cnt.sum())
+    A = T * K
+    assert total < A
+    y = synth.normal_bf16(A, H, seed=72)
+    _, _, src_now = oracle.dispatch(np.zeros((T, 8), np.uint16), idx_np, off, pos, E, 0, A)
+    src = src_now.copy().reshape(-1, 3)
+    # the tail keeps triples from an earlier, full routing: they name slots that exist now as well
+    tail = np.arange(total, A)
+    src[tail, 0] = 0
+    src[tail, 1] = tail % T
+    src[tail, 2] = (tail // T) % K
+    src = src.reshape(-1)
+    row_of = oracle.rows_from_src_info(src_now, total, T, K)
+    want = oracle.combine(synth.bf16_bits(y), row_of, w.numpy())
+    recv_count = torch.from_numpy((off + cnt).astype(np.int32)).to(gpu)
+    ws = torch.full((T * K * 4 + 256,), 0xFF, dtype=torch.uint8, device=gpu)
+    from umdk_original_amd import _lib
+    for _ in range(2):
+        out = torch.empty((T, H), dtype=torch.bfloat16, device=gpu)
+        _lib.call("MoeCombineNormal", [y.to(gpu), torch.from_numpy(src).to(gpu), recv_count, w.to(gpu), None, "", 1, 0,
+                                       "", 1, 0, E, 0, out], workspace=ws)
+        assert_bits_equal(to_np(out), want, "combined x")
+        # poison the inverse map with the stale rows, as a racing stale triple would have left it
+        ws[:T * K * 4].view(torch.int32).copy_(torch.from_numpy(
+            oracle.rows_from_src_info(src, A, T, K).reshape(-1)).to(gpu))
+
+
+def test_prefill_with_worst_case_rows_then_combine(gpu, oracle):
+    """moe_dispatch_prefill with num_worst_tokens > 0 leaves the tail of expand_x / expand_idx unwritten;
+    moe_combine_prefill must still return the right tokens."""
+    announce("prefill worst-case sizing + combine")
+    T, K, E, H = 48, 4, 8, 1024
+    ids, w = synth.softmax_topk_routing(T, E, K, seed=81)
+    ids[::4, 0] = -1
+    x = synth.normal_bf16(T, H, seed=82).to(gpu)
+    per_rank, per_expert, in_rank = cam.get_dispatch_layout(ids.to(gpu), E, 1)
+    # first a full routing into the same allocator blocks, so that the tail holds plausible triples
+    full_ids, _ = synth.softmax_topk_routing(T, E, K, seed=83)
+    first = cam.moe_dispatch_prefill(x, full_ids.to(gpu), w.to(gpu), per_rank, in_rank, per_expert, T * K, "g", 0, 1)
+    del first
+    ex, eidx, recv_count, _ = cam.moe_dispatch_prefill(x, ids.to(gpu), w.to(gpu), per_rank, in_rank, per_expert,
+                                                       T * K, "g", 0, 1)
+    assert ex.shape[0] == T * K
+    comb = cam.moe_combine_prefill(ex, ids.to(gpu), w.to(gpu), eidx, recv_count, "g", 0, 1)
+    cnt, off, pos, _ = plan_oracle(oracle, ids.numpy(), E)
+    total = int(cnt.sum())
+    want_x, _, want_src = oracle.dispatch(synth.bf16_bits(x.cpu()), ids.numpy(), off, pos, E, 0, total)
+    want = oracle.combine(want_x, oracle.rows_from_src_info(want_src, total, T, K), w.numpy())
+    assert_bits_equal(to_np(comb), want, "combined x")

@@ -170,3 +170,131 @@ def test_moe_dispatch_prefill_surface(gpu, oracle):
     # and back: combine of the un-quantised rows with weights summing to one returns x (K copies averaged)
     comb = torch.ops.umdk_cam_op_lib.moe_combine_prefill(ex, ids.to(gpu), w.to(gpu), eidx, recv_count, "group", 0, 1)
     assert (comb.float() - x.float()).abs().max().item() <= 0.04
+
+
+def test_ids_at_or_above_E_are_skipped(gpu, oracle):
+    """Ids >= E (which the reference kernel does not guard against) behave like negative ids everywhere."""
+    announce("ids >= E")
+    T, K, E, H = 90, 4, 16, 1024
+    g = torch.Generator().manual_seed(31)
+    ids = torch.randint(-2, E + 5, (T, K), generator=g, dtype=torch.int64)  # -2..20 with E = 16
+    idx_np = ids.numpy()
+    assert (idx_np >= E).sum() > 20 and (idx_np < 0).sum() > 10
+    per_rank, per_expert, in_rank = cam.get_dispatch_layout(ids.to(gpu), E, 4)
+    want_rank, want_cnt, want_in = oracle.layout(idx_np, E, 4, skip_out_of_range=True)
+    assert_bits_equal(to_np(per_expert), want_cnt, "num_tokens_per_expert")
+    assert_bits_equal(to_np(per_rank), want_rank, "num_tokens_per_rank")
+    assert_bits_equal(to_np(in_rank), want_in, "is_token_in_rank")
+    cnt, off, pos, _ = plan_oracle(oracle, idx_np, E, skip_out_of_range=True)
+    plan = cam.moe_dispatch_plan(ids.to(gpu), E)
+    assert_bits_equal(to_np(plan["send_token_idx"]), pos, "send_token_idx")
+    assert_bits_equal(to_np(plan["num_tokens_per_expert"]), cnt, "num_tokens_per_expert")
+    assert_bits_equal(to_np(plan["slot_row"]), oracle.rows_from_pos(idx_np, off, pos, E), "slot_row")
+    total = int(cnt.sum())
+    assert int(plan["total"].item()) == total == int(((idx_np >= 0) & (idx_np < E)).sum())
+    x = synth.normal_bf16(T, H, seed=32)
+    recv_x, scales, assist = cam.moe_dispatch_normal(
+        x.to(gpu), ids.to(gpu), plan["send_offset"], plan["send_token_idx"], plan["recv_offset"], plan["recv_count"],
+        total, E, quant_mode=2)
+    want_x, want_s, want_src = oracle.dispatch(synth.bf16_bits(x), idx_np, off, pos, E, 1, total)
+    assert_bits_equal(to_np(recv_x), want_x, "recv_x")
+    assert_bits_equal(to_np(assist), want_src, "assist_info")
+    assert_bits_equal(to_np(scales).view(np.uint32), want_s.view(np.uint32), "scales")
+
+
+def _check_fused(oracle, d, x, idx_np, E, quant_mode, fp16=False):
+    cnt, off, pos, _ = plan_oracle(oracle, idx_np, E, skip_out_of_range=True)
+    total = int(cnt.sum())
+    variant = {0: 0, 2: 1, 3: 2}[quant_mode]
+    bits = x.view(torch.int16).numpy().view(np.uint16)
+    want_x, want_s, want_src = oracle.dispatch(bits, idx_np, off, pos, E, variant, total, fp16=fp16)
+    assert int(d["total"].item()) == total
+    assert_bits_equal(to_np(d["send_token_idx"]), pos, "send_token_idx")
+    assert_bits_equal(to_np(d["slot_row"]), oracle.rows_from_pos(idx_np, off, pos, E), "slot_row")
+    assert_bits_equal(to_np(d["num_tokens_per_expert"]), cnt, "num_tokens_per_expert")
+    assert_bits_equal(to_np(d["send_offset"]), off, "send_offset")
+    assert_bits_equal(to_np(d["recv_count"]), (off + cnt).astype(np.int32), "recv_count")
+    assert_bits_equal(to_np(d["num_recv_tokens_per_expert"]), cnt.astype(np.int64), "tokens per expert")
+    got_x = d["recv_x"].view(torch.int16) if quant_mode == 0 else d["recv_x"]
+    assert_bits_equal(got_x.cpu().numpy()[:total].view(want_x.dtype), want_x[:total], "recv_x")
+    assert_bits_equal(to_np(d["expand_idx"])[:3 * total], want_src[:3 * total], "expand_idx")
+    if quant_mode != 0:
+        assert_bits_equal(to_np(d["recv_x_scales"])[:total].view(np.uint32), want_s[:total].view(np.uint32), "scales")
+
+
+@pytest.mark.parametrize("quant_mode", [0, 2, 3])
+@pytest.mark.parametrize("T,K,E,H,dtype,neg", [
+    (1, 1, 2, 1024, torch.int64, 0.0),
+    (37, 3, 8, 1024, torch.int32, 0.2),
+    (300, 8, 256, 7168, torch.int64, 0.0),     # two chunks of 2048 ids
+    (1500, 16, 512, 1032, torch.int64, 0.05),  # twelve chunks, odd row length
+])
+def test_dispatch_prefill_single_launch(gpu, oracle, T, K, E, H, dtype, neg, quant_mode):
+    announce("fused dispatch T=%d K=%d E=%d H=%d quant=%d" % (T, K, E, H, quant_mode))
+    ids = _random_ids(T, K, E, seed=T + K + E, neg_frac=neg, dtype=dtype)
+    x = synth.normal_bf16(T, H, seed=T + 3)
+    if T > 4:
+        x[4] = 0
+    d = cam.moe_dispatch_fused(x.to(gpu), ids.to(gpu), E, quant_mode=quant_mode)
+    _check_fused(oracle, d, x, ids.numpy().astype(np.int64), E, quant_mode)
+
+
+def test_dispatch_prefill_workspace_reuse_and_garbage(gpu, oracle):
+    """The same workspace, first filled with arbitrary bytes, serves several launches with different routings."""
+    announce("fused dispatch workspace reuse")
+    from umdk_original_amd import _lib
+    T, K, E, H = 513, 8, 64, 2048
+    ws = torch.full((1 << 20,), 0xA5, dtype=torch.uint8, device=gpu)
+    for seed, fill in ((1, None), (2, None), (3, 0xFF), (4, None)):
+        if fill is not None:
+            ws.fill_(fill)
+        ids = _random_ids(T, K, E, seed=seed, neg_frac=0.1)
+        x = synth.normal_bf16(T, H, seed=seed + 10)
+        A = T * K
+        i32 = dict(dtype=torch.int32, device=gpu)
+        d = dict(recv_x=torch.empty((A, H), dtype=torch.int8, device=gpu),
+                 recv_x_scales=torch.empty(A, dtype=torch.float32, device=gpu), expand_idx=torch.empty(3 * A, **i32),
+                 send_token_idx=torch.empty((T, K), **i32), slot_row=torch.empty((T, K), **i32),
+                 num_tokens_per_expert=torch.empty(E, **i32), send_offset=torch.empty(E, **i32),
+                 recv_count=torch.empty(E, **i32),
+                 num_recv_tokens_per_expert=torch.empty(E, dtype=torch.int64, device=gpu),
+                 total=torch.empty(1, dtype=torch.int64, device=gpu))
+        _lib.call("MoeDispatchPrefill", [x.to(gpu), ids.to(gpu), E, 1, 0, 2, d["recv_x"], d["recv_x_scales"],
+                                         d["expand_idx"], d["send_token_idx"], d["slot_row"],
+                                         d["num_tokens_per_expert"], d["send_offset"], d["recv_count"],
+                                         d["num_recv_tokens_per_expert"], d["total"]], workspace=ws)
+        _check_fused(oracle, d, x, ids.numpy(), E, 2)
+
+
+def test_dispatch_prefill_full_size_config(gpu, oracle):
+    announce("fused dispatch C2 full size")
+    T, K, E, H = 4096, 8, 256, 7168
+    ids, _ = synth.sigmoid_zipf_routing(T, E, K, seed=44)
+    x = synth.normal_bf16(T, H, seed=44)
+    d = cam.moe_dispatch_fused(x.to(gpu), ids.to(gpu), E, quant_mode=2)
+    _check_fused(oracle, d, x, ids.numpy(), E, 2)
+    again = cam.moe_dispatch_fused(x.to(gpu), ids.to(gpu), E, quant_mode=2)
+    assert torch.equal(again["recv_x"], d["recv_x"]) and torch.equal(again["send_token_idx"], d["send_token_idx"])
+
+
+@pytest.mark.parametrize("quant_mode", [0, 2, 3])
+def test_dispatch_fp16_activations(gpu, oracle, quant_mode):
+    """fp16 activations (moe_dispatch_normal.cpp op_host :17-22 lists them beside bf16), both dispatch operators."""
+    announce("dispatch fp16 quant=%d" % quant_mode)
+    T, K, E, H = 70, 4, 16, 2048
+    ids = _random_ids(T, K, E, seed=61, neg_frac=0.1)
+    x = (torch.randn(T, H, generator=torch.Generator().manual_seed(62)) * 4).half()
+    x[9] = 0
+    x[10, :5] = torch.tensor([6e-8, -6e-5, 65504.0, -1e-3, 3e-7]).half()  # subnormals and the largest value
+    idx_np = ids.numpy()
+    d = cam.moe_dispatch_fused(x.to(gpu), ids.to(gpu), E, quant_mode=quant_mode)
+    _check_fused(oracle, d, x, idx_np, E, quant_mode, fp16=True)
+    plan = cam.moe_dispatch_plan(ids.to(gpu), E)
+    total = int(plan["total"].item())
+    recv_x, scales, assist = cam.moe_dispatch_normal(
+        x.to(gpu), ids.to(gpu), plan["send_offset"], plan["send_token_idx"], plan["recv_offset"], plan["recv_count"],
+        total, E, quant_mode=quant_mode)
+    assert torch.equal(recv_x[:total], d["recv_x"][:total])
+    assert torch.equal(assist[:3 * total], d["expand_idx"][:3 * total])
+    if quant_mode:
+        assert torch.equal(scales[:total], d["recv_x_scales"][:total])

@@ -127,3 +127,79 @@ def test_full_size_grouped_gemm_sampled_rows(gpu):
     c1 = cam.grouped_matmul_int32(a_small.to(gpu), wp, gl.to(gpu))
     c2 = cam.grouped_matmul_int32((a_small * 2).to(gpu), wp, gl.to(gpu))
     assert torch.equal(c2, c1 * 2)
+
+
+def _sample_rows(n):
+    """Rows of an expert with n rows: both ends, the middle, the neighbours of every multiple of 32 that is also a
+    multiple of 128 or 256 (tile edges of any tiling in those units), and a sparse stride through the rest."""
+    pick = {0, n - 1, n // 2}
+    for edge in range(0, n, 128):
+        pick.update({edge - 1, edge, edge + 1, edge + 31, edge + 32, edge + 33})
+    pick.update(range(5, n, 61))
+    return sorted(p for p in pick if 0 <= p < n)
+
+
+def test_full_size_epilogues_sampled_rows(gpu, oracle):
+    """Both GEMM operators with their epilogues at the benchmark shape (32 experts, 8192 Zipf rows, H 7168,
+    I 2048): y int8, y_scale and the bf16 output of sampled rows against the oracle run on exactly those rows
+    (rows are independent, so a group list over the sampled rows gives bit-identical expectations)."""
+    announce("gemm C3 full size, both epilogues, sampled rows")
+    G, H, I, rows = 32, 7168, 2048, 8192
+    sizes = synth.zipf_group_sizes(G, rows, seed=45)
+    gl = torch.cumsum(sizes, 0)
+    starts = (gl - sizes).tolist()
+    a = synth.uniform_int8((rows, H), 45)
+    a[starts[int(torch.argmax(sizes))] + 7] = 0  # an all-zero row inside the largest expert
+    xs = synth.channel_scales((rows,), 451, 0.005, 0.05)
+    g_cpu = torch.Generator().manual_seed(452)
+    w1 = torch.randint(-127, 128, (G, H, 2 * I), generator=g_cpu, dtype=torch.int8)
+    w2 = torch.randint(-127, 128, (G, I, H), generator=g_cpu, dtype=torch.int8)
+    w1s = synth.channel_scales((G, 2 * I), 453)
+    w2s = synth.channel_scales((G, H), 454)
+    w1p = cam.prepack_weight(w1.to(gpu), True)
+    w2p = cam.prepack_weight(w2.to(gpu), False)
+    y, ysc = cam.grouped_matmul_swiglu_quant(a.to(gpu), xs.to(gpu), w1p, w1s.to(gpu), gl.to(gpu))
+    out = cam.grouped_matmul_dequant(y, ysc, w2p, w2s.to(gpu), gl.to(gpu))
+    y_c, ysc_c, out_c = y.cpu(), ysc.cpu(), out.cpu()
+    checked = 0
+    for g in range(G):
+        n = int(sizes[g])
+        if n == 0:
+            continue
+        r = torch.tensor([starts[g] + p for p in _sample_rows(n)])
+        sub_gl = np.array([len(r)], np.int64)
+        # exact integer products through float64 (|sum| <= 7168 * 127 * 127 < 2^53)
+        c1 = (a[r].double() @ w1[g].double()).to(torch.int32).numpy()
+        d = oracle.gmm1_epilogue(c1, w1s[g:g + 1].numpy(), xs[r].numpy(), sub_gl)
+        want_q, want_s = oracle.swiglu_quant(d)
+        assert_bits_equal(to_np(ysc_c[r]).view(np.uint32), want_s.view(np.uint32), "y_scale, expert %d" % g)
+        assert_bits_equal(to_np(y_c[r]), want_q, "y int8, expert %d" % g)
+        c2 = (y_c[r].double() @ w2[g].double()).to(torch.int32).numpy()
+        want_o = oracle.gmm2_epilogue(c2, w2s[g:g + 1].numpy(), ysc_c[r].numpy(), sub_gl)
+        assert_bits_equal(to_np(out_c[r]), want_o, "bf16 output, expert %d" % g)
+        checked += len(r)
+    assert checked >= 400
+    zr = starts[int(torch.argmax(sizes))] + 7
+    assert (y_c[zr] == 0).all() and float(ysc_c[zr]) == 0.0 and (out_c[zr].float() == 0).all()
+
+
+def test_many_tiles_per_expert_epilogues(gpu, oracle):
+    """Experts of 5 and 9 row tiles of 128 (and a ragged one) through both epilogues, every row checked."""
+    announce("gemm epilogues, many tiles per expert")
+    sizes, H, I = [600, 0, 1100, 77], 512, 256
+    a, w, gl, A = _inputs(sizes, H, 2 * I, seed=99, wrange=16)
+    G = len(sizes)
+    ws = synth.channel_scales((G, 2 * I), seed=41)
+    xs = synth.channel_scales((A,), seed=42, lo=0.005, hi=0.05)
+    y, ysc = cam.grouped_matmul_swiglu_quant(a.to(gpu), xs.to(gpu), cam.prepack_weight(w.to(gpu), True), ws.to(gpu),
+                                             gl.to(gpu))
+    c = oracle.gmm_int32(a.numpy(), w.numpy(), gl.numpy())
+    want_q, want_s = oracle.swiglu_quant(oracle.gmm1_epilogue(c, ws.numpy(), xs.numpy(), gl.numpy()), rows=A)
+    assert_bits_equal(to_np(ysc).view(np.uint32), want_s.view(np.uint32), "y_scale")
+    assert_bits_equal(to_np(y), want_q, "y int8")
+    w2 = synth.uniform_int8((G, I, H), 98, -16, 16)
+    w2s = synth.channel_scales((G, H), seed=43)
+    out = cam.grouped_matmul_dequant(y, ysc, cam.prepack_weight(w2.to(gpu), False), w2s.to(gpu), gl.to(gpu))
+    c2 = oracle.gmm_int32(want_q, w2.numpy(), gl.numpy())
+    want = oracle.gmm2_epilogue(c2, w2s.numpy(), want_s, gl.numpy())
+    assert_bits_equal(to_np(out), want, "bf16 output")

@@ -48,6 +48,48 @@ def test_layout_rejects_out_of_range(oracle):
         oracle.layout(np.array([[0, 8]], np.int64), 8, 1)
 
 
+def test_layout_can_skip_out_of_range_ids(oracle):
+    """The skipping mode equals the strict mode run on the same ids with the out-of-range ones set to -1."""
+    rng = _rng(77)
+    idx = rng.integers(-2, 12, size=(50, 4)).astype(np.int64)  # E = 8: ids 8..11 are out of range
+    got = oracle.layout(idx, 8, 2, skip_out_of_range=True)
+    want = oracle.layout(np.where(idx >= 8, -1, idx), 8, 2)
+    for g, w in zip(got, want):
+        assert np.array_equal(g, w)
+    assert got[1].sum() == ((idx >= 0) & (idx < 8)).sum() == np.bincount(idx[(idx >= 0) & (idx < 8)], minlength=8).sum()
+    pos = oracle.send_token_idx(idx, 8)
+    assert ((pos == -1) == ((idx < 0) | (idx >= 8))).all()
+
+
+def test_fp16_conversion_matches_numpy_on_every_pattern(oracle):
+    bits = np.arange(65536, dtype=np.uint16)
+    got = oracle.fp16_bits_to_f32(bits)
+    want = bits.view(np.float16).astype(np.float32)
+    nan = np.isnan(want)
+    assert np.array_equal(np.isnan(got), nan)
+    assert np.array_equal(got[~nan].view(np.uint32), want[~nan].view(np.uint32))
+
+
+def test_fp16_quant_rows_follow_the_float32_definition(oracle):
+    """Same arithmetic as the bf16 rows, on exactly converted fp16 inputs."""
+    rng = _rng(5)
+    x = (rng.standard_normal((9, 256)) * 3).astype(np.float16)
+    x[3] = 0
+    for variant in (1, 2):
+        q, s = oracle.quant_rows(x.view(np.uint16), variant, fp16=True)
+        xf = x.astype(np.float32)
+        m = np.abs(xf).max(axis=1)
+        with np.errstate(divide="ignore", invalid="ignore"):
+            sc = np.float32(127.0) / (m + np.float32(1e-12)) if variant == 1 else np.float32(127.0) / m
+        want_q = np.rint(xf * sc[:, None].astype(np.float32)).astype(np.float32)
+        want_s = (np.float32(1.0) / sc).astype(np.float32)
+        if variant == 2:
+            want_q[3] = 0
+            want_s[3] = 0
+        assert np.array_equal(q.astype(np.float32), want_q)
+        assert np.array_equal(s.view(np.uint32), want_s.view(np.uint32))
+
+
 def test_offsets_are_exclusive_cumsum_with_triplets(oracle):
     cnt = _rng(1).integers(0, 50, size=37).astype(np.int32)
     off, trip = oracle.offsets(cnt, 99)

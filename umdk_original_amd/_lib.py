@@ -90,12 +90,13 @@ _PHASE1_TAIL = [ctypes.POINTER(ctypes.c_uint64), ctypes.POINTER(ctypes.c_void_p)
 SIGNATURES = {
     "DispatchLayout": [_TP, _I64, _I64, _I64, _I64, _TP, _TP, _TP],
     "NotifyDispatch": [_TP, _TP, _I64, _I64, _STR, _I64, _I64, _I64, _I64, _TP, _TP],
-    "MoeDispatchPlan": [_TP, _I64, _I64, _I64, _TP, _TP, _TP, _TP, _TP, _TP, _TP],
+    "MoeDispatchPlan": [_TP, _I64, _I64, _I64, _TP, _TP, _TP, _TP, _TP, _TP, _TP, _TP],
+    "MoeDispatchPrefill": [_TP, _TP, _I64, _I64, _I64, _I64, _TP, _TP, _TP, _TP, _TP, _TP, _TP, _TP, _TP, _TP],
     "MoeDispatchNormal": [_TP, _TP, _TP, _TP, _TP, _TP, _STR, _I64, _I64, _STR, _I64, _I64, _I64, _I64, _I64,
                           _TP, _TP, _TP],
     "MoeCombineNormal": [_TP, _TP, _TP, _TP, _TP, _STR, _I64, _I64, _STR, _I64, _I64, _I64, _I64, _TP],
     "MoeCombineIndex": [_TP, _I64, _TP],
-    "MoeCombineGather": [_TP, _TP, _TP, _TP, _TP],
+    "MoeCombineGather": [_TP, _TP, _TP, _TP, _TP, _TP],
     "PrepackWeight": [_TP, _I64, _TP],
     "GroupedMatmulSwigluQuant": [_TP, _TP, _LP, _LP, _TP, _I64, _TP, _TP],
     "GroupedMatmulDequant": [_TP, _TP, _LP, _LP, _TP, _I64, _TP],

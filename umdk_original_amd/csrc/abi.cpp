@@ -40,6 +40,7 @@ enum OpTag {
     kOpNotify = 0x4e4f5449,
     kOpPlan = 0x504c414e,
     kOpDispatch = 0x44495350,
+    kOpPrefill = 0x50524546,
     kOpCombine = 0x434f4d42,
     kOpCombIndex = 0x43494458,
     kOpCombGather = 0x43475448,
@@ -430,8 +431,8 @@ camStatus camMoeDispatchPlanGetWorkspaceSize(const camTensor *topkIdx, int64_t n
                                              const camTensor *numTokensPerExpert, const camTensor *sendOffset,
                                              const camTensor *recvOffset, const camTensor *recvCount,
                                              const camTensor *numRecvTokensPerExpert,
-                                             const camTensor *totalRecvTokens, uint64_t *workspaceSize,
-                                             camOpExecutor **executor)
+                                             const camTensor *totalRecvTokens, const camTensor *slotRowOptional,
+                                             uint64_t *workspaceSize, camOpExecutor **executor)
 {
     CAM_TRY(check_tensor(topkIdx, "topkIdx", 2, CAM_DT_INT64, CAM_DT_INT32));
     if (numExperts <= 0 || numExperts > cam::kMaxExperts) {
@@ -476,6 +477,12 @@ camStatus camMoeDispatchPlanGetWorkspaceSize(const camTensor *topkIdx, int64_t n
             return fail(CAM_ERR_SHAPE, "totalRecvTokens must hold one element");
         }
     }
+    if (slotRowOptional != nullptr) {
+        CAM_TRY(check_tensor(slotRowOptional, "slotRow", 2, CAM_DT_INT32));
+        if (slotRowOptional->sizes[0] != T || slotRowOptional->sizes[1] != K) {
+            return fail(CAM_ERR_SHAPE, "slotRow must be [T,K]");
+        }
+    }
     cam::PlanArgs p{};
     p.idx = topkIdx->data;
     p.idx_is64 = topkIdx->dtype == CAM_DT_INT64;
@@ -484,6 +491,7 @@ camStatus camMoeDispatchPlanGetWorkspaceSize(const camTensor *topkIdx, int64_t n
     p.E = (int)numExperts;
     p.R = 1;
     p.pos = (int32_t *)sendTokenIdx->data;
+    p.dst_row = slotRowOptional ? (int32_t *)slotRowOptional->data : nullptr;
     p.cnt = numTokensPerExpert ? (int32_t *)numTokensPerExpert->data : nullptr;
     p.off = sendOffset ? (int32_t *)sendOffset->data : nullptr;
     p.recv_off = recvOffset ? (int32_t *)recvOffset->data : nullptr;
@@ -575,9 +583,6 @@ camStatus camMoeDispatchNormalGetWorkspaceSize(const camTensor *x, const camTens
         return fail(CAM_ERR_SHAPE, "sendTokenIdx must be [T,K]");
     }
     const bool quant = quantMode != 0;
-    if (quant && x->dtype != CAM_DT_BF16) {
-        return fail(CAM_ERR_UNSUPPORTED, "quantised dispatch of float16 activations is not built");
-    }
     CAM_TRY(check_tensor(recvX, "recvX", 2, quant ? CAM_DT_INT8 : x->dtype));
     if (recvX->sizes[1] != H) {
         return fail(CAM_ERR_SHAPE, "recvX dimension 1 must equal the hidden size");
@@ -608,6 +613,7 @@ camStatus camMoeDispatchNormalGetWorkspaceSize(const camTensor *x, const camTens
     d.E = (int)moeExpertNum;
     d.A = A;
     d.quant = quantMode == 0 ? 0 : (quantMode == 2 ? 1 : 2);
+    d.x_is_fp16 = x->dtype == CAM_DT_FLOAT16;
     d.out = recvX->data;
     d.scales = quant ? (float *)recvXScales->data : nullptr;
     d.src_info = (int32_t *)assistInfoForCombine->data;
@@ -620,6 +626,178 @@ camStatus camMoeDispatchNormal(void *workspace, uint64_t workspaceSize, camOpExe
                                camStream_t stream)
 {
     return run_phase2(kOpDispatch, "camMoeDispatchNormal", workspace, workspaceSize, executor, stream);
+}
+
+// ------------------------------------------------------------------------------------------------
+camStatus camMoeDispatchPrefillGetWorkspaceSize(const camTensor *x, const camTensor *topkIdx, int64_t numExperts,
+                                                int64_t numRanks, int64_t rankId, int64_t quantMode,
+                                                const camTensor *recvX, const camTensor *recvXScalesOptional,
+                                                const camTensor *expandIdx, const camTensor *sendTokenIdx,
+                                                const camTensor *slotRowOptional,
+                                                const camTensor *numTokensPerExpertOptional,
+                                                const camTensor *sendOffsetOptional,
+                                                const camTensor *recvCountOptional,
+                                                const camTensor *numRecvTokensPerExpertOptional,
+                                                const camTensor *totalRecvTokensOptional, uint64_t *workspaceSize,
+                                                camOpExecutor **executor)
+{
+    CAM_TRY(check_tensor(x, "x", 2, CAM_DT_BF16, CAM_DT_FLOAT16));
+    CAM_TRY(check_tensor(topkIdx, "topkIdx", 2, CAM_DT_INT64, CAM_DT_INT32));
+    if (numExperts <= 0 || numExperts > cam::kMaxExperts) {
+        return fail(CAM_ERR_RANGE, "numExperts %lld outside (0, %d]", (long long)numExperts, cam::kMaxExperts);
+    }
+    if (numRanks <= 0 || rankId < 0 || rankId >= numRanks) {
+        return fail(CAM_ERR_RANGE, "rank %lld / numRanks %lld invalid", (long long)rankId, (long long)numRanks);
+    }
+    if (numRanks != 1) {
+        return fail(CAM_ERR_UNSUPPORTED, "MoeDispatchPrefill: numRanks must be 1 (single-GPU library)");
+    }
+    if (quantMode < 0 || quantMode > 3) {
+        return fail(CAM_ERR_RANGE, "quantMode %lld outside [0, 3]", (long long)quantMode);
+    }
+    if (quantMode == 1) {
+        return fail(CAM_ERR_UNSUPPORTED, "quantMode 1 (static quantisation) is not built");
+    }
+    const int64_t T = x->sizes[0], H = x->sizes[1], K = topkIdx->sizes[1];
+    if (T < 1) {
+        return fail(CAM_ERR_RANGE, "batch size must be at least 1");
+    }
+    if (H < 1024 || H > 7168) {
+        return fail(CAM_ERR_RANGE, "hidden size %lld outside [1024, 7168]", (long long)H);
+    }
+    if (H % 8 != 0) {
+        return fail(CAM_ERR_ALIGN, "hidden size %lld must be a multiple of 8", (long long)H);
+    }
+    if (topkIdx->sizes[0] != T) {
+        return fail(CAM_ERR_SHAPE, "x and topkIdx must agree on dimension 0");
+    }
+    if (K <= 0 || K > cam::kMaxTopk || K > numExperts) {
+        return fail(CAM_ERR_RANGE, "top-k %lld outside (0, min(%d, numExperts)]", (long long)K, cam::kMaxTopk);
+    }
+    if (T * K > 0x7fffffffll) {
+        return fail(CAM_ERR_RANGE, "tokens * top-k does not fit 32 bits");
+    }
+    const bool quant = quantMode != 0;
+    CAM_TRY(check_tensor(recvX, "recvX", 2, quant ? CAM_DT_INT8 : x->dtype));
+    if (recvX->sizes[1] != H) {
+        return fail(CAM_ERR_SHAPE, "recvX dimension 1 must equal the hidden size");
+    }
+    const int64_t A = recvX->sizes[0];
+    CAM_TRY(check_aligned(x, "x", 16));
+    CAM_TRY(check_aligned(recvX, "recvX", 16));
+    if (quant) {
+        CAM_TRY(check_tensor(recvXScalesOptional, "recvXScales", 1, CAM_DT_FLOAT));
+        if (recvXScalesOptional->sizes[0] < A) {
+            return fail(CAM_ERR_SHAPE, "recvXScales must hold one value per recvX row");
+        }
+    }
+    CAM_TRY(check_tensor(expandIdx, "expandIdx", 1, CAM_DT_INT32));
+    if (expandIdx->sizes[0] < 3 * A) {
+        return fail(CAM_ERR_SHAPE, "expandIdx must hold 3 values per recvX row");
+    }
+    CAM_TRY(check_tensor(sendTokenIdx, "sendTokenIdx", 2, CAM_DT_INT32));
+    if (sendTokenIdx->sizes[0] != T || sendTokenIdx->sizes[1] != K) {
+        return fail(CAM_ERR_SHAPE, "sendTokenIdx must be [T,K]");
+    }
+    if (slotRowOptional != nullptr) {
+        CAM_TRY(check_tensor(slotRowOptional, "slotRow", 2, CAM_DT_INT32));
+        if (slotRowOptional->sizes[0] != T || slotRowOptional->sizes[1] != K) {
+            return fail(CAM_ERR_SHAPE, "slotRow must be [T,K]");
+        }
+    }
+    const camTensor *opt_e[3] = {numTokensPerExpertOptional, sendOffsetOptional, recvCountOptional};
+    const char *opt_n[3] = {"numTokensPerExpert", "sendOffset", "recvCount"};
+    for (int i = 0; i < 3; ++i) {
+        if (opt_e[i] != nullptr) {
+            CAM_TRY(check_tensor(opt_e[i], opt_n[i], 1, CAM_DT_INT32));
+            if (opt_e[i]->sizes[0] != numExperts) {
+                return fail(CAM_ERR_SHAPE, "%s must hold numExperts elements", opt_n[i]);
+            }
+        }
+    }
+    if (numRecvTokensPerExpertOptional != nullptr) {
+        CAM_TRY(check_tensor(numRecvTokensPerExpertOptional, "numRecvTokensPerExpert", 1, CAM_DT_INT64));
+        if (numRecvTokensPerExpertOptional->sizes[0] != numExperts / numRanks) {
+            return fail(CAM_ERR_SHAPE, "numRecvTokensPerExpert must hold numExperts / numRanks elements");
+        }
+    }
+    if (totalRecvTokensOptional != nullptr) {
+        CAM_TRY(check_tensor(totalRecvTokensOptional, "totalRecvTokens", 1, CAM_DT_INT64));
+        if (totalRecvTokensOptional->sizes[0] < 1) {
+            return fail(CAM_ERR_SHAPE, "totalRecvTokens must hold one element");
+        }
+    }
+    cam::FusedDispatchArgs f{};
+    f.p.idx = topkIdx->data;
+    f.p.idx_is64 = topkIdx->dtype == CAM_DT_INT64;
+    f.p.T = (int)T;
+    f.p.K = (int)K;
+    f.p.E = (int)numExperts;
+    f.p.R = 1;
+    f.p.pos = (int32_t *)sendTokenIdx->data;
+    f.p.dst_row = slotRowOptional ? (int32_t *)slotRowOptional->data : nullptr;
+    f.p.cnt = numTokensPerExpertOptional ? (int32_t *)numTokensPerExpertOptional->data : nullptr;
+    f.p.off = sendOffsetOptional ? (int32_t *)sendOffsetOptional->data : nullptr;
+    f.p.recv_count = recvCountOptional ? (int32_t *)recvCountOptional->data : nullptr;
+    f.p.tokens_per_expert =
+        numRecvTokensPerExpertOptional ? (int64_t *)numRecvTokensPerExpertOptional->data : nullptr;
+    f.p.total = totalRecvTokensOptional ? (int64_t *)totalRecvTokensOptional->data : nullptr;
+    f.x = (const uint16_t *)x->data;
+    f.x_is_fp16 = x->dtype == CAM_DT_FLOAT16;
+    f.H = (int)H;
+    f.A = A;
+    f.quant = quantMode == 0 ? 0 : (quantMode == 2 ? 1 : 2);
+    f.out = recvX->data;
+    f.scales = quant ? (float *)recvXScalesOptional->data : nullptr;
+    f.src_info = (int32_t *)expandIdx->data;
+    f.src_rank = (int)rankId;
+    Carver c;
+    if (cam::fused_dispatch_fits(T, K)) {
+        const uint64_t o_ctrl = c.take(cam::fused_dispatch_ctrl_bytes());
+        const uint64_t o_table = c.take(cam::fused_dispatch_table_bytes(T, K, (int)numExperts));
+        auto run = [f, o_ctrl, o_table](void *ws, hipStream_t s) mutable -> hipError_t {
+            f.ctrl = (unsigned long long *)((char *)ws + o_ctrl);
+            f.p.hist_ws = (int32_t *)((char *)ws + o_table);
+            return cam::launch_dispatch_fused(f, s);
+        };
+        return finish_phase1(kOpPrefill, c.off, run, workspaceSize, executor);
+    }
+    // More ids than the single launch is built for: the plan and the permute as separate launches.
+    const uint64_t o_hist = c.take(cam::plan_workspace_bytes(T, K, (int)numExperts));
+    const uint64_t o_row = c.take((uint64_t)T * K * 4);
+    auto run = [f, o_hist, o_row](void *ws, hipStream_t s) mutable -> hipError_t {
+        cam::PlanArgs p = f.p;
+        p.hist_ws = (int32_t *)((char *)ws + o_hist);
+        if (p.dst_row == nullptr) {
+            p.dst_row = (int32_t *)((char *)ws + o_row);
+        }
+        hipError_t e = cam::launch_plan(p, s);
+        if (e != hipSuccess) {
+            return e;
+        }
+        cam::DispatchArgs d{};
+        d.x = f.x;
+        d.x_is_fp16 = f.x_is_fp16;
+        d.dst_row = p.dst_row;
+        d.T = p.T;
+        d.K = p.K;
+        d.H = f.H;
+        d.E = p.E;
+        d.A = f.A;
+        d.quant = f.quant;
+        d.out = f.out;
+        d.scales = f.scales;
+        d.src_info = f.src_info;
+        d.src_rank = f.src_rank;
+        return cam::launch_dispatch(d, s);
+    };
+    return finish_phase1(kOpPrefill, c.off, run, workspaceSize, executor);
+}
+
+camStatus camMoeDispatchPrefill(void *workspace, uint64_t workspaceSize, camOpExecutor *executor,
+                                camStream_t stream)
+{
+    return run_phase2(kOpPrefill, "camMoeDispatchPrefill", workspace, workspaceSize, executor, stream);
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -696,10 +874,12 @@ camStatus camMoeCombineNormalGetWorkspaceSize(const camTensor *recvX, const camT
     g.K = (int)K;
     g.H = (int)H;
     g.A = A;
+    // Rows at or past the receive total were never written (moe_combine_normal.h:206-207 bounds its loop the same way).
+    g.row_limit = (const int32_t *)epRecvCounts->data + (moeExpertNum - 1);
     g.out = (uint16_t *)out->data;
     auto run = [g, o_slot](void *ws, hipStream_t s) mutable -> hipError_t {
         int32_t *slot = (int32_t *)((char *)ws + o_slot);
-        hipError_t e = cam::launch_invert_src_info(g.src_info, g.A, g.T, g.K, slot, s);
+        hipError_t e = cam::launch_invert_src_info(g.src_info, g.A, g.row_limit, g.T, g.K, slot, s);
         if (e != hipSuccess) {
             return e;
         }
@@ -731,7 +911,7 @@ camStatus camMoeCombineIndexGetWorkspaceSize(const camTensor *tokenSrcInfo, int6
     int32_t *slot = (int32_t *)slotRow->data;
     const int iT = (int)T, iK = (int)K;
     auto run = [=](void *, hipStream_t s) -> hipError_t {
-        return cam::launch_invert_src_info(src, numRows, iT, iK, slot, s);
+        return cam::launch_invert_src_info(src, numRows, nullptr, iT, iK, slot, s);
     };
     return finish_phase1(kOpCombIndex, 0, run, workspaceSize, executor);
 }
@@ -741,13 +921,12 @@ camStatus camMoeCombineIndex(void *workspace, uint64_t workspaceSize, camOpExecu
     return run_phase2(kOpCombIndex, "camMoeCombineIndex", workspace, workspaceSize, executor, stream);
 }
 
-camStatus camMoeCombineGatherGetWorkspaceSize(const camTensor *recvX, const camTensor *tokenSrcInfo,
-                                              const camTensor *slotRow, const camTensor *recvTopkWeights,
-                                              const camTensor *out, uint64_t *workspaceSize,
-                                              camOpExecutor **executor)
+camStatus camMoeCombineGatherGetWorkspaceSize(const camTensor *recvX, const camTensor *tokenSrcInfoOptional,
+                                              const camTensor *slotRow, const camTensor *epRecvCountsOptional,
+                                              const camTensor *recvTopkWeights, const camTensor *out,
+                                              uint64_t *workspaceSize, camOpExecutor **executor)
 {
     CAM_TRY(check_tensor(recvX, "recvX", 2, CAM_DT_BF16));
-    CAM_TRY(check_tensor(tokenSrcInfo, "tokenSrcInfo", 1, CAM_DT_INT32));
     CAM_TRY(check_tensor(slotRow, "slotRow", 2, CAM_DT_INT32));
     CAM_TRY(check_tensor(recvTopkWeights, "recvTopkWeights", 2, CAM_DT_FLOAT));
     CAM_TRY(check_tensor(out, "out", 2, CAM_DT_BF16));
@@ -768,8 +947,17 @@ camStatus camMoeCombineGatherGetWorkspaceSize(const camTensor *recvX, const camT
     if (out->sizes[0] != T || out->sizes[1] != H) {
         return fail(CAM_ERR_SHAPE, "out must be [T,H]");
     }
-    if (tokenSrcInfo->sizes[0] < 3 * A) {
-        return fail(CAM_ERR_SHAPE, "tokenSrcInfo must hold 3 values per recvX row");
+    if (tokenSrcInfoOptional != nullptr) {
+        CAM_TRY(check_tensor(tokenSrcInfoOptional, "tokenSrcInfo", 1, CAM_DT_INT32));
+        if (tokenSrcInfoOptional->sizes[0] < 3 * A) {
+            return fail(CAM_ERR_SHAPE, "tokenSrcInfo must hold 3 values per recvX row");
+        }
+    }
+    if (epRecvCountsOptional != nullptr) {
+        CAM_TRY(check_tensor(epRecvCountsOptional, "epRecvCounts", 1, CAM_DT_INT32));
+        if (epRecvCountsOptional->sizes[0] < 1) {
+            return fail(CAM_ERR_SHAPE, "epRecvCounts must hold at least one element");
+        }
     }
     if (T * K > 0x7fffffffll || A > 0x7fffffffll) {
         return fail(CAM_ERR_RANGE, "row counts do not fit 32 bits");
@@ -779,7 +967,10 @@ camStatus camMoeCombineGatherGetWorkspaceSize(const camTensor *recvX, const camT
     cam::CombineArgs g{};
     g.y = (const uint16_t *)recvX->data;
     g.slot_row = (const int32_t *)slotRow->data;
-    g.src_info = (const int32_t *)tokenSrcInfo->data;
+    g.src_info = tokenSrcInfoOptional ? (const int32_t *)tokenSrcInfoOptional->data : nullptr;
+    g.row_limit = epRecvCountsOptional
+                      ? (const int32_t *)epRecvCountsOptional->data + (epRecvCountsOptional->sizes[0] - 1)
+                      : nullptr;
     g.w = (const float *)recvTopkWeights->data;
     g.T = (int)T;
     g.K = (int)K;
@@ -1151,7 +1342,10 @@ camStatus camFusedDeepMoeGetWorkspaceSize(const camTensor *x, const camTensor *e
     const uint64_t o_pos = c.take((uint64_t)A * 4);
     const uint64_t o_row = c.take((uint64_t)A * 4);
     const uint64_t o_tiles = c.take(tile_table_bytes(max_tiles));
-    const uint64_t o_hist = c.take(cam::plan_workspace_bytes(T, K, (int)Epr));
+    const bool fused_dispatch = cam::fused_dispatch_fits(T, K);
+    const uint64_t o_hist = c.take(fused_dispatch ? cam::fused_dispatch_table_bytes(T, K, (int)Epr)
+                                                  : cam::plan_workspace_bytes(T, K, (int)Epr));
+    const uint64_t o_ctrl = c.take(cam::fused_dispatch_ctrl_bytes());
     const uint64_t o_x1 = c.take((uint64_t)A * H);
     const uint64_t o_x1s = c.take((uint64_t)A * 4);
     const uint64_t o_prod = c.take((uint64_t)A * I * 4);
@@ -1192,23 +1386,37 @@ camStatus camFusedDeepMoeGetWorkspaceSize(const camTensor *x, const camTensor *e
         p.tokens_per_expert = etn;
         p.tiles = tiles;
         p.hist_ws = (int32_t *)(w + o_hist);
-        hipError_t e = cam::launch_plan(p, s);
-        if (e != hipSuccess) return e;
-
-        cam::DispatchArgs d{};
-        d.x = xp;
-        d.idx = ids;
-        d.dst_row = row;
-        d.T = iT;
-        d.K = iK;
-        d.H = iH;
-        d.E = iE;
-        d.A = A;
-        d.quant = 2;
-        d.out = x1;
-        d.scales = x1s;
-        e = cam::launch_dispatch(d, s);
-        if (e != hipSuccess) return e;
+        hipError_t e;
+        if (fused_dispatch) {
+            cam::FusedDispatchArgs f{};
+            f.p = p;
+            f.x = xp;
+            f.H = iH;
+            f.A = A;
+            f.quant = 2;
+            f.out = x1;
+            f.scales = x1s;
+            f.ctrl = (unsigned long long *)(w + o_ctrl);
+            e = cam::launch_dispatch_fused(f, s);
+            if (e != hipSuccess) return e;
+        } else {
+            e = cam::launch_plan(p, s);
+            if (e != hipSuccess) return e;
+            cam::DispatchArgs d{};
+            d.x = xp;
+            d.idx = ids;
+            d.dst_row = row;
+            d.T = iT;
+            d.K = iK;
+            d.H = iH;
+            d.E = iE;
+            d.A = A;
+            d.quant = 2;
+            d.out = x1;
+            d.scales = x1s;
+            e = cam::launch_dispatch(d, s);
+            if (e != hipSuccess) return e;
+        }
 
         cam::GemmArgs g1{};
         g1.a = x1;

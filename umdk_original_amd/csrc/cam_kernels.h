@@ -41,6 +41,8 @@ struct PlanArgs {
     int32_t *hist_ws;         // required scratch of plan_workspace_bytes(T, K, E) bytes
 };
 uint64_t plan_workspace_bytes(int64_t T, int64_t K, int E);
+// Chunking of the flat id sequence: `it` ids per thread (1, 2, 4 or 8) and `nb` workgroups of 256 threads.
+void plan_geometry(long long n_all, int *it_out, int *nb_out);
 hipError_t launch_plan(const PlanArgs &a, hipStream_t stream);
 
 // isTokenInRank / numTokensPerRank (per_rank must have been zeroed on the same stream).
@@ -72,6 +74,7 @@ struct DispatchArgs {
     int T, K, H, E;
     int64_t A;           // rows in the outputs
     int quant;           // 0 copy, 1 = epsilon variant, 2 = no-epsilon variant
+    int x_is_fp16;       // activations are IEEE fp16 instead of bf16 (matters only when quantising)
     void *out;           // [A,H] bf16 bits or int8
     float *scales;       // [A]   (quant only)
     int32_t *src_info;   // [3A]  optional
@@ -79,10 +82,35 @@ struct DispatchArgs {
 };
 hipError_t launch_dispatch(const DispatchArgs &a, hipStream_t stream);
 
+// Plan + permute in one launch (dispatch_fused.hip).  `p` is the plan (pos required; hist_ws must hold
+// fused_dispatch_table_bytes()); ctrl points at fused_dispatch_ctrl_bytes() of workspace, 8-byte aligned, whose
+// content is arbitrary on the first use and is left cleared by every launch.
+constexpr int kFusedMaxChunks = 256;                 // chunks of 2048 flat ids: T*K <= 524288
+constexpr int kFusedCtrlWords = kFusedMaxChunks + 4;
+struct FusedDispatchArgs {
+    PlanArgs p;
+    const uint16_t *x;   // [T,H] bf16 or fp16 bits
+    int x_is_fp16;
+    int H;
+    int64_t A;           // rows in the outputs
+    int quant;           // as DispatchArgs
+    void *out;
+    float *scales;
+    int32_t *src_info;   // optional
+    int src_rank;
+    unsigned long long *ctrl;
+    int nb;              // set by the launcher
+};
+bool fused_dispatch_fits(int64_t T, int64_t K);
+uint64_t fused_dispatch_table_bytes(int64_t T, int64_t K, int E);
+uint64_t fused_dispatch_ctrl_bytes();
+hipError_t launch_dispatch_fused(FusedDispatchArgs a, hipStream_t stream);
+
 // ---------------------------------------------------------------------------------------------
 // Combine.
-hipError_t launch_invert_src_info(const int32_t *src_info, int64_t A, int T, int K, int32_t *slot_row,
-                                  hipStream_t stream);
+// row_limit: optional device scalar; rows >= *row_limit are ignored (they were never written).
+hipError_t launch_invert_src_info(const int32_t *src_info, int64_t A, const int32_t *row_limit, int T, int K,
+                                  int32_t *slot_row, hipStream_t stream);
 struct CombineArgs {
     const uint16_t *y;        // [A,H] bf16 bits
     const int32_t *slot_row;  // [T,K] row of slot (t,k) (<0: skip)
@@ -90,6 +118,7 @@ struct CombineArgs {
     const float *w;           // [T,K]
     int T, K, H;
     int64_t A;
+    const int32_t *row_limit; // optional device scalar: rows >= *row_limit are never read
     const int32_t *t_active;  // optional device scalar: tokens >= *t_active produce zero rows
     uint16_t *out;            // [T,H]
 };

@@ -22,9 +22,15 @@ namespace {
 constexpr int kCombThreads = 128;
 constexpr int kCombBatch = 8;
 
-__global__ void invert_src_info_kernel(const int32_t *src_info, long long A, int T, int K, int32_t *slot_row)
+// Rows at or beyond *row_limit (the receive total, epRecvCounts[E-1] of moe_combine_normal.h:206-207) were
+// never written by the dispatch that filled the buffers; whatever triple they hold is ignored.
+__global__ void invert_src_info_kernel(const int32_t *src_info, long long A, const int32_t *row_limit, int T, int K,
+                                       int32_t *slot_row)
 {
     long long r = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (row_limit != nullptr) {
+        A = min(A, (long long)*row_limit);
+    }
     if (r >= A) {
         return;
     }
@@ -49,6 +55,7 @@ __global__ __launch_bounds__(kCombThreads) void combine_kernel(CombineArgs a, in
         acc[j] = 0.0f;
     }
     const bool live = a.t_active == nullptr || t < *a.t_active;
+    const long long rows = a.row_limit == nullptr ? a.A : min(a.A, (long long)*a.row_limit);
     if (live) {
         for (int k0 = 0; k0 < a.K; k0 += kCombBatch) {
             v4u v[kCombBatch];
@@ -63,7 +70,7 @@ __global__ __launch_bounds__(kCombThreads) void combine_kernel(CombineArgs a, in
                 if (k < a.K) {
                     const long long slot = (long long)t * a.K + k;
                     const long long row = a.slot_row[slot];
-                    bool good = row >= 0 && row < a.A;
+                    bool good = row >= 0 && row < rows;
                     if (good && a.src_info != nullptr) {
                         // The inverse map is not pre-cleared: accept a row only if it names this slot.
                         good = a.src_info[3 * row + 1] == t && a.src_info[3 * row + 2] == k;
@@ -99,14 +106,14 @@ __global__ __launch_bounds__(kCombThreads) void combine_kernel(CombineArgs a, in
 
 }  // namespace
 
-hipError_t launch_invert_src_info(const int32_t *src_info, int64_t A, int T, int K, int32_t *slot_row,
-                                  hipStream_t stream)
+hipError_t launch_invert_src_info(const int32_t *src_info, int64_t A, const int32_t *row_limit, int T, int K,
+                                  int32_t *slot_row, hipStream_t stream)
 {
     if (A <= 0) {
         return hipSuccess;
     }
     hipLaunchKernelGGL(invert_src_info_kernel, dim3((unsigned)((A + 255) / 256)), dim3(256), 0, stream, src_info,
-                       (long long)A, T, K, slot_row);
+                       (long long)A, row_limit, T, K, slot_row);
     return hipGetLastError();
 }
 

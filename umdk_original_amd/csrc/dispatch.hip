@@ -16,13 +16,11 @@
 // algorithmic minimum: H*2 bytes read and K*H bytes written per token.
 #include "cam_device.h"
 #include "cam_kernels.h"
+#include "permute_device.h"
 
 namespace cam {
 
 namespace {
-
-constexpr int kDispWaves = 4;         // tokens (waves) per workgroup
-constexpr int kDispMaxChunks = 14;    // 16-byte chunks per lane: H <= 14 * 64 * 8 = 7168
 
 // Output row of entry (t,k), or -1.
 __device__ __forceinline__ long long dispatch_row(const DispatchArgs &a, int t, int k)
@@ -40,13 +38,7 @@ __device__ __forceinline__ long long dispatch_row(const DispatchArgs &a, int t, 
     return pre + (window_row - a.recv_offset[e]);
 }
 
-__device__ __forceinline__ uint32_t pack4(int a, int b, int c, int d)
-{
-    return (uint32_t)(a & 0xff) | ((uint32_t)(b & 0xff) << 8) | ((uint32_t)(c & 0xff) << 16) |
-           ((uint32_t)(d & 0xff) << 24);
-}
-
-template <int QUANT>
+template <int QUANT, int ACT>
 __global__ __launch_bounds__(kDispWaves * kWave) void dispatch_kernel(DispatchArgs a)
 {
     const int t = blockIdx.x * kDispWaves + (threadIdx.x >> 6);
@@ -54,86 +46,17 @@ __global__ __launch_bounds__(kDispWaves * kWave) void dispatch_kernel(DispatchAr
     if (t >= a.T) {
         return;
     }
-    const int nch = a.H >> 3;  // 8 bf16 values per chunk
-    const v4u *src = (const v4u *)(a.x + (long long)t * a.H);
-    v4u raw[kDispMaxChunks];
-#pragma unroll
-    for (int j = 0; j < kDispMaxChunks; ++j) {
-        const int c = j * kWave + lane;
-        raw[j] = v4u{0u, 0u, 0u, 0u};
-        if (c < nch) {
-            raw[j] = __builtin_nontemporal_load(src + c);
-        }
-    }
-
-    v2u q[kDispMaxChunks];
-    float scale_out = 0.0f;
+    TokenRow r;
+    load_token_row(a.x, t, a.H, lane, r);
     if (QUANT != 0) {
-        float m = 0.0f;
-#pragma unroll
-        for (int j = 0; j < kDispMaxChunks; ++j) {
-#pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                m = fmaxf(m, fabsf(bf16_bits_to_f32(raw[j][i] & 0xffffu)));
-                m = fmaxf(m, fabsf(bf16_bits_to_f32(raw[j][i] >> 16)));
-            }
-        }
-        m = wave_max(m);
-        float s;
-        bool zero_row = false;
-        if (QUANT == 1) {
-            s = __fdiv_rn(127.0f, __fadd_rn(m, 1e-12f));
-        } else {
-            zero_row = (m == 0.0f);
-            s = zero_row ? 0.0f : __fdiv_rn(127.0f, m);
-        }
-        scale_out = zero_row ? 0.0f : __fdiv_rn(1.0f, s);
-#pragma unroll
-        for (int j = 0; j < kDispMaxChunks; ++j) {
-            int v[8];
-#pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                v[2 * i] = (int)rintf(__fmul_rn(bf16_bits_to_f32(raw[j][i] & 0xffffu), s));
-                v[2 * i + 1] = (int)rintf(__fmul_rn(bf16_bits_to_f32(raw[j][i] >> 16), s));
-            }
-            q[j] = v2u{pack4(v[0], v[1], v[2], v[3]), pack4(v[4], v[5], v[6], v[7])};
-        }
+        quant_token_row<QUANT, ACT>(r);
     }
-
     for (int k = 0; k < a.K; ++k) {
         const long long row = dispatch_row(a, t, k);
         if (row < 0 || row >= a.A) {
             continue;
         }
-        if (QUANT != 0) {
-            v2u *dst = (v2u *)((int8_t *)a.out + row * a.H);
-#pragma unroll
-            for (int j = 0; j < kDispMaxChunks; ++j) {
-                const int c = j * kWave + lane;
-                if (c < nch) {
-                    __builtin_nontemporal_store(q[j], dst + c);
-                }
-            }
-        } else {
-            v4u *dst = (v4u *)((uint16_t *)a.out + row * a.H);
-#pragma unroll
-            for (int j = 0; j < kDispMaxChunks; ++j) {
-                const int c = j * kWave + lane;
-                if (c < nch) {
-                    __builtin_nontemporal_store(raw[j], dst + c);
-                }
-            }
-        }
-        if (lane == 0) {
-            if (QUANT != 0) {
-                a.scales[row] = scale_out;
-            }
-            if (a.src_info != nullptr) {
-                a.src_info[3 * row + 0] = a.src_rank;
-                a.src_info[3 * row + 1] = t;
-                a.src_info[3 * row + 2] = k;
-            }
-        }
+        store_token_row<QUANT>(r, a.out, a.scales, a.src_info, a.src_rank, row, t, k, a.H, lane);
     }
 }
 
@@ -149,11 +72,19 @@ hipError_t launch_dispatch(const DispatchArgs &a, hipStream_t stream)
     }
     dim3 grid((a.T + kDispWaves - 1) / kDispWaves), block(kDispWaves * kWave);
     if (a.quant == 0) {
-        hipLaunchKernelGGL(dispatch_kernel<0>, grid, block, 0, stream, a);
+        hipLaunchKernelGGL((dispatch_kernel<0, 0>), grid, block, 0, stream, a);  // a copy does not look at the format
     } else if (a.quant == 1) {
-        hipLaunchKernelGGL(dispatch_kernel<1>, grid, block, 0, stream, a);
+        if (a.x_is_fp16) {
+            hipLaunchKernelGGL((dispatch_kernel<1, 1>), grid, block, 0, stream, a);
+        } else {
+            hipLaunchKernelGGL((dispatch_kernel<1, 0>), grid, block, 0, stream, a);
+        }
     } else {
-        hipLaunchKernelGGL(dispatch_kernel<2>, grid, block, 0, stream, a);
+        if (a.x_is_fp16) {
+            hipLaunchKernelGGL((dispatch_kernel<2, 1>), grid, block, 0, stream, a);
+        } else {
+            hipLaunchKernelGGL((dispatch_kernel<2, 0>), grid, block, 0, stream, a);
+        }
     }
     return hipGetLastError();
 }

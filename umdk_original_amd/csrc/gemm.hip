@@ -74,7 +74,8 @@ __device__ __forceinline__ int a_lds_offset(int r, int c)
 // data lands at LDS byte address lds_base + 16*i.
 __device__ __forceinline__ void dma16(const void *g, unsigned lds_base)
 {
-    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(lds_base), "v"(g) : "memory");
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(lds_base), "v"(g)
+                 : "memory", "m0");
 }
 
 template <int N>

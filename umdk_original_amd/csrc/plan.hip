@@ -17,172 +17,29 @@
 //      device-to-host copy.
 #include "cam_device.h"
 #include "cam_kernels.h"
+#include "rank_device.h"
 
 namespace cam {
 
 namespace {
 
 constexpr int kScanThreads = 1024;  // single-workgroup scan kernels (notify, tile table)
-constexpr int kLocalThreads = 256;  // phase 1: 4 waves per workgroup
-constexpr int kLocalWaves = kLocalThreads / kWave;
 constexpr int kGlobalThreads = 512; // phase 2: one thread per expert column
 
-template <typename IdT>
-__device__ __forceinline__ int load_id(const IdT *p, long long i, int E)
-{
-    long long v = (long long)p[i];
-    return (v < 0 || v >= (long long)E) ? -1 : (int)v;
-}
-
-// Exclusive scan of one value per thread across a workgroup of NWAVES waves; returns the exclusive
-// prefix and leaves the grand total in *total_out (LDS).  Uses `scratch` (>= NWAVES ints of LDS).
-template <int NWAVES>
-__device__ __forceinline__ int block_exclusive_scan(int v, int tid, int *scratch, int *total_out)
-{
-    int lane = tid & (kWave - 1);
-    int w = tid >> 6;
-    int inc = wave_inclusive_scan(v, lane);
-    if (lane == kWave - 1) {
-        scratch[w] = inc;
-    }
-    __syncthreads();
-    if (w == 0) {
-        int t = lane < NWAVES ? scratch[lane] : 0;
-        int ti = wave_inclusive_scan(t, lane);
-        if (lane < NWAVES) {
-            scratch[lane] = ti - t;
-        }
-        if (lane == NWAVES - 1) {
-            *total_out = ti;
-        }
-    }
-    __syncthreads();
-    int r = inc - v + scratch[w];
-    __syncthreads();
-    return r;
-}
-
-__device__ __forceinline__ int count_active(const uint8_t *mask, int T, int tid, int nthreads, int *slot)
-{
-    if (mask == nullptr) {
-        return T;
-    }
-    int c = 0;
-    for (int t = tid; t < T; t += nthreads) {
-        c += mask[t] != 0 ? 1 : 0;
-    }
-    c = wave_sum(c);
-    if (tid == 0) {
-        *slot = 0;
-    }
-    __syncthreads();
-    if ((tid & (kWave - 1)) == 0 && c != 0) {
-        atomicAdd(slot, c);
-    }
-    __syncthreads();
-    return *slot;
-}
-
-// Tile records of one expert: its `cnt` rows from row `off` on, split evenly over `nt` tiles (equal
-// tiles keep the workgroups that stream the same weight panel in step with each other).
-__device__ __forceinline__ void write_tile_records(int32_t *tiles, int expert, int off, int cnt, int tbase, int nt,
-                                                   int max_tiles)
-{
-    const int q = nt > 0 ? (cnt + nt - 1) / nt : 0;
-    for (int j = 0; j < nt && tbase + j < max_tiles; ++j) {
-        int32_t *t = tiles + kTileHeader + kTileRecord * (tbase + j);
-        t[0] = expert;
-        t[1] = off + j * q;
-        t[2] = min(q, cnt - j * q);
-        t[3] = tbase;
-        t[4] = nt;
-        t[5] = 0;
-        t[6] = 0;
-        t[7] = 0;
-    }
-}
-
-// Phase 1.  Workgroup b owns the flat entries [b*chunk, (b+1)*chunk), chunk = IT*256; wave w of it the
-// IT*64 entries from b*chunk + w*IT*64.  Each lane keeps its IT ids in registers.  64 ids at a time,
-// lanes holding the same id find each other with one ballot per id bit; the rank inside the wave is the
-// wave's running count of that id (LDS) plus the number of lower lanes in the group, and the group's
-// highest lane publishes the new count.  A scan over the 4 waves' histograms turns wave-local ranks
-// into workgroup-local ones; the workgroup's histogram goes to hist_out[b][*].
+// Phase 1.  Workgroup b ranks the flat entries [b*chunk, (b+1)*chunk), chunk = IT*256 (rank_chunk), and
+// publishes the chunk's per-expert histogram in hist_out[b][*].
 template <typename IdT, int IT>
 __global__ __launch_bounds__(kLocalThreads) void plan_local_kernel(PlanArgs a, int32_t *hist_out)
 {
     __shared__ int hist[kLocalWaves * kMaxExperts];
     __shared__ int active_s;
     const int tid = threadIdx.x;
-    const int lane = tid & (kWave - 1);
-    const int w = tid >> 6;
     const int b = blockIdx.x;
-    const int E = a.E;
-    const IdT *__restrict__ idx = (const IdT *)a.idx;
-
-    for (int i = tid; i < kLocalWaves * kMaxExperts; i += kLocalThreads) {
-        hist[i] = 0;
-    }
     const int t_active = count_active(a.mask, a.T, tid, kLocalThreads, &active_s);
-    __syncthreads();
-    const long long n = (long long)t_active * a.K;
-    const long long n_all = (long long)a.T * a.K;
-    const long long base = (long long)b * (IT * kLocalThreads) + (long long)w * (IT * kWave);
-    int nbits = 0;
-    while ((1 << nbits) < E) {
-        ++nbits;
-    }
-    int *my_hist = hist + w * kMaxExperts;
-    const unsigned long long lt_mask = (1ull << lane) - 1ull;
-
-    int e[IT], r[IT];
-#pragma unroll
-    for (int it = 0; it < IT; ++it) {
-        const long long i = base + it * kWave + lane;
-        e[it] = i < n ? load_id(idx, i, E) : -1;
-    }
-#pragma unroll
-    for (int it = 0; it < IT; ++it) {
-        const bool act = e[it] >= 0;
-        unsigned long long peers = __ballot(act);
-        for (int bit_i = 0; bit_i < nbits; ++bit_i) {
-            const bool bit = act && ((e[it] >> bit_i) & 1);
-            const unsigned long long bal = __ballot(bit);
-            peers &= bit ? bal : ~bal;
-        }
-        int prior = 0;
-        r[it] = -1;
-        if (act) {
-            prior = my_hist[e[it]];
-            r[it] = prior + __popcll(peers & lt_mask);
-        }
-        __builtin_amdgcn_wave_barrier();
-        if (act && (peers >> lane) == 1ull) {
-            my_hist[e[it]] = prior + __popcll(peers);
-        }
-        __builtin_amdgcn_wave_barrier();
-    }
-    __syncthreads();
-    for (int ee = tid; ee < E; ee += kLocalThreads) {
-        int run = 0;
-#pragma unroll
-        for (int ww = 0; ww < kLocalWaves; ++ww) {
-            const int t = hist[ww * kMaxExperts + ee];
-            hist[ww * kMaxExperts + ee] = run;
-            run += t;
-        }
-        hist_out[(long long)b * E + ee] = run;
-    }
+    rank_chunk<IdT, IT>((const IdT *)a.idx, b, (long long)t_active * a.K, (long long)a.T * a.K, a.E, hist, a.pos,
+                        hist_out + (long long)b * a.E);
     if (b == 0 && tid == 0) {
-        hist_out[(long long)gridDim.x * E] = t_active;
-    }
-    __syncthreads();
-#pragma unroll
-    for (int it = 0; it < IT; ++it) {
-        const long long i = base + it * kWave + lane;
-        if (i < n_all) {
-            a.pos[i] = e[it] >= 0 ? r[it] + my_hist[e[it]] : -1;
-        }
+        hist_out[(long long)gridDim.x * a.E] = t_active;
     }
 }
 
@@ -394,17 +251,6 @@ __global__ __launch_bounds__(kScanThreads) void build_tiles_kernel(const int64_t
     }
 }
 
-void plan_geometry(long long n_all, int *it_out, int *nb_out)
-{
-    int it = 1;
-    while (it < 8 && (n_all + (long long)it * kLocalThreads - 1) / ((long long)it * kLocalThreads) > 64) {
-        it *= 2;
-    }
-    long long nb = (n_all + (long long)it * kLocalThreads - 1) / ((long long)it * kLocalThreads);
-    *it_out = it;
-    *nb_out = (int)(nb < 1 ? 1 : nb);
-}
-
 template <typename IdT>
 hipError_t launch_plan_t(const PlanArgs &a, int it, int nb, int32_t *hist, hipStream_t stream)
 {
@@ -425,6 +271,17 @@ hipError_t launch_plan_t(const PlanArgs &a, int it, int nb, int32_t *hist, hipSt
 }
 
 }  // namespace
+
+void plan_geometry(long long n_all, int *it_out, int *nb_out)
+{
+    int it = 1;
+    while (it < 8 && (n_all + (long long)it * kLocalThreads - 1) / ((long long)it * kLocalThreads) > 64) {
+        it *= 2;
+    }
+    long long nb = (n_all + (long long)it * kLocalThreads - 1) / ((long long)it * kLocalThreads);
+    *it_out = it;
+    *nb_out = (int)(nb < 1 ? 1 : nb);
+}
 
 uint64_t plan_workspace_bytes(int64_t T, int64_t K, int E)
 {

@@ -25,7 +25,7 @@ from . import _lib
 from ._lib import CamError, CAM_FORMAT_MFMA_B
 
 __all__ = [
-    "CamError", "get_dispatch_layout", "moe_dispatch_plan", "moe_dispatch_prefill", "moe_dispatch_normal",
+    "CamError", "get_dispatch_layout", "moe_dispatch_plan", "moe_dispatch_fused", "moe_dispatch_prefill", "moe_dispatch_normal",
     "moe_combine_prefill", "moe_combine_normal", "moe_combine_index", "moe_combine_gather", "notify_dispatch", "prepack_weight",
     "grouped_matmul_swiglu_quant", "grouped_matmul_dequant", "grouped_matmul_int32", "fused_deep_moe",
 ]
@@ -75,7 +75,8 @@ def moe_dispatch_plan(topk_idx, num_experts, num_ranks=1, rank=0):
     """Device-side replacement of the binding's two CPU loops.
 
     -> dict(send_token_idx [T,K] i32, num_tokens_per_expert [E] i32, send_offset [E] i32,
-            recv_offset [E] i32, recv_count [E] i32, num_recv_tokens_per_expert [E/R] i64, total [1] i64)
+            recv_offset [E] i32, recv_count [E] i32, num_recv_tokens_per_expert [E/R] i64, total [1] i64,
+            slot_row [T,K] i32: output row of every (token, k), -1 where the entry is skipped)
     """
     _require_gpu(topk_idx, "topk_idx")
     T, K = topk_idx.shape
@@ -89,10 +90,44 @@ def moe_dispatch_plan(topk_idx, num_experts, num_ranks=1, rank=0):
         recv_count=torch.empty(num_experts, **i32),
         num_recv_tokens_per_expert=torch.empty(num_experts // max(num_ranks, 1), dtype=torch.int64, device=dev),
         total=torch.empty(1, dtype=torch.int64, device=dev),
+        slot_row=torch.empty((T, K), **i32),
     )
     _lib.call("MoeDispatchPlan", [topk_idx, num_experts, num_ranks, rank, out["send_token_idx"],
                                   out["num_tokens_per_expert"], out["send_offset"], out["recv_offset"],
-                                  out["recv_count"], out["num_recv_tokens_per_expert"], out["total"]])
+                                  out["recv_count"], out["num_recv_tokens_per_expert"], out["total"],
+                                  out["slot_row"]])
+    return out
+
+
+def moe_dispatch_fused(x, topk_idx, num_experts, quant_mode=0, num_rows=None, rank=0, num_ranks=1):
+    """Plan + permute (+ quantisation) in one launch (MoeDispatchPrefill of the C ABI).
+
+    Outputs are sized for `num_rows` rows (default: the worst case T*K); rows at or past total[0] are
+    left unwritten.  -> dict(recv_x, recv_x_scales, expand_idx, send_token_idx, slot_row,
+    num_tokens_per_expert, send_offset, recv_count, num_recv_tokens_per_expert, total)
+    """
+    _require_gpu(x, "x")
+    T, H = x.shape
+    K = topk_idx.size(1)
+    A = max(int(T * K if num_rows is None else num_rows), 1)
+    dev = x.device
+    i32 = dict(dtype=torch.int32, device=dev)
+    out = dict(
+        recv_x=torch.empty((A, H), dtype=torch.int8 if quant_mode != 0 else x.dtype, device=dev),
+        recv_x_scales=torch.empty(A, dtype=torch.float32, device=dev),
+        expand_idx=torch.empty(3 * A, **i32),
+        send_token_idx=torch.empty((T, K), **i32),
+        slot_row=torch.empty((T, K), **i32),
+        num_tokens_per_expert=torch.empty(num_experts, **i32),
+        send_offset=torch.empty(num_experts, **i32),
+        recv_count=torch.empty(num_experts, **i32),
+        num_recv_tokens_per_expert=torch.empty(num_experts // max(num_ranks, 1), dtype=torch.int64, device=dev),
+        total=torch.empty(1, dtype=torch.int64, device=dev),
+    )
+    _lib.call("MoeDispatchPrefill", [x, topk_idx, num_experts, num_ranks, rank, quant_mode, out["recv_x"],
+                                     out["recv_x_scales"], out["expand_idx"], out["send_token_idx"], out["slot_row"],
+                                     out["num_tokens_per_expert"], out["send_offset"], out["recv_count"],
+                                     out["num_recv_tokens_per_expert"], out["total"]])
     return out
 
 
@@ -118,10 +153,11 @@ def moe_dispatch_prefill(x, topk_idx, topk_weights, num_tokens_per_rank, is_toke
     """-> (expand_x [total,H], expand_idx int32 [3*total], recv_count int32 [E],
            num_recv_tokens_per_expert int64 [E/R] on the CPU).
 
-    The total row count decides the output shapes, so one 8-byte device-to-host copy is made (the
-    reference makes two larger ones and runs the index arithmetic on the CPU).  With
-    `num_worst_tokens` > 0 the outputs are allocated at that bound instead, nothing is copied until
-    the fourth return value is produced, and rows beyond the true total are left unwritten.
+    One launch (MoeDispatchPrefill) ranks, places and copies/quantises the rows.  The total row count
+    decides the output shapes, so one 8-byte device-to-host copy is made afterwards (the reference makes
+    two larger ones and runs the index arithmetic on the CPU).  With `num_worst_tokens` > 0 the outputs keep
+    that many rows instead, nothing is copied until the fourth return value is produced, and rows beyond the
+    true total are left unwritten (moe_combine_prefill ignores them: it stops at recv_count[-1]).
     """
     _bind_assert(is_token_in_rank.dtype == torch.bool, "isTokenInRank.scalar_type() == at::kBool")
     _bind_assert(num_tokens_per_expert.dtype == torch.int32, "numTokensPerExpert.scalar_type() == at::kInt")
@@ -147,20 +183,19 @@ def moe_dispatch_prefill(x, topk_idx, topk_weights, num_tokens_per_rank, is_toke
     _bind_assert(topk_weights.dtype == torch.float32, "topkWeights.scalar_type() == at::kFloat")
     _require_gpu(x, "x")
 
-    plan = moe_dispatch_plan(topk_idx, num_experts, num_ranks, rank)
-    if num_worst_tokens and num_worst_tokens > 0:
-        total = int(num_worst_tokens)
-    else:
-        total = int(plan["total"].item())
-    global_bs = max(x.size(0) * num_ranks, int(num_worst_tokens or 0))
-    recv_x, scales, expand_idx = moe_dispatch_normal(
-        x, topk_idx, plan["send_offset"], plan["send_token_idx"], plan["recv_offset"], plan["recv_count"],
-        total, num_experts, quant_mode=quant_mode, group_ep=group_ep, rank=rank, num_ranks=num_ranks,
-        global_bs=global_bs)
-    per_expert_cpu = plan["num_recv_tokens_per_expert"].cpu()
+    worst = bool(num_worst_tokens and num_worst_tokens > 0)
+    d = moe_dispatch_fused(x, topk_idx, num_experts, quant_mode=quant_mode,
+                           num_rows=int(num_worst_tokens) if worst else None, rank=rank, num_ranks=num_ranks)
+    recv_x, scales, expand_idx = d["recv_x"], d["recv_x_scales"], d["expand_idx"]
+    if not worst:
+        # The reference sizes expand_x by the true total (moe_dispatch_prefill.cpp:156-162); the rows were written
+        # into worst-case buffers, so the results are prefix views of those and nothing is copied.
+        total = int(d["total"].item())
+        recv_x, scales, expand_idx = recv_x[:total], scales[:total], expand_idx[:3 * total]
+    per_expert_cpu = d["num_recv_tokens_per_expert"].cpu()
     if return_scales:
-        return recv_x, expand_idx, plan["recv_count"], per_expert_cpu, scales
-    return recv_x, expand_idx, plan["recv_count"], per_expert_cpu
+        return recv_x, expand_idx, d["recv_count"], per_expert_cpu, scales
+    return recv_x, expand_idx, d["recv_count"], per_expert_cpu
 
 
 def moe_combine_normal(recv_x, token_src_info, ep_recv_counts, topk_weights, group_ep="", rank=0, num_ranks=1,
@@ -182,12 +217,16 @@ def moe_combine_index(token_src_info, num_rows, num_tokens, top_k):
     return slot_row
 
 
-def moe_combine_gather(recv_x, token_src_info, slot_row, topk_weights, out=None):
-    """Weighted gather-reduce with a prebuilt map: -> combined bf16 [T,H]."""
+def moe_combine_gather(recv_x, token_src_info, slot_row, topk_weights, out=None, ep_recv_counts=None):
+    """Weighted gather-reduce with a prebuilt map: -> combined bf16 [T,H].
+
+    token_src_info=None trusts slot_row as it stands (the dispatch operators' slot_row output); with the
+    triples given, entries whose row does not point back at the slot are skipped (a map from moe_combine_index).
+    """
     _require_gpu(recv_x, "recv_x")
     if out is None:
         out = torch.empty((topk_weights.size(0), recv_x.size(1)), dtype=recv_x.dtype, device=recv_x.device)
-    _lib.call("MoeCombineGather", [recv_x, token_src_info, slot_row, topk_weights, out])
+    _lib.call("MoeCombineGather", [recv_x, token_src_info, slot_row, ep_recv_counts, topk_weights, out])
     return out
 
 
