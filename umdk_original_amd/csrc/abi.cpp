@@ -426,13 +426,14 @@ camStatus camNotifyDispatch(void *workspace, uint64_t workspaceSize, camOpExecut
 }
 
 // ------------------------------------------------------------------------------------------------
-camStatus camMoeDispatchPlanGetWorkspaceSize(const camTensor *topkIdx, int64_t numExperts, int64_t numRanks,
-                                             int64_t rankId, const camTensor *sendTokenIdx,
-                                             const camTensor *numTokensPerExpert, const camTensor *sendOffset,
-                                             const camTensor *recvOffset, const camTensor *recvCount,
-                                             const camTensor *numRecvTokensPerExpert,
-                                             const camTensor *totalRecvTokens, const camTensor *slotRowOptional,
-                                             uint64_t *workspaceSize, camOpExecutor **executor)
+namespace {
+
+// Validation shared by the two plan entry points; fills every PlanArgs field except the scratch pointer.
+camStatus validate_plan(const camTensor *topkIdx, int64_t numExperts, int64_t numRanks, int64_t rankId,
+                        const camTensor *sendTokenIdx, const camTensor *numTokensPerExpert,
+                        const camTensor *sendOffset, const camTensor *recvOffset, const camTensor *recvCount,
+                        const camTensor *numRecvTokensPerExpert, const camTensor *totalRecvTokens,
+                        const camTensor *slotRowOptional, cam::PlanArgs *out)
 {
     CAM_TRY(check_tensor(topkIdx, "topkIdx", 2, CAM_DT_INT64, CAM_DT_INT32));
     if (numExperts <= 0 || numExperts > cam::kMaxExperts) {
@@ -498,7 +499,24 @@ camStatus camMoeDispatchPlanGetWorkspaceSize(const camTensor *topkIdx, int64_t n
     p.recv_count = recvCount ? (int32_t *)recvCount->data : nullptr;
     p.tokens_per_expert = numRecvTokensPerExpert ? (int64_t *)numRecvTokensPerExpert->data : nullptr;
     p.total = totalRecvTokens ? (int64_t *)totalRecvTokens->data : nullptr;
-    const uint64_t ws_bytes = align_up(cam::plan_workspace_bytes(T, K, (int)numExperts));
+    *out = p;
+    return CAM_OK;
+}
+
+}  // namespace
+
+camStatus camMoeDispatchPlanGetWorkspaceSize(const camTensor *topkIdx, int64_t numExperts, int64_t numRanks,
+                                             int64_t rankId, const camTensor *sendTokenIdx,
+                                             const camTensor *numTokensPerExpert, const camTensor *sendOffset,
+                                             const camTensor *recvOffset, const camTensor *recvCount,
+                                             const camTensor *numRecvTokensPerExpert,
+                                             const camTensor *totalRecvTokens, const camTensor *slotRowOptional,
+                                             uint64_t *workspaceSize, camOpExecutor **executor)
+{
+    cam::PlanArgs p{};
+    CAM_TRY(validate_plan(topkIdx, numExperts, numRanks, rankId, sendTokenIdx, numTokensPerExpert, sendOffset,
+                          recvOffset, recvCount, numRecvTokensPerExpert, totalRecvTokens, slotRowOptional, &p));
+    const uint64_t ws_bytes = align_up(cam::plan_workspace_bytes(p.T, p.K, p.E));
     auto run = [p](void *ws, hipStream_t s) mutable -> hipError_t {
         p.hist_ws = (int32_t *)ws;
         return cam::launch_plan(p, s);
