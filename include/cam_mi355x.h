@@ -157,6 +157,24 @@ CAM_API camStatus camMoeDispatchPlan(void *workspace, uint64_t workspaceSize, ca
                                      camStream_t stream);
 
 /* ------------------------------------------------------------------------------------------------
+ * MoeDispatchPlanNoAlloc -- MoeDispatchPlan in one call that allocates nothing.  It has no counterpart in
+ * the reference; it is for callers that cannot allocate device memory at the call site (code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc): there is no workspace to size and pass and
+ * no executor object.  Same arguments, outputs and validation as MoeDispatchPlan, followed by the stream.
+ * The plan's scratch (one histogram row per ranking workgroup) lives in a 129 KiB array inside the library's
+ * device image; every GPU the library runs on holds its own copy until the process ends.  Limit: at most
+ * 131072 (token, k) entries (T*K); more returns CAM_ERR_RANGE.  Every call on a GPU uses that GPU's one
+ * array, so calls that overlap on one GPU (two streams, two threads) race; calls on one stream do not.
+ * Nothing in the array has to start at zero.  The call must be made with the target device current. */
+CAM_API camStatus camMoeDispatchPlanNoAlloc(const camTensor *topkIdx, int64_t numExperts, int64_t numRanks,
+                                            int64_t rankId, const camTensor *sendTokenIdx,
+                                            const camTensor *numTokensPerExpert, const camTensor *sendOffset,
+                                            const camTensor *recvOffset, const camTensor *recvCount,
+                                            const camTensor *numRecvTokensPerExpert,
+                                            const camTensor *totalRecvTokens, const camTensor *slotRowOptional,
+                                            camStream_t stream);
+
+/* ------------------------------------------------------------------------------------------------
  * MoeDispatchNormal -- replaces aclnnMoeDispatchNormal (AUTOGEN/aclnn_moe_dispatch_normal.h:17-25).
  * x bf16 or fp16 [T,H]; topkIdx int32 [T,K]; sendOffset, recvOffset, recvCount int32 [E]; sendTokenIdx
  * int32 [T,K] -> recvX [A,H] (int8 when quantMode == 2, else x's dtype), recvXScales fp32 [A],

@@ -105,7 +105,13 @@ SIGNATURES = {
                      _TP, _TP],
 }
 
+# Single-call entry points (no executor, no workspace): name -> argument types before the stream.
+DIRECT_SIGNATURES = {
+    "MoeDispatchPlanNoAlloc": [_TP, _I64, _I64, _I64, _TP, _TP, _TP, _TP, _TP, _TP, _TP, _TP],
+}
+
 EXPORTS = ["camGetRecentErrMsg", "camDestroyExecutor", "camGetVersion"] + [
+    "cam%s" % op for op in DIRECT_SIGNATURES] + [
     "cam%s%s" % (op, suffix) for op in SIGNATURES for suffix in ("GetWorkspaceSize", "")
 ]
 
@@ -131,6 +137,10 @@ def lib():
             f2 = getattr(handle, "cam%s" % op)
             f2.argtypes = [ctypes.c_void_p, ctypes.c_uint64, ctypes.c_void_p, ctypes.c_void_p]
             f2.restype = ctypes.c_int32
+        for op, argtypes in DIRECT_SIGNATURES.items():
+            f = getattr(handle, "cam%s" % op)
+            f.argtypes = argtypes + [ctypes.c_void_p]
+            f.restype = ctypes.c_int32
         _lib = handle
     return _lib
 
@@ -233,6 +243,31 @@ def call(op, args, device=None, stream=None, workspace=None):
     if st != CAM_OK:
         raise CamError(st, recent_error())
     return ws
+
+
+def call_direct(op, args, stream=None):
+    """Run a single-call entry point (DIRECT_SIGNATURES) on `stream` (default: torch's current stream)."""
+    handle = lib()
+    argtypes = DIRECT_SIGNATURES[op]
+    if len(args) != len(argtypes):
+        raise TypeError("%s expects %d arguments, got %d" % (op, len(argtypes), len(args)))
+    keep = []
+    cargs = []
+    device = None
+    for a, ty in zip(args, argtypes):
+        if ty is _TP:
+            ct = as_cam_tensor(a) if isinstance(a, torch.Tensor) else a
+            keep.append(ct)
+            if device is None and isinstance(a, torch.Tensor) and a.is_cuda:
+                device = a.device
+            cargs.append(_ptr(ct))
+        else:
+            cargs.append(int(a))
+    if stream is None:
+        stream = torch.cuda.current_stream(device).cuda_stream if device is not None else 0
+    st = getattr(handle, "cam%s" % op)(*cargs, ctypes.c_void_p(stream))
+    if st != CAM_OK:
+        raise CamError(st, recent_error())
 
 
 def phase1(op, args):

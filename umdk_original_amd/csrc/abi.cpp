@@ -12,6 +12,7 @@
 #include <cstdio>
 #include <cstring>
 #include <functional>
+#include <mutex>
 #include <new>
 #include <string>
 
@@ -527,6 +528,79 @@ camStatus camMoeDispatchPlanGetWorkspaceSize(const camTensor *topkIdx, int64_t n
 camStatus camMoeDispatchPlan(void *workspace, uint64_t workspaceSize, camOpExecutor *executor, camStream_t stream)
 {
     return run_phase2(kOpPlan, "camMoeDispatchPlan", workspace, workspaceSize, executor, stream);
+}
+
+// The plan's scratch (one histogram row per ranking workgroup) as library-owned device memory, for the
+// entry point below.  Host code must not use this name as an address: the per-device address comes from
+// hipGetSymbolAddress (scratch_on_current_device).
+constexpr int64_t kNoAllocMaxEntries = 131072;  // T*K: 64 ranking workgroups of 2048 ids
+constexpr size_t kNoAllocScratchBytes = (64 * (size_t)cam::kMaxExperts + 64) * sizeof(int32_t);
+static __device__ __align__(256) unsigned char scratch[kNoAllocScratchBytes];
+
+namespace {
+
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mu;
+void *g_scratch_ptr[kMaxDevices] = {};
+
+// Device address of `scratch` on the current device, resolved once per device.
+hipError_t scratch_on_current_device(void **out)
+{
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) {
+        return e;
+    }
+    if (dev < 0 || dev >= kMaxDevices) {
+        return hipErrorInvalidDevice;
+    }
+    std::lock_guard<std::mutex> lock(g_scratch_mu);
+    if (g_scratch_ptr[dev] == nullptr) {
+        void *ptr = nullptr;
+        e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+        if (e != hipSuccess) {
+            return e;
+        }
+        if (ptr == nullptr) {
+            return hipErrorInvalidSymbol;
+        }
+        g_scratch_ptr[dev] = ptr;
+    }
+    *out = g_scratch_ptr[dev];
+    return hipSuccess;
+}
+
+}  // namespace
+
+camStatus camMoeDispatchPlanNoAlloc(const camTensor *topkIdx, int64_t numExperts, int64_t numRanks, int64_t rankId,
+                                    const camTensor *sendTokenIdx, const camTensor *numTokensPerExpert,
+                                    const camTensor *sendOffset, const camTensor *recvOffset,
+                                    const camTensor *recvCount, const camTensor *numRecvTokensPerExpert,
+                                    const camTensor *totalRecvTokens, const camTensor *slotRowOptional,
+                                    camStream_t stream)
+{
+    cam::PlanArgs p{};
+    CAM_TRY(validate_plan(topkIdx, numExperts, numRanks, rankId, sendTokenIdx, numTokensPerExpert, sendOffset,
+                          recvOffset, recvCount, numRecvTokensPerExpert, totalRecvTokens, slotRowOptional, &p));
+    const int64_t entries = (int64_t)p.T * p.K;
+    if (entries > kNoAllocMaxEntries || cam::plan_workspace_bytes(p.T, p.K, p.E) > kNoAllocScratchBytes) {
+        return fail(CAM_ERR_RANGE,
+                    "MoeDispatchPlanNoAlloc: %lld (token, k) entries exceed the %lld the built-in scratch holds; "
+                    "use MoeDispatchPlan with a workspace",
+                    (long long)entries, (long long)kNoAllocMaxEntries);
+    }
+    void *ptr = nullptr;
+    hipError_t e = scratch_on_current_device(&ptr);
+    if (e != hipSuccess) {
+        return fail(CAM_ERR_LAUNCH, "MoeDispatchPlanNoAlloc: cannot resolve the scratch array: %s",
+                    hipGetErrorString(e));
+    }
+    p.hist_ws = (int32_t *)ptr;
+    e = cam::launch_plan(p, (hipStream_t)stream);
+    if (e != hipSuccess) {
+        return fail(CAM_ERR_LAUNCH, "MoeDispatchPlanNoAlloc: %s", hipGetErrorString(e));
+    }
+    return CAM_OK;
 }
 
 // ------------------------------------------------------------------------------------------------
