@@ -2,14 +2,16 @@
 """Benchmark of the CAM MoE hot path on one MI355X.
 
 One "step" = one dispatch pass (routing plan + permute with per-token int8 quantisation, 4096 tokens x
-7168 bf16, 256 experts, top-8) followed by one combine pass (32768 bf16 rows x 7168 gathered back to
-4096 tokens).  `value` is the algorithmic HBM bytes of both passes divided by the measured time, with all
-inputs resident in HBM.  The same run also reports the grouped w8a8 GEMM (32 local experts, 8192 rows,
-hidden 7168, intermediate 2048) in TOPS and whole fused layers in microseconds.
+7168 bf16, 256 experts, top-8; one kernel launch) followed by one combine pass (32768 bf16 rows x 7168
+gathered back to 4096 tokens).  `value` is the algorithmic HBM bytes of both passes divided by the measured
+time, with all inputs resident in HBM.  The same run also reports the grouped w8a8 GEMM (32 local experts,
+8192 rows, hidden 7168, intermediate 2048) in TOPS and whole fused layers in microseconds.
 
-Every timed region is a HIP graph replayed on torch's current stream and bracketed by HIP events on that
-stream; inside a graph the operator is issued several times on rotating buffer sets, so that no pass finds
-its inputs in the 256 MB last-level cache.  All launches go through the C ABI (libcam_mi355x.so).
+Timing.  The timed region is ONE HIP graph holding exactly --steps steps, replayed once on torch's current
+stream between two HIP events recorded on that stream (after --warmup steps of the same work).  Inside the
+graph consecutive steps use rotating buffer sets, so that no pass finds its inputs in the 256 MB last-level
+cache.  Spread figures (median, p10, p90) come from replays of short graphs, each timed on its own.  All
+launches go through the C ABI (libcam_mi355x.so).
 """
 import argparse
 import json
@@ -39,18 +41,46 @@ def graph_of(fn):
     return g
 
 
-def time_graph(g, replays, warmup):
-    for _ in range(warmup):
-        g.replay()
-    torch.cuda.synchronize()
+def time_once(g):
+    """Seconds of one replay, HIP events on the launch stream."""
     e0 = torch.cuda.Event(enable_timing=True)
     e1 = torch.cuda.Event(enable_timing=True)
     e0.record()
-    for _ in range(replays):
-        g.replay()
+    g.replay()
     e1.record()
     torch.cuda.synchronize()
-    return e0.elapsed_time(e1) * 1e-3 / replays  # seconds per replay
+    return e0.elapsed_time(e1) * 1e-3
+
+
+def spread(g, passes, replays, warm=2):
+    """Per-pass seconds over `replays` individually timed replays of a graph of `passes` passes."""
+    for _ in range(warm):
+        g.replay()
+    torch.cuda.synchronize()
+    ts = sorted(time_once(g) / passes for _ in range(replays))
+    n = len(ts)
+    return dict(mean=sum(ts) / n, median=ts[n // 2], p10=ts[int(0.1 * (n - 1))], p90=ts[int(round(0.9 * (n - 1)))],
+                samples=n)
+
+
+def us(stats):
+    return {k: (v * 1e6 if k != "samples" else v) for k, v in stats.items()}
+
+
+def recorded_traffic(kernel):
+    """HBM bytes per launch of `kernel` from the last committed counter run (profiles/hbm_traffic.txt:
+    rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, calibrated with a copy of known size), or None."""
+    path = os.path.join(ROOT, "profiles", "hbm_traffic.txt")
+    if not os.path.exists(path):
+        return None, None
+    source = None
+    for line in open(path):
+        if line.startswith("# source:"):
+            source = line.split(":", 1)[1].strip()
+        f = line.split()
+        if len(f) >= 2 and f[0] == kernel:
+            return float(f[1]), source
+    return None, source
 
 
 def main():
@@ -61,7 +91,7 @@ def main():
     ap.add_argument("--skip-gemm", action="store_true")
     ap.add_argument("--skip-layer", action="store_true")
     ap.add_argument("--skip-cpu", action="store_true")
-    ap.add_argument("--only", default="", help="comma list of sections: dispatch,combine,gemm,layer")
+    ap.add_argument("--only", default="", help="comma list of sections: step,dispatch,combine,gemm,layer,copy")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build is single-GPU; every figure is measured on one MI355X. "
@@ -82,10 +112,10 @@ def main():
     props = torch.cuda.get_device_properties(dev)
     log("device: %s, %d CUs" % (props.name, props.multi_processor_count))
     NBUF = 4   # rotating buffer sets
-    ROT = 16   # passes per graph (buffer set = pass % NBUF): one replay = ROT steps, which amortises
-               # the ~8 us a graph launch costs
-    replays = max(1, (args.steps + ROT - 1) // ROT)
-    warm = max(1, (args.warmup + ROT - 1) // ROT)
+    ROT = 16   # passes per short graph (spread figures)
+    K_STEPS = max(1, args.steps)
+    W_STEPS = max(0, args.warmup)
+    SPREAD_REPLAYS = 20
 
     result = {}
     kernels = {}
@@ -102,182 +132,258 @@ def main():
         log("copy calibration: 5 launches, 268435456 B read + 268435456 B written each")
         del src, dst
 
-    # ------------------------------------------------------------------ dispatch (config 2)
+    # ------------------------------------------------------------------ dispatch (config 2) + combine (config 4)
     T, H, E, K = 4096, 7168, 256, 8
     A = T * K
     ids64, gate_w = synth.sigmoid_zipf_routing(T, E, K, seed=44)
     ids = ids64.to(torch.int32).to(dev)
     disp_bytes = synth.dispatch_bytes(T, H, K, E)
     comb_bytes = synth.combine_bytes(T, H, K)
-    t_disp = t_plan = t_perm = t_comb = None
+    step_t = t_disp = t_comb = None
+    i32 = dict(dtype=torch.int32, device=dev)
 
-    if want("dispatch"):
+    if want("step") or want("dispatch") or want("combine"):
         xs = [synth.normal_bf16(T, H, seed=44 + i).to(dev) for i in range(NBUF)]
-        i32 = dict(dtype=torch.int32, device=dev)
-        plan_bufs = [dict(pos=torch.empty((T, K), **i32), cnt=torch.empty(E, **i32), off=torch.empty(E, **i32),
-                          roff=torch.empty(E, **i32), rcnt=torch.empty(E, **i32),
-                          tpe=torch.empty(E, dtype=torch.int64, device=dev),
-                          total=torch.empty(1, dtype=torch.int64, device=dev),
-                          ws=torch.empty(1 << 18, dtype=torch.uint8, device=dev)) for _ in range(NBUF)]
-        outs = [dict(rx=torch.empty((A, H), dtype=torch.int8, device=dev),
-                     sc=torch.empty(A, dtype=torch.float32, device=dev),
-                     info=torch.empty(3 * A, **i32)) for _ in range(NBUF)]
-
-        def run_plan(i):
-            p = plan_bufs[i % NBUF]
-            _lib.call("MoeDispatchPlan", [ids, E, 1, 0, p["pos"], p["cnt"], p["off"], p["roff"], p["rcnt"], p["tpe"],
-                                          p["total"]], workspace=p["ws"])
-
-        def run_permute(i):
-            p, o, i = plan_bufs[i % NBUF], outs[i % NBUF], i % NBUF
-            _lib.call("MoeDispatchNormal", [xs[i], ids, p["off"], p["pos"], p["roff"], p["rcnt"], "", 1, 0, "", 1, 0,
-                                            E, 2, 0, o["rx"], o["sc"], o["info"]])
-
-        def disp_all():
-            for i in range(ROT):
-                run_plan(i)
-                run_permute(i)
-
-        def plan_only():
-            for i in range(ROT):
-                run_plan(i)
-
-        def perm_only():
-            for i in range(ROT):
-                run_permute(i)
-
-        t_disp = time_graph(graph_of(disp_all), replays, warm) / ROT
-        t_plan = time_graph(graph_of(plan_only), replays, warm) / ROT
-        t_perm = time_graph(graph_of(perm_only), replays, warm) / ROT
-        log("dispatch: %.1f us (plan kernel %.1f us, permute+quant kernel %.1f us) -> %.0f GB/s = %.1f%% of HBM peak"
-            % (t_disp * 1e6, t_plan * 1e6, t_perm * 1e6, disp_bytes / t_disp / 1e9, 100 * disp_bytes / t_disp / HBM_PEAK))
-        perm_bytes = T * H * 2 + A * 4 + A * H + A * 4 + A * 12  # x, row ids, int8 rows, scales, triples
-        kernels["dispatch_permute_quant"] = dict(bound="hbm", us=t_perm * 1e6, bytes=perm_bytes,
-                                                 achieved=perm_bytes / t_perm / 1e9, peak=HBM_PEAK / 1e9, unit="GB/s",
-                                                 frac=perm_bytes / t_perm / HBM_PEAK)
-        kernels["dispatch_plan"] = dict(bound="latency", us=t_plan * 1e6)
-        del xs, outs
-        torch.cuda.empty_cache()
-
-    # ------------------------------------------------------------------ combine (config 4)
-    if want("combine"):
-        import numpy as np
-        plan = cam.moe_dispatch_plan(ids, E)
         ys = [synth.normal_bf16(A, H, seed=46 + i).to(dev) for i in range(NBUF)]
-        # triples as the dispatch kernel writes them
-        dummy = torch.empty((A, 1024), dtype=torch.bfloat16, device=dev)
-        _, _, info = cam.moe_dispatch_normal(torch.zeros((T, 1024), dtype=torch.bfloat16, device=dev), ids,
-                                             plan["send_offset"], plan["send_token_idx"], plan["recv_offset"],
-                                             plan["recv_count"], A, E)
-        del dummy
         gw = gate_w.to(dev)
+        st, ws_bytes, msg = _lib.phase1("MoeDispatchPrefill", [
+            xs[0], ids, E, 1, 0, 2, torch.empty((A, H), dtype=torch.int8), torch.empty(A), torch.empty(3 * A, dtype=torch.int32),
+            torch.empty((T, K), dtype=torch.int32), torch.empty((T, K), dtype=torch.int32), None, None,
+            torch.empty(E, dtype=torch.int32), None, torch.empty(1, dtype=torch.int64)])
+        assert st == 0, msg
+        dsets = [dict(rx=torch.empty((A, H), dtype=torch.int8, device=dev),
+                      sc=torch.empty(A, dtype=torch.float32, device=dev), info=torch.empty(3 * A, **i32),
+                      pos=torch.empty((T, K), **i32), slot=torch.empty((T, K), **i32), cnt=torch.empty(E, **i32),
+                      off=torch.empty(E, **i32), rcnt=torch.empty(E, **i32),
+                      tpe=torch.empty(E, dtype=torch.int64, device=dev),
+                      total=torch.empty(1, dtype=torch.int64, device=dev),
+                      ws=torch.empty(ws_bytes + 256, dtype=torch.uint8, device=dev)) for _ in range(NBUF)]
         couts = [torch.empty((T, H), dtype=torch.bfloat16, device=dev) for _ in range(NBUF)]
-        wss = [torch.empty(T * K * 4 + 256, dtype=torch.uint8, device=dev) for _ in range(NBUF)]
 
-        def comb_all():
+        def run_dispatch(i):
+            d = dsets[i % NBUF]
+            _lib.call("MoeDispatchPrefill", [xs[i % NBUF], ids, E, 1, 0, 2, d["rx"], d["sc"], d["info"], d["pos"],
+                                             d["slot"], d["cnt"], d["off"], d["rcnt"], d["tpe"], d["total"]],
+                      workspace=d["ws"])
+
+        def run_combine(i):
+            d = dsets[i % NBUF]
+            # the (token, k) -> row map the dispatch produced, handed straight to the gather
+            _lib.call("MoeCombineGather", [ys[i % NBUF], None, d["slot"], d["rcnt"], gw, couts[i % NBUF]])
+
+        for i in range(NBUF):
+            run_dispatch(i)  # fills every set's map before any combine-only graph runs
+        torch.cuda.synchronize()
+
+        if want("step"):
+            def steps(n):
+                def f():
+                    for i in range(n):
+                        run_dispatch(i)
+                        run_combine(i)
+                return f
+            if W_STEPS:
+                graph_of(steps(W_STEPS)).replay()
+            g_step = graph_of(steps(K_STEPS))
+            torch.cuda.synchronize()
+            step_t = time_once(g_step) / K_STEPS
+            step_spread = spread(graph_of(steps(ROT)), ROT, SPREAD_REPLAYS)
+            log("step (dispatch + combine): %.1f us over exactly %d steps -> %.0f GB/s = %.1f%% of HBM peak; "
+                "median %.1f us (p10 %.1f, p90 %.1f)"
+                % (step_t * 1e6, K_STEPS, (disp_bytes + comb_bytes) / step_t / 1e9,
+                   100 * (disp_bytes + comb_bytes) / step_t / HBM_PEAK, step_spread["median"] * 1e6,
+                   step_spread["p10"] * 1e6, step_spread["p90"] * 1e6))
+            result["step_us"] = us(step_spread)
+
+        def disp_rot():
             for i in range(ROT):
-                _lib.call("MoeCombineNormal", [ys[i % NBUF], info, plan["recv_count"], gw, None, "", 1, 0, "", 1, 0, E,
-                                               0, couts[i % NBUF]], workspace=wss[i % NBUF])
+                run_dispatch(i)
 
-        t_comb = time_graph(graph_of(comb_all), replays, warm) / ROT
-        # The operator is two kernels (inverse map, then gather); the two halves exist as operators of their
-        # own, which lets the gather kernel be timed alone.
-        slots = [torch.empty((T, K), dtype=torch.int32, device=dev) for _ in range(NBUF)]
-
-        def index_only():
+        def comb_rot():
             for i in range(ROT):
-                _lib.call("MoeCombineIndex", [info, A, slots[i % NBUF]])
+                run_combine(i)
 
-        def gather_only():
-            for i in range(ROT):
-                _lib.call("MoeCombineGather", [ys[i % NBUF], info, slots[i % NBUF], gw, couts[i % NBUF]])
+        if want("step") or want("dispatch"):
+            s_disp = spread(graph_of(disp_rot), ROT, SPREAD_REPLAYS)
+            t_disp = s_disp["mean"]
+            perm_bytes = T * H * 2 + A * 4 + A * H + A * 4 + A * 12 + 2 * A * 4  # x, ids, rows, scales, triples, pos + map
+            kernels["dispatch_fused"] = dict(bound="hbm", us=us(s_disp), bytes=perm_bytes,
+                                             achieved=perm_bytes / t_disp / 1e9, peak=HBM_PEAK / 1e9, unit="GB/s",
+                                             frac=perm_bytes / t_disp / HBM_PEAK,
+                                             note="MoeDispatchPrefill: plan + permute + int8 quant, one launch")
+            log("dispatch (one launch): %.1f us -> %.0f GB/s = %.1f%% of HBM peak"
+                % (t_disp * 1e6, disp_bytes / t_disp / 1e9, 100 * disp_bytes / t_disp / HBM_PEAK))
+            # the same work as the reference's operator pair: plan, then aclnn-shaped permute (3 launches)
+            plan_bufs = [dict(pos=torch.empty((T, K), **i32), cnt=torch.empty(E, **i32), off=torch.empty(E, **i32),
+                              roff=torch.empty(E, **i32), rcnt=torch.empty(E, **i32),
+                              tpe=torch.empty(E, dtype=torch.int64, device=dev),
+                              total=torch.empty(1, dtype=torch.int64, device=dev),
+                              ws=torch.empty(1 << 18, dtype=torch.uint8, device=dev)) for _ in range(NBUF)]
 
-        t_index = time_graph(graph_of(index_only), replays, warm) / ROT
-        t_gather = time_graph(graph_of(gather_only), replays, warm) / ROT
-        log("combine: %.1f us (inverse-map kernel %.1f us, gather kernel %.1f us) -> %.0f GB/s = %.1f%% of HBM peak"
-            % (t_comb * 1e6, t_index * 1e6, t_gather * 1e6, comb_bytes / t_comb / 1e9,
-               100 * comb_bytes / t_comb / HBM_PEAK))
-        gather_bytes = A * H * 2 + A * 4 + A * 4 + T * H * 2  # rows, weights, map, output
-        kernels["combine_gather"] = dict(bound="hbm", us=t_gather * 1e6, bytes=gather_bytes,
-                                         achieved=gather_bytes / t_gather / 1e9, peak=HBM_PEAK / 1e9, unit="GB/s",
-                                         frac=gather_bytes / t_gather / HBM_PEAK)
-        kernels["combine_index"] = dict(bound="latency", us=t_index * 1e6)
-        # decode-shaped variant
-        Td = 128
-        idd, gwd = synth.sigmoid_zipf_routing(Td, E, K, seed=47)
-        idd32 = idd.to(torch.int32).to(dev)
-        pland = cam.moe_dispatch_plan(idd32, E)
-        _, _, infod = cam.moe_dispatch_normal(torch.zeros((Td, 1024), dtype=torch.bfloat16, device=dev), idd32,
-                                              pland["send_offset"], pland["send_token_idx"], pland["recv_offset"],
-                                              pland["recv_count"], Td * K, E)
-        yd = [synth.normal_bf16(Td * K, H, seed=48 + i).to(dev) for i in range(NBUF)]
-        od = [torch.empty((Td, H), dtype=torch.bfloat16, device=dev) for _ in range(NBUF)]
-        gwd = gwd.to(dev)
+            def pair_rot():
+                for i in range(ROT):
+                    p, d = plan_bufs[i % NBUF], dsets[i % NBUF]
+                    _lib.call("MoeDispatchPlan", [ids, E, 1, 0, p["pos"], p["cnt"], p["off"], p["roff"], p["rcnt"],
+                                                  p["tpe"], p["total"], None], workspace=p["ws"])
+                    _lib.call("MoeDispatchNormal", [xs[i % NBUF], ids, p["off"], p["pos"], p["roff"], p["rcnt"], "", 1,
+                                                    0, "", 1, 0, E, 2, 0, d["rx"], d["sc"], d["info"]])
 
-        def comb_decode():
-            for i in range(ROT):
-                _lib.call("MoeCombineNormal", [yd[i % NBUF], infod, pland["recv_count"], gwd, None, "", 1, 0, "", 1, 0,
-                                               E, 0, od[i % NBUF]], workspace=wss[i % NBUF])
+            s_pair = spread(graph_of(pair_rot), ROT, SPREAD_REPLAYS)
+            kernels["dispatch_plan_then_normal"] = dict(bound="hbm", us=us(s_pair),
+                                                        achieved=disp_bytes / s_pair["mean"] / 1e9, unit="GB/s",
+                                                        frac=disp_bytes / s_pair["mean"] / HBM_PEAK,
+                                                        note="MoeDispatchPlan + MoeDispatchNormal, three launches")
+            log("dispatch as plan + normal operators: %.1f us" % (s_pair["mean"] * 1e6))
+            del plan_bufs
 
-        t_cd = time_graph(graph_of(comb_decode), replays, warm) / ROT
-        cd_bytes = synth.combine_bytes(Td, H, K)
-        log("combine decode (T=128): %.2f us -> %.0f GB/s" % (t_cd * 1e6, cd_bytes / t_cd / 1e9))
-        result["combine_decode"] = dict(tokens=Td, us=t_cd * 1e6, gb_per_s=cd_bytes / t_cd / 1e9, bytes=cd_bytes)
-        del ys, couts
+        if want("step") or want("combine"):
+            s_comb = spread(graph_of(comb_rot), ROT, SPREAD_REPLAYS)
+            t_comb = s_comb["mean"]
+            gather_bytes = A * H * 2 + A * 4 + A * 4 + T * H * 2  # rows, weights, map, output
+            kernels["combine_gather"] = dict(bound="hbm", us=us(s_comb), bytes=gather_bytes,
+                                             achieved=gather_bytes / t_comb / 1e9, peak=HBM_PEAK / 1e9, unit="GB/s",
+                                             frac=gather_bytes / t_comb / HBM_PEAK,
+                                             note="MoeCombineGather with the dispatch's (token, k) -> row map")
+            log("combine (gather with the dispatch's map): %.1f us -> %.0f GB/s = %.1f%% of HBM peak"
+                % (t_comb * 1e6, comb_bytes / t_comb / 1e9, 100 * comb_bytes / t_comb / HBM_PEAK))
+            wss = [torch.empty(T * K * 4 + 256, dtype=torch.uint8, device=dev) for _ in range(NBUF)]
+
+            def normal_rot():
+                for i in range(ROT):
+                    d = dsets[i % NBUF]
+                    _lib.call("MoeCombineNormal", [ys[i % NBUF], d["info"], d["rcnt"], gw, None, "", 1, 0, "", 1, 0, E,
+                                                   0, couts[i % NBUF]], workspace=wss[i % NBUF])
+
+            s_norm = spread(graph_of(normal_rot), ROT, SPREAD_REPLAYS)
+            kernels["combine_normal"] = dict(bound="hbm", us=us(s_norm), achieved=comb_bytes / s_norm["mean"] / 1e9,
+                                             unit="GB/s", frac=comb_bytes / s_norm["mean"] / HBM_PEAK,
+                                             note="MoeCombineNormal: inverse map from the triples, then gather")
+            log("combine as the aclnn-shaped operator (inverse map + gather): %.1f us" % (s_norm["mean"] * 1e6))
+            # decode-shaped variant
+            Td = 128
+            idd, gwd = synth.sigmoid_zipf_routing(Td, E, K, seed=47)
+            dd = cam.moe_dispatch_fused(torch.zeros((Td, 1024), dtype=torch.bfloat16, device=dev),
+                                        idd.to(torch.int32).to(dev), E)
+            yd = [synth.normal_bf16(Td * K, H, seed=48 + i).to(dev) for i in range(NBUF)]
+            od = [torch.empty((Td, H), dtype=torch.bfloat16, device=dev) for _ in range(NBUF)]
+            gwd = gwd.to(dev)
+
+            def comb_decode():
+                for i in range(ROT):
+                    _lib.call("MoeCombineGather", [yd[i % NBUF], None, dd["slot_row"], dd["recv_count"], gwd,
+                                                   od[i % NBUF]])
+
+            s_cd = spread(graph_of(comb_decode), ROT, SPREAD_REPLAYS)
+            cd_bytes = synth.combine_bytes(Td, H, K)
+            log("combine decode (T=128): %.2f us -> %.0f GB/s" % (s_cd["mean"] * 1e6, cd_bytes / s_cd["mean"] / 1e9))
+            result["combine_decode"] = dict(tokens=Td, us=us(s_cd), gb_per_s=cd_bytes / s_cd["mean"] / 1e9,
+                                            bytes=cd_bytes)
+            del wss, yd, od
+        del xs, ys, dsets, couts
         torch.cuda.empty_cache()
 
     # ------------------------------------------------------------------ grouped GEMM (config 3)
     if want("gemm") and not args.skip_gemm:
         G, I, rows = 32, 2048, 8192
+        NG = 3  # rotating operand sets (weights 1.4 GB each): no pass finds its weights in the last-level cache
         sizes = synth.zipf_group_sizes(G, rows, seed=45)
         gl = torch.cumsum(sizes, 0).to(dev)
-        a = synth.uniform_int8((rows, H), 45).to(dev)
-        xsc = synth.channel_scales((rows,), 451, 0.005, 0.05).to(dev)
-        gen = torch.Generator(device=dev).manual_seed(452)
-        w1 = torch.randint(-127, 128, (G, H, 2 * I), generator=gen, dtype=torch.int8, device=dev)
-        w2 = torch.randint(-127, 128, (G, I, H), generator=gen, dtype=torch.int8, device=dev)
-        w1p = cam.prepack_weight(w1, True)
-        w2p = cam.prepack_weight(w2, False)
-        del w1, w2
-        w1s = synth.channel_scales((G, 2 * I), 453).to(dev)
-        w2s = synth.channel_scales((G, H), 454).to(dev)
-        y = torch.empty((rows, I), dtype=torch.int8, device=dev)
-        ysc = torch.empty(rows, dtype=torch.float32, device=dev)
-        out = torch.empty((rows, H), dtype=torch.bfloat16, device=dev)
-        ws1 = torch.empty(rows * I * 4 + (1 << 16), dtype=torch.uint8, device=dev)
-        ws2 = torch.empty(1 << 16, dtype=torch.uint8, device=dev)
+        gsets = []
+        for j in range(NG):
+            gen = torch.Generator(device=dev).manual_seed(452 + j)
+            w1 = torch.randint(-127, 128, (G, H, 2 * I), generator=gen, dtype=torch.int8, device=dev)
+            w2 = torch.randint(-127, 128, (G, I, H), generator=gen, dtype=torch.int8, device=dev)
+            gsets.append(dict(a=synth.uniform_int8((rows, H), 45 + j).to(dev),
+                              xsc=synth.channel_scales((rows,), 451 + j, 0.005, 0.05).to(dev),
+                              w1p=cam.prepack_weight(w1, True), w2p=cam.prepack_weight(w2, False),
+                              w1s=synth.channel_scales((G, 2 * I), 453).to(dev),
+                              w2s=synth.channel_scales((G, H), 454).to(dev),
+                              y=torch.empty((rows, I), dtype=torch.int8, device=dev),
+                              ysc=torch.empty(rows, dtype=torch.float32, device=dev),
+                              out=torch.empty((rows, H), dtype=torch.bfloat16, device=dev)))
+            del w1, w2
+        s0 = gsets[0]
+        st, ws1_bytes, msg = _lib.phase1("GroupedMatmulSwigluQuant", [s0["a"], s0["xsc"], [s0["w1p"]], [s0["w1s"]], gl,
+                                                                      0, s0["y"], s0["ysc"]])
+        assert st == 0, msg
+        st, ws2_bytes, msg = _lib.phase1("GroupedMatmulDequant", [s0["y"], s0["ysc"], [s0["w2p"]], [s0["w2s"]], gl, 0,
+                                                                  s0["out"]])
+        assert st == 0, msg
+        ws1 = torch.empty(ws1_bytes + 256, dtype=torch.uint8, device=dev)
+        ws2 = torch.empty(ws2_bytes + 256, dtype=torch.uint8, device=dev)
 
-        def gmm1():
-            _lib.call("GroupedMatmulSwigluQuant", [a, xsc, [w1p], [w1s], gl, 0, y, ysc], workspace=ws1)
+        def gmm1(j):
+            s = gsets[j % NG]
+            _lib.call("GroupedMatmulSwigluQuant", [s["a"], s["xsc"], [s["w1p"]], [s["w1s"]], gl, 0, s["y"], s["ysc"]],
+                      workspace=ws1)
 
-        def gmm2():
-            _lib.call("GroupedMatmulDequant", [y, ysc, [w2p], [w2s], gl, 0, out], workspace=ws2)
+        def gmm2(j):
+            s = gsets[j % NG]
+            _lib.call("GroupedMatmulDequant", [s["y"], s["ysc"], [s["w2p"]], [s["w2s"]], gl, 0, s["out"]],
+                      workspace=ws2)
 
-        def both():
-            gmm1()
-            gmm2()
+        for j in range(NG):
+            gmm1(j)  # every set's y holds real GMM1 output before GMM2 is timed alone
+        PG = 2 * NG
 
-        n = max(10, args.steps // 4)
-        t_g1 = time_graph(graph_of(gmm1), n, 5)
-        t_g2 = time_graph(graph_of(gmm2), n, 5)
-        t_g = time_graph(graph_of(both), n, 5)
+        def rot(fn):
+            def f():
+                for j in range(PG):
+                    fn(j)
+            return f
+
+        def both(j):
+            gmm1(j)
+            gmm2(j)
+
+        reps = max(5, min(SPREAD_REPLAYS, K_STEPS // PG))
+        s_g1 = spread(graph_of(rot(gmm1)), PG, reps)
+        s_g2 = spread(graph_of(rot(gmm2)), PG, reps)
+        s_g = spread(graph_of(rot(both)), PG, reps)
+        t_g = s_g["mean"]
         ops1 = 2 * rows * H * 2 * I
         ops2 = 2 * rows * I * H
-        gemm_bytes = G * (H * 2 * I + I * H) + rows * H + 2 * rows * I + rows * H * 2
-        log("grouped GEMM: %.1f us total (GMM1 op %.1f us, GMM2 op %.1f us) -> %.0f TOPS = %.1f%% of int8 peak; "
-            "%.0f GB/s" % (t_g * 1e6, t_g1 * 1e6, t_g2 * 1e6, (ops1 + ops2) / t_g / 1e12,
-                           100 * (ops1 + ops2) / t_g / INT8_PEAK, gemm_bytes / t_g / 1e9))
-        result["grouped_gemm"] = dict(us=t_g * 1e6, tops=(ops1 + ops2) / t_g / 1e12, ops=ops1 + ops2,
-                                      frac_int8_peak=(ops1 + ops2) / t_g / INT8_PEAK, gb_per_s=gemm_bytes / t_g / 1e9,
-                                      rows=rows, experts=G, empty_experts=int((sizes == 0).sum()),
-                                      max_rows_per_expert=int(sizes.max()))
-        kernels["gmm1_swiglu_quant"] = dict(bound="mfma", us=t_g1 * 1e6, ops=ops1, achieved=ops1 / t_g1 / 1e12,
-                                            peak=INT8_PEAK / 1e12, unit="TOP/s", frac=ops1 / t_g1 / INT8_PEAK,
+        live = int((sizes > 0).sum())
+        gemm_bytes = live * (H * 2 * I + I * H) + rows * H + 2 * rows * I + rows * H * 2
+        log("grouped GEMM: %.1f us both operators (GMM1 %.1f us, GMM2 %.1f us; median of both %.1f us) -> %.0f TOPS = "
+            "%.1f%% of int8 peak; %.0f GB/s" % (t_g * 1e6, s_g1["mean"] * 1e6, s_g2["mean"] * 1e6, s_g["median"] * 1e6,
+                                                (ops1 + ops2) / t_g / 1e12, 100 * (ops1 + ops2) / t_g / INT8_PEAK,
+                                                gemm_bytes / t_g / 1e9))
+        result["grouped_gemm"] = dict(us=us(s_g), tops=(ops1 + ops2) / t_g / 1e12, ops=ops1 + ops2,
+                                      frac_int8_peak=(ops1 + ops2) / t_g / INT8_PEAK,
+                                      min_bytes=gemm_bytes, gb_per_s=gemm_bytes / t_g / 1e9,
+                                      frac_hbm_peak=gemm_bytes / t_g / HBM_PEAK, rows=rows, experts=G,
+                                      empty_experts=int((sizes == 0).sum()), max_rows_per_expert=int(sizes.max()),
+                                      operand_sets=NG)
+        kernels["gmm1_swiglu_quant"] = dict(bound="mfma", us=us(s_g1), ops=ops1, achieved=ops1 / s_g1["mean"] / 1e12,
+                                            peak=INT8_PEAK / 1e12, unit="TOP/s", frac=ops1 / s_g1["mean"] / INT8_PEAK,
                                             note="operator time: tile table + GEMM + re-quant kernels")
-        kernels["gmm2_dequant"] = dict(bound="mfma", us=t_g2 * 1e6, ops=ops2, achieved=ops2 / t_g2 / 1e12,
-                                       peak=INT8_PEAK / 1e12, unit="TOP/s", frac=ops2 / t_g2 / INT8_PEAK,
+        kernels["gmm2_dequant"] = dict(bound="mfma", us=us(s_g2), ops=ops2, achieved=ops2 / s_g2["mean"] / 1e12,
+                                       peak=INT8_PEAK / 1e12, unit="TOP/s", frac=ops2 / s_g2["mean"] / INT8_PEAK,
                                        note="operator time: tile table + GEMM kernels")
-        del w1p, w2p, a, y, out, ws1
+        # uniform experts: the inner kernel without the grouped shape's skew (8 experts x 1024 rows)
+        Gu = 8
+        glu = torch.arange(1, Gu + 1, dtype=torch.int64, device=dev) * (rows // Gu)
+
+        for s in gsets:
+            s["w1p_u"] = s["w1p"][:Gu]  # the first 8 experts' packed weights: a view, tagged like its parent
+            s["w1p_u"]._cam_format = _lib.CAM_FORMAT_MFMA_B
+            s["w1s_u"] = s["w1s"][:Gu].contiguous()
+
+        def uni(j):
+            s = gsets[j % NG]
+            _lib.call("GroupedMatmulSwigluQuant", [s["a"], s["xsc"], [s["w1p_u"]], [s["w1s_u"]], glu, 0, s["y"],
+                                                   s["ysc"]], workspace=ws1)
+
+        try:
+            s_u = spread(graph_of(rot(uni)), PG, reps)
+            result["gmm1_uniform_8x1024"] = dict(us=us(s_u), tops=ops1 / s_u["mean"] / 1e12,
+                                                 frac_int8_peak=ops1 / s_u["mean"] / INT8_PEAK)
+            log("GMM1 on 8 uniform experts of 1024 rows: %.1f us -> %.0f TOPS" % (s_u["mean"] * 1e6,
+                                                                                   ops1 / s_u["mean"] / 1e12))
+        except cam.CamError as ex:  # the slice lost its format tag
+            log("uniform-expert GEMM skipped: %s" % ex)
+        del gsets, ws1, ws2
         torch.cuda.empty_cache()
 
     # ------------------------------------------------------------------ whole fused layers
@@ -311,53 +417,106 @@ def main():
                 _lib.call("FusedDeepMoe", [xl, idl32, [w1], [w1s], [w2], [w2s], gl_w, None, None, "", 1, 0, El, 1, 0,
                                            0, 0, outl, etn], workspace=wsl)
 
-            n = max(10, args.steps // 4)
-            t_l = time_graph(graph_of(layer), n, 5)
+            s_l = spread(graph_of(layer), 1, max(10, min(SPREAD_REPLAYS, K_STEPS // 4)))
             ops = synth.gemm_ops(Tl * Kl, Hl, Il)
-            log("fused layer %s: %.1f us (%.0f TOPS)" % (name, t_l * 1e6, ops / t_l / 1e12))
-            layers[name] = dict(us=t_l * 1e6, tokens=Tl, hidden=Hl, experts=El, top_k=Kl, intermediate=Il,
-                                tops=ops / t_l / 1e12, dtype="int8 weights and activations (w8a8)")
+            log("fused layer %s: %.1f us (median %.1f; %.0f TOPS)" % (name, s_l["mean"] * 1e6, s_l["median"] * 1e6,
+                                                                      ops / s_l["mean"] / 1e12))
+            layers[name] = dict(us=s_l["mean"] * 1e6, us_spread=us(s_l), tokens=Tl, hidden=Hl, experts=El, top_k=Kl,
+                                intermediate=Il, tops=ops / s_l["mean"] / 1e12, workspace_bytes=ws_bytes,
+                                dtype="int8 weights and activations (w8a8)")
             del w1, w2, wsl, xl, outl
             torch.cuda.empty_cache()
         result["fused_layer_us"] = layers
 
-    # ------------------------------------------------------------------ CPU baseline (oracle, bounded sample)
+    # ------------------------------------------------------------------ CPU baseline (the oracle on the host cores)
     cpu = None
-    if not args.skip_cpu and want("dispatch") and want("combine"):
+    if not args.skip_cpu and want("step"):
         sys.path.insert(0, os.path.join(ROOT, "oracle"))
         import cam_oracle
         import numpy as np
-        Ts = 1024  # a quarter of the workload's tokens, same H / E / K
-        ids_s = ids64[:Ts].numpy()
-        x_s = synth.bf16_bits(synth.normal_bf16(Ts, H, seed=44))
-        y_s = synth.bf16_bits(synth.normal_bf16(Ts * K, H, seed=46))
-        gw_s = gate_w[:Ts].numpy()
-        t0 = time.perf_counter()
-        reps = 0
-        while True:
-            _, cnt, _ = cam_oracle.layout(ids_s, E, 1)
-            off, _ = cam_oracle.offsets(cnt, Ts)
-            pos = cam_oracle.send_token_idx(ids_s, E)
-            cam_oracle.dispatch(x_s, ids_s, off, pos, E, 1, Ts * K)
-            row_of = cam_oracle.rows_from_pos(ids_s, off, pos, E)
-            cam_oracle.combine(y_s, row_of, gw_s)
-            reps += 1
-            el = time.perf_counter() - t0
-            if el > 12.0:
-                break
-        sample_bytes = synth.dispatch_bytes(Ts, H, K, E) + synth.combine_bytes(Ts, H, K)
-        cpu = dict(value=sample_bytes * reps / el / 1e9, unit="GB/s", cores=cam_oracle.num_threads(), kind="port",
-                   sample="%d of %d tokens of the same dispatch+combine workload (H=%d, E=%d, top-%d), %d passes in "
-                          "%.1f s, OpenMP over rows" % (Ts, T, H, E, K, reps, el))
-        log("cpu baseline: %.2f GB/s on %d threads" % (cpu["value"], cpu["cores"]))
+        ids_np = ids64.numpy()
+        x_np = synth.bf16_bits(synth.normal_bf16(T, H, seed=44))
+        y_np = synth.bf16_bits(synth.normal_bf16(A, H, seed=46))
+        gw_np = gate_w.numpy()
+
+        def cpu_step():
+            _, cnt, _ = cam_oracle.layout(ids_np, E, 1)
+            off, _ = cam_oracle.offsets(cnt, T)
+            pos = cam_oracle.send_token_idx(ids_np, E)
+            cam_oracle.dispatch(x_np, ids_np, off, pos, E, 1, A)
+            row_of = cam_oracle.rows_from_pos(ids_np, off, pos, E)
+            cam_oracle.combine(y_np, row_of, gw_np)
+
+        def cpu_time(fn, budget, min_runs=3, warm=1):
+            for _ in range(warm):
+                fn()
+            ts = []
+            t_start = time.perf_counter()
+            while len(ts) < min_runs or (time.perf_counter() - t_start < budget and len(ts) < 50):
+                t0 = time.perf_counter()
+                fn()
+                ts.append(time.perf_counter() - t0)
+            ts.sort()
+            return ts[len(ts) // 2], len(ts)
+
+        full_bytes = disp_bytes + comb_bytes
+        nthr = cam_oracle.num_threads()
+        t_mt, n_mt = cpu_time(cpu_step, 8.0, min_runs=10, warm=2)
+        cam_oracle.set_num_threads(1)
+        t_1, n_1 = cpu_time(cpu_step, 6.0, min_runs=3, warm=1)
+        cam_oracle.set_num_threads(nthr)
+        cpu = dict(value=full_bytes / t_mt / 1e9, unit="GB/s", cores=nthr, kind="port",
+                   sample="the full dispatch+combine workload (4096 tokens, H=7168, E=256, top-8; 32768 rows), median "
+                          "of %d passes after 2 warm-ups, OpenMP over rows on %d threads" % (n_mt, nthr),
+                   ms_per_step=t_mt * 1e3)
+        result["cpu_baseline_1thread"] = dict(value=full_bytes / t_1 / 1e9, unit="GB/s", cores=1, kind="port",
+                                              sample="same full workload, median of %d passes, one thread" % n_1,
+                                              ms_per_step=t_1 * 1e3)
+        log("cpu baseline: %.2f GB/s on %d threads, %.2f GB/s on one" % (cpu["value"], nthr, full_bytes / t_1 / 1e9))
+        # C1 layer (128 tokens, hidden 1024, 8 experts, top-2, intermediate 512) on the CPU
+        T1, H1, E1, K1, I1 = 128, 1024, 8, 2, 512
+        id1, g1 = synth.softmax_topk_routing(T1, E1, K1, seed=43)
+        w1c, w1sc = synth.absmax_int8_weights(E1, H1, 2 * I1, seed=431)
+        w2c, w2sc = synth.absmax_int8_weights(E1, I1, H1, seed=432)
+        x1 = synth.bf16_bits(synth.normal_bf16(T1, H1, seed=433))
+        a1 = [x1, id1.numpy(), g1.numpy(), w1c.numpy(), w1sc.numpy(), w2c.numpy(), w2sc.numpy()]
+        t_c1, n_c1 = cpu_time(lambda: cam_oracle.fused_layer(*a1), 2.0, min_runs=10, warm=2)
+        cam_oracle.set_num_threads(1)
+        t_c1s, _ = cpu_time(lambda: cam_oracle.fused_layer(*a1), 2.0, min_runs=5, warm=1)
+        cam_oracle.set_num_threads(nthr)
+        result["cpu_golden_layer_us"] = dict(threads=t_c1 * 1e6, one_thread=t_c1s * 1e6, cores=nthr, runs=n_c1,
+                                             config="128 tokens, hidden 1024, 8 experts, top-2, intermediate 512")
+        # grouped GEMM on the CPU at a reduced row count (512 rows, same hidden / intermediate / expert count)
+        if want("gemm") and not args.skip_gemm:
+            Gc, Ic, rc = 32, 2048, 512
+            szc = synth.zipf_group_sizes(Gc, rc, seed=45).numpy()
+            glc = np.cumsum(szc)
+            rng = np.random.default_rng(45)
+            ac = rng.integers(-127, 128, size=(rc, H), dtype=np.int8)
+            w1n = rng.integers(-127, 128, size=(Gc, H, 2 * Ic), dtype=np.int8)
+            t0 = time.perf_counter()
+            c_cpu = cam_oracle.gmm_int32(ac, w1n, glc)
+            t_cg = time.perf_counter() - t0
+            opsc = 2 * rc * H * 2 * Ic
+            # cross-check of the timed result against an exact float64 matmul of one expert
+            gbig = int(np.argmax(szc))
+            r0 = int(glc[gbig] - szc[gbig])
+            ref = (torch.from_numpy(ac[r0:r0 + 4].astype(np.float64)) @
+                   torch.from_numpy(w1n[gbig].astype(np.float64))).to(torch.int32).numpy()
+            assert np.array_equal(c_cpu[r0:r0 + 4], ref), "CPU GEMM cross-check failed"
+            result["cpu_gemm_reduced"] = dict(reduced=True, rows=rc, experts=Gc, hidden=H, intermediate=Ic,
+                                              what="GMM1 int32 accumulation only (gate/up projection), one pass",
+                                              seconds=t_cg, tops=opsc / t_cg / 1e12, cores=nthr)
+            log("cpu GEMM (reduced, 512 rows): %.2f s -> %.3f TOPS" % (t_cg, opsc / t_cg / 1e12))
+            del w1n, c_cpu
 
     # ------------------------------------------------------------------ the JSON line
     line = {
         "metric": "dispatch+combine HBM GB/s; w8a8 grouped GEMM TOPS; us per MoE layer",
         "unit": "GB/s",
         "n_gpus": 1,
-        "steps": args.steps,
-        "warmup": args.warmup,
+        "steps": K_STEPS,
+        "warmup": W_STEPS,
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
@@ -370,25 +529,25 @@ def main():
                         "per-token int8 quant + fp32 scales; then combine: 32768 bf16 rows x 7168 -> 4096 tokens",
             "tokens": T, "hidden": H, "experts": E, "top_k": K,
             "dispatch_bytes": disp_bytes, "combine_bytes": comb_bytes,
-            "timing": "HIP graph replays (%d passes each) bracketed by HIP events on the launch stream; %d rotating "
-                      "buffer sets" % (ROT, NBUF),
+            "timing": "one HIP graph of exactly `steps` steps (after `warmup` steps), one replay bracketed by HIP "
+                      "events on the launch stream; %d rotating buffer sets; spreads from %d replays of %d-pass graphs"
+                      % (NBUF, SPREAD_REPLAYS, ROT),
         },
     }
-    if t_disp is not None and t_comb is not None:
-        total_t = t_disp + t_comb
-        line["value"] = (disp_bytes + comb_bytes) / total_t / 1e9
-        line["ms_per_step"] = total_t * 1e3
-        line["dispatch"] = dict(us=t_disp * 1e6, gb_per_s=disp_bytes / t_disp / 1e9, frac_hbm_peak=disp_bytes / t_disp / HBM_PEAK)
-        line["combine"] = dict(us=t_comb * 1e6, gb_per_s=comb_bytes / t_comb / 1e9, frac_hbm_peak=comb_bytes / t_comb / HBM_PEAK)
-        dom = "combine_gather" if kernels["combine_gather"]["us"] >= kernels["dispatch_permute_quant"]["us"] \
-            else "dispatch_permute_quant"
+    if step_t is not None:
+        line["value"] = (disp_bytes + comb_bytes) / step_t / 1e9
+        line["ms_per_step"] = step_t * 1e3
+        line["dispatch"] = dict(us=t_disp * 1e6, gb_per_s=disp_bytes / t_disp / 1e9,
+                                frac_hbm_peak=disp_bytes / t_disp / HBM_PEAK)
+        line["combine"] = dict(us=t_comb * 1e6, gb_per_s=comb_bytes / t_comb / 1e9,
+                               frac_hbm_peak=comb_bytes / t_comb / HBM_PEAK)
+        dom = "combine_gather" if kernels["combine_gather"]["us"]["mean"] >= kernels["dispatch_fused"]["us"]["mean"] \
+            else "dispatch_fused"
         k = kernels[dom]
-        # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, each scaled by what the same
-        # counter shows for a 256 MiB device copy (x2.000 and x1.000): profiles/dispatch_combine_c2_c4.md.
-        measured_traffic = {"combine_gather": 539.0e6, "dispatch_permute_quant": 295.9e6}
+        traffic, source = recorded_traffic(dom)
         line["roofline"] = {"kernel": dom, "bound": "hbm", "achieved": k["achieved"], "peak": HBM_PEAK / 1e9,
-                            "unit": "GB/s", "frac": k["frac"], "traffic": measured_traffic[dom], "us": k["us"],
-                            "bytes": k["bytes"]}
+                            "unit": "GB/s", "frac": k["frac"], "traffic": traffic, "traffic_source": source,
+                            "us": k["us"]["mean"], "bytes": k["bytes"]}
     else:
         line["value"] = None
         line["ms_per_step"] = None

@@ -97,6 +97,16 @@ ORACLE_API int cam_oracle_num_threads(void)
 #endif
 }
 
+/* Threads used by the row-parallel loops from now on (the benchmark's single-thread CPU figure uses 1). */
+ORACLE_API void cam_oracle_set_num_threads(int n)
+{
+#ifdef _OPENMP
+    omp_set_num_threads(n < 1 ? 1 : n);
+#else
+    (void)n;
+#endif
+}
+
 ORACLE_API float cam_oracle_expf(float x) { return cam_expf_spec(x); }
 ORACLE_API float cam_oracle_silu(float x) { return cam_silu_spec(x); }
 ORACLE_API uint16_t cam_oracle_f32_to_bf16(float x) { return f32_to_bf16(x); }

@@ -56,6 +56,10 @@ def num_threads():
     return int(lib().cam_oracle_num_threads())
 
 
+def set_num_threads(n):
+    lib().cam_oracle_set_num_threads(ctypes.c_int(int(n)))
+
+
 def expf(x):
     return float(lib().cam_oracle_expf(ctypes.c_float(x)))
 

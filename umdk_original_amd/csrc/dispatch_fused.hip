@@ -9,16 +9,22 @@
 // Design.  A destination row depends on every id before it, so the plan has to be complete before the
 // first row can be placed; run as separate launches, the plan's few microseconds of latency-bound work
 // sit in front of the bandwidth-bound permute.  Here the grid has three kinds of workgroups:
-//   * workgroups [0, nb): rank one chunk of 2048 flat ids each (rank_chunk), publish the chunk's
+//   * workgroups [0, nb) first rank one chunk of 2048 flat ids each (rank_chunk), publish the chunk's
 //     per-expert histogram and the chunk-local ranks, then raise their tag;
-//   * workgroup nb, the finisher: waits for the nb tags, turns the histograms into per-(chunk, expert)
-//     bases and per-expert offsets, writes the plan's per-expert outputs, then raises the flag;
-//   * the remaining workgroups, one wavefront per token: load the token row and quantise it in
-//     registers -- none of which needs the plan -- and only then wait for the flag, compute their K
-//     destination rows (offset + chunk base + chunk-local rank) and store.
+//   * workgroup nb, the finisher, first waits for the nb tags, turns the histograms into per-(chunk,
+//     expert) bases and per-expert offsets, writes the plan's per-expert outputs, then raises the flag;
+//   * every workgroup (those above once their plan duty is done) then handles four tokens, one wavefront
+//     each: load the token row and quantise it in registers -- none of which needs the plan -- and only
+//     then wait for the flag, compute the K destination rows (offset + chunk base + chunk-local rank)
+//     and store.
 // The plan therefore runs underneath the first row loads.  Waiting is safe because workgroups are
 // started in index order: the ones being waited for never wait themselves and are resident before any
 // waiter.  Every wait is bounded; a wave that gives up raises an error word and stores nothing.
+// Everything one workgroup hands to another (histograms, chunk-local ranks, bases, offsets, tags, flag) is
+// written with device-scope write-through stores and read with device-scope loads, and a tag or flag is
+// raised only after the stores before it have completed.  A release or acquire FENCE at device scope is
+// deliberately not used: on this part it writes back, or invalidates, a whole L2, which costs several
+// microseconds per fence while the row traffic is in flight.
 // The tags and the flag live in the caller's workspace.  A launch leaves them cleared (the last token
 // workgroup to finish does it), and "raised" means "equal to a 64-bit magic number", so a workspace
 // that has never been used, whatever it holds, reads as "not raised".
@@ -38,7 +44,7 @@ constexpr int kSpinLimit = 1 << 21;                      // polls (about a secon
 
 __device__ __forceinline__ unsigned long long peek(const unsigned long long *p)
 {
-    return __hip_atomic_load(p, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_AGENT);
+    return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
 __device__ __forceinline__ int peek_i32(const int32_t *p)
@@ -50,6 +56,7 @@ __device__ __forceinline__ bool wait_raised(const unsigned long long *p)
 {
     for (int i = 0; i < kSpinLimit; ++i) {
         if (peek(p) == kRaised) {
+            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");  // orders the loads that follow; no cache action
             return true;
         }
         __builtin_amdgcn_s_sleep(16);
@@ -57,9 +64,22 @@ __device__ __forceinline__ bool wait_raised(const unsigned long long *p)
     return false;
 }
 
+__device__ __forceinline__ void poke_i32(int32_t *p, int v)
+{
+    __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// All threads: wait until this thread's write-through stores have completed, then meet at the barrier.
+__device__ __forceinline__ void stores_done_barrier()
+{
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+    __builtin_amdgcn_s_waitcnt(0);  // vmcnt(0) expcnt(0) lgkmcnt(0) on gfx9
+    __syncthreads();
+}
+
 __device__ __forceinline__ void raise(unsigned long long *p)
 {
-    __hip_atomic_store(p, kRaised, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
+    __hip_atomic_store(p, kRaised, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
 // Workspace words used by one launch (64-bit each): tags[kFusedMaxChunks], flag, finished-workgroup counter,
@@ -84,23 +104,28 @@ __global__ __launch_bounds__(kLocalThreads) void dispatch_fused_kernel(FusedDisp
     int32_t *off_ws = table + (long long)nb * E + 4;     // [E] exclusive offsets
     unsigned long long *ctrl = a.ctrl;
 
+#ifdef CAM_FUSED_PROBE
+    // Timing probes (probe builds only): 100 MHz timestamps into the padding behind the control words.
+    if (tid == 0 && b == 0) ctrl[kFusedCtrlWords + 0] = wall_clock64();
+    if (tid == 0 && b == nb + 1) ctrl[kFusedCtrlWords + 3] = wall_clock64();
+    if (tid == 0 && b == gridDim.x - 1) ctrl[kFusedCtrlWords + 6] = wall_clock64();
+#endif
     if (b < nb) {
         // ---- ranking workgroup
         const int t_active = count_active(a.p.mask, a.p.T, tid, kLocalThreads, &total_s);
-        rank_chunk<IdT, kFusedIT>((const IdT *)a.p.idx, b, (long long)t_active * K, (long long)a.p.T * K, E, hist,
-                                  a.p.pos, table + (long long)b * E);
+        rank_chunk<IdT, kFusedIT, true>((const IdT *)a.p.idx, b, (long long)t_active * K, (long long)a.p.T * K, E,
+                                        hist, a.p.pos, table + (long long)b * E);
         if (b == 0 && tid == 0) {
-            table[(long long)nb * E] = t_active;
+            poke_i32(&table[(long long)nb * E], t_active);
         }
-        __threadfence();
-        __syncthreads();
+        stores_done_barrier();
         if (tid == 0) {
             raise(&ctrl[b]);
+#ifdef CAM_FUSED_PROBE
+            if (b == 0) ctrl[kFusedCtrlWords + 1] = wall_clock64();
+#endif
         }
-        return;
-    }
-
-    if (b == nb) {
+    } else if (b == nb) {
         // ---- finisher
         bool ok = true;
         for (int j = tid; j < nb; j += kLocalThreads) {
@@ -138,13 +163,13 @@ __global__ __launch_bounds__(kLocalThreads) void dispatch_fused_kernel(FusedDisp
                     }
 #pragma unroll
                     for (int j = 0; j < 16; ++j) {
-                        col[(long long)(bb + j) * E] = run;
+                        poke_i32(&col[(long long)(bb + j) * E], run);
                         run += v[j];
                     }
                 }
                 for (; bb < nb; ++bb) {
                     const int v = peek_i32(&col[(long long)bb * E]);
-                    col[(long long)bb * E] = run;
+                    poke_i32(&col[(long long)bb * E], run);
                     run += v;
                 }
                 cnt2[h] = run;
@@ -159,7 +184,7 @@ __global__ __launch_bounds__(kLocalThreads) void dispatch_fused_kernel(FusedDisp
             const int e = 2 * tid + h;
             nt2[h] = e < E ? (cnt2[h] + kGemmTileM - 1) / kGemmTileM : 0;
             if (e < E) {
-                off_ws[e] = off2[h];
+                poke_i32(&off_ws[e], off2[h]);
                 if (a.p.cnt) a.p.cnt[e] = cnt2[h];
                 if (a.p.off) a.p.off[e] = off2[h];
                 if (a.p.recv_off) a.p.recv_off[e] = off2[h];
@@ -189,19 +214,20 @@ __global__ __launch_bounds__(kLocalThreads) void dispatch_fused_kernel(FusedDisp
             }
         }
         if (tid == 0) {
-            ctrl[kCtrlDone] = 0ull;
+            __hip_atomic_store(&ctrl[kCtrlDone], 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         }
-        __threadfence();
-        __syncthreads();
+        stores_done_barrier();
         if (tid == 0) {
             raise(&ctrl[kCtrlFlag]);
+#ifdef CAM_FUSED_PROBE
+            ctrl[kFusedCtrlWords + 2] = wall_clock64();
+#endif
         }
-        return;
     }
 
-    // ---- token workgroup: one wavefront per token
+    // ---- every workgroup, the first nb + 1 after their plan duty: one wavefront per token
     const int lane = tid & (kWave - 1);
-    const int t = (b - nb - 1) * kDispWaves + (tid >> 6);
+    const int t = b * kDispWaves + (tid >> 6);
     const bool have_token = t < a.p.T;
     TokenRow r;
     if (have_token) {
@@ -210,10 +236,17 @@ __global__ __launch_bounds__(kLocalThreads) void dispatch_fused_kernel(FusedDisp
             quant_token_row<QUANT, ACT>(r);
         }
     }
+#ifdef CAM_FUSED_PROBE
+    if (tid == 0 && b == nb + 1) ctrl[kFusedCtrlWords + 4] = wall_clock64();
+#endif
     if (tid == 0) {
         ok_s = wait_raised(&ctrl[kCtrlFlag]) ? 1 : 0;
     }
     __syncthreads();
+#ifdef CAM_FUSED_PROBE
+    if (tid == 0 && b == nb + 1) ctrl[kFusedCtrlWords + 5] = wall_clock64();
+    if (tid == 0 && b == gridDim.x - 1) ctrl[kFusedCtrlWords + 7] = wall_clock64();
+#endif
     if (ok_s == 0) {
         if (tid == 0) {
             atomicAdd(&ctrl[kCtrlErr], 1ull);
@@ -247,8 +280,12 @@ __global__ __launch_bounds__(kLocalThreads) void dispatch_fused_kernel(FusedDisp
         }
     }
     __syncthreads();
+#ifdef CAM_FUSED_PROBE
+    if (tid == 0 && b == nb + 1) ctrl[kFusedCtrlWords + 8] = wall_clock64();
+    if (tid == 0 && b == gridDim.x - 1) ctrl[kFusedCtrlWords + 9] = wall_clock64();
+#endif
     if (tid == 0) {
-        const unsigned long long token_blocks = gridDim.x - nb - 1;
+        const unsigned long long token_blocks = gridDim.x;
         if (atomicAdd(&ctrl[kCtrlDone], 1ull) == token_blocks - 1) {
             // Last one out: leave the workspace as "not raised" for the next launch that uses it.
             for (int j = 0; j < nb; ++j) {
@@ -306,7 +343,8 @@ hipError_t launch_dispatch_fused(FusedDispatchArgs a, hipStream_t stream)
     }
     const long long n_all = (long long)a.p.T * a.p.K;
     a.nb = (int)((n_all + kFusedChunk - 1) / kFusedChunk);
-    const long long blocks = (long long)a.nb + 1 + (a.p.T + kDispWaves - 1) / kDispWaves;
+    const long long token_blocks = (a.p.T + kDispWaves - 1) / kDispWaves;
+    const long long blocks = token_blocks > a.nb + 1 ? token_blocks : a.nb + 1;
     if (blocks > 0x7fffffffll) {
         return hipErrorInvalidValue;
     }
