@@ -8,6 +8,7 @@
 //   AK/moe_combine_normal/op_host/moe_combine_normal_tiling.cc:144-400
 //   AK/fused_deep_moe/op_host/fused_deep_moe_tiling.cpp:49-61,83-348
 //   src/cam/comm_operator/pybind/moe_dispatch_prefill.cpp:44-70
+#include <algorithm>
 #include <cstdarg>
 #include <cstdio>
 #include <cstring>
@@ -279,10 +280,13 @@ camStatus check_gemm_dims(const char *op, int64_t Kd, int64_t N, bool gate_up)
     return CAM_OK;
 }
 
-int max_tiles_for(int64_t rows, int64_t G) { return (int)(rows / cam::kGemmTileM + G); }
-uint64_t tile_table_bytes(int max_tiles)
+// One schedule for a GEMM of N packed columns over `rows` rows of G experts, carved out of a workspace.
+cam::SchedSpec sched_spec(int64_t rows, int64_t G, int64_t N)
 {
-    return (uint64_t)(cam::kTileHeader + cam::kTileRecord * (int64_t)max_tiles) * 4;
+    cam::SchedSpec sp{};
+    sp.N = (int)N;
+    sp.max_items = cam::sched_max_items(rows, (int)G, (int)N);
+    return sp;
 }
 
 }  // namespace
@@ -1183,9 +1187,9 @@ camStatus camGroupedMatmulSwigluQuantGetWorkspaceSize(const camTensor *x, const 
     WeightSet ws{};
     CAM_TRY(resolve_weights(weight, weightScale, "weight", gc.G, gc.Kd, 2 * I, true, &ws));
     CAM_TRY(check_aligned(y, "y", 16));
-    const int max_tiles = max_tiles_for(gc.A, gc.G);
+    cam::SchedSpec sp = sched_spec(gc.A, gc.G, 2 * I);
     Carver c;
-    const uint64_t o_tiles = c.take(tile_table_bytes(max_tiles));
+    const uint64_t o_sched = c.take(cam::sched_bytes(gc.A, (int)gc.G, (int)(2 * I)));
     const uint64_t o_prod = c.take((uint64_t)gc.A * I * 4);
     cam::GemmArgs g{};
     g.a = (const int8_t *)x->data;
@@ -1194,7 +1198,6 @@ camStatus camGroupedMatmulSwigluQuantGetWorkspaceSize(const camTensor *x, const 
     g.w_scale = ws.s;
     g.per_expert = ws.per_expert;
     g.list = ws.list;
-    g.max_tiles = max_tiles;
     g.Kd = (int)gc.Kd;
     g.N = (int)(2 * I);
     g.gate_up = 1;
@@ -1202,19 +1205,19 @@ camStatus camGroupedMatmulSwigluQuantGetWorkspaceSize(const camTensor *x, const 
     int8_t *yq = (int8_t *)y->data;
     float *ys = (float *)yScale->data;
     auto run = [=](void *wsp, hipStream_t s) mutable -> hipError_t {
-        int32_t *tiles = (int32_t *)((char *)wsp + o_tiles);
+        sp.sched = (int32_t *)((char *)wsp + o_sched);
         float *prod = (float *)((char *)wsp + o_prod);
-        hipError_t e = cam::launch_build_tiles(gc.group_list, gc.cumulative, (int)gc.G, gc.A, max_tiles, tiles, s);
+        hipError_t e = cam::launch_build_sched(gc.group_list, gc.cumulative, (int)gc.G, gc.A, 1, &sp, s);
         if (e != hipSuccess) {
             return e;
         }
-        g.tiles = tiles;
+        g.sched = sp.sched;
         g.out = prod;
         e = cam::launch_gemm(g, s);
         if (e != hipSuccess) {
             return e;
         }
-        return cam::launch_requant(prod, gc.A, (int)I, tiles, yq, ys, s);
+        return cam::launch_requant(prod, gc.A, (int)I, sp.sched, yq, ys, s);
     };
     return finish_phase1(kOpGmm1, c.off, run, workspaceSize, executor);
 }
@@ -1241,9 +1244,9 @@ camStatus camGroupedMatmulDequantGetWorkspaceSize(const camTensor *x, const camT
     CAM_TRY(check_gemm_dims("GroupedMatmulDequant", gc.Kd, N, false));
     WeightSet ws{};
     CAM_TRY(resolve_weights(weight, weightScale, "weight", gc.G, gc.Kd, N, true, &ws));
-    const int max_tiles = max_tiles_for(gc.A, gc.G);
+    cam::SchedSpec sp = sched_spec(gc.A, gc.G, N);
     Carver c;
-    const uint64_t o_tiles = c.take(tile_table_bytes(max_tiles));
+    const uint64_t o_sched = c.take(cam::sched_bytes(gc.A, (int)gc.G, (int)N));
     cam::GemmArgs g{};
     g.a = (const int8_t *)x->data;
     g.a_scale = (const float *)xScale->data;
@@ -1251,19 +1254,18 @@ camStatus camGroupedMatmulDequantGetWorkspaceSize(const camTensor *x, const camT
     g.w_scale = ws.s;
     g.per_expert = ws.per_expert;
     g.list = ws.list;
-    g.max_tiles = max_tiles;
     g.Kd = (int)gc.Kd;
     g.N = (int)N;
     g.gate_up = 0;
     g.epilogue = cam::kEpiDequantBf16;
     g.out = out->data;
     auto run = [=](void *wsp, hipStream_t s) mutable -> hipError_t {
-        int32_t *tiles = (int32_t *)((char *)wsp + o_tiles);
-        hipError_t e = cam::launch_build_tiles(gc.group_list, gc.cumulative, (int)gc.G, gc.A, max_tiles, tiles, s);
+        sp.sched = (int32_t *)((char *)wsp + o_sched);
+        hipError_t e = cam::launch_build_sched(gc.group_list, gc.cumulative, (int)gc.G, gc.A, 1, &sp, s);
         if (e != hipSuccess) {
             return e;
         }
-        g.tiles = tiles;
+        g.sched = sp.sched;
         return cam::launch_gemm(g, s);
     };
     return finish_phase1(kOpGmm2, c.off, run, workspaceSize, executor);
@@ -1290,27 +1292,26 @@ camStatus camGroupedMatmulInt32GetWorkspaceSize(const camTensor *x, const camTen
     CAM_TRY(check_gemm_dims("GroupedMatmulInt32", gc.Kd, N, gateUp != 0));
     WeightSet ws{};
     CAM_TRY(resolve_weights(weight, nullptr, "weight", gc.G, gc.Kd, N, false, &ws));
-    const int max_tiles = max_tiles_for(gc.A, gc.G);
+    cam::SchedSpec sp = sched_spec(gc.A, gc.G, N);
     Carver c;
-    const uint64_t o_tiles = c.take(tile_table_bytes(max_tiles));
+    const uint64_t o_sched = c.take(cam::sched_bytes(gc.A, (int)gc.G, (int)N));
     cam::GemmArgs g{};
     g.a = (const int8_t *)x->data;
     g.w = ws.w;
     g.per_expert = ws.per_expert;
     g.list = ws.list;
-    g.max_tiles = max_tiles;
     g.Kd = (int)gc.Kd;
     g.N = (int)N;
     g.gate_up = gateUp != 0;
     g.epilogue = cam::kEpiInt32;
     g.out = out->data;
     auto run = [=](void *wsp, hipStream_t s) mutable -> hipError_t {
-        int32_t *tiles = (int32_t *)((char *)wsp + o_tiles);
-        hipError_t e = cam::launch_build_tiles(gc.group_list, gc.cumulative, (int)gc.G, gc.A, max_tiles, tiles, s);
+        sp.sched = (int32_t *)((char *)wsp + o_sched);
+        hipError_t e = cam::launch_build_sched(gc.group_list, gc.cumulative, (int)gc.G, gc.A, 1, &sp, s);
         if (e != hipSuccess) {
             return e;
         }
-        g.tiles = tiles;
+        g.sched = sp.sched;
         return cam::launch_gemm(g, s);
     };
     return finish_phase1(kOpGmmI32, c.off, run, workspaceSize, executor);
@@ -1429,21 +1430,29 @@ camStatus camFusedDeepMoeGetWorkspaceSize(const camTensor *x, const camTensor *e
     CAM_TRY(check_aligned(output, "output", 16));
 
     const int64_t A = T * K;  // maxTokenNum of AK/fused_deep_moe/op_kernel/fused_deep_moe.h:336 for one rank
-    const int max_tiles = max_tiles_for(A, Epr);
+    cam::SchedSpec sp1 = sched_spec(A, Epr, 2 * I);
+    cam::SchedSpec sp2 = sched_spec(A, Epr, H);
     Carver c;
     const uint64_t o_pos = c.take((uint64_t)A * 4);
     const uint64_t o_row = c.take((uint64_t)A * 4);
-    const uint64_t o_tiles = c.take(tile_table_bytes(max_tiles));
+    const uint64_t o_meta = c.take(cam::kPlanMeta * 4);
+    const uint64_t o_sched1 = c.take(cam::sched_bytes(A, (int)Epr, (int)(2 * I)));
+    const uint64_t o_sched2 = c.take(cam::sched_bytes(A, (int)Epr, (int)H));
     const bool fused_dispatch = cam::fused_dispatch_fits(T, K);
     const uint64_t o_hist = c.take(fused_dispatch ? cam::fused_dispatch_table_bytes(T, K, (int)Epr)
                                                   : cam::plan_workspace_bytes(T, K, (int)Epr));
     const uint64_t o_ctrl = c.take(cam::fused_dispatch_ctrl_bytes());
-    const uint64_t o_x1 = c.take((uint64_t)A * H);
+    // The bf16 rows GMM2 writes (2*A*H bytes) live where the quantised rows (A*H) and the fp32 SwiGLU products
+    // (4*A*I) lived: both are dead once the re-quantisation has run (the reference overlays its stages the same
+    // way, AK/fused_deep_moe/op_kernel/fused_deep_moe.h:362-391).  GMM2's own input stays apart.
+    const uint64_t x1_bytes = align_up((uint64_t)A * H);
+    const uint64_t shared_bytes = std::max<uint64_t>((uint64_t)A * H * 2, x1_bytes + (uint64_t)A * I * 4);
+    const uint64_t o_x1 = c.take(shared_bytes);
+    const uint64_t o_prod = o_x1 + x1_bytes;
+    const uint64_t o_y = o_x1;
     const uint64_t o_x1s = c.take((uint64_t)A * 4);
-    const uint64_t o_prod = c.take((uint64_t)A * I * 4);
     const uint64_t o_x2 = c.take((uint64_t)A * I);
     const uint64_t o_x2s = c.take((uint64_t)A * 4);
-    const uint64_t o_y = c.take((uint64_t)A * H * 2);
 
     const uint16_t *xp = (const uint16_t *)x->data;
     const int32_t *ids = (const int32_t *)expertIds->data;
@@ -1457,7 +1466,7 @@ camStatus camFusedDeepMoeGetWorkspaceSize(const camTensor *x, const camTensor *e
         char *w = (char *)wsp;
         int32_t *pos = (int32_t *)(w + o_pos);
         int32_t *row = (int32_t *)(w + o_row);
-        int32_t *tiles = (int32_t *)(w + o_tiles);
+        int32_t *meta = (int32_t *)(w + o_meta);
         int8_t *x1 = (int8_t *)(w + o_x1);
         float *x1s = (float *)(w + o_x1s);
         float *prod = (float *)(w + o_prod);
@@ -1476,7 +1485,7 @@ camStatus camFusedDeepMoeGetWorkspaceSize(const camTensor *x, const camTensor *e
         p.pos = pos;
         p.dst_row = row;
         p.tokens_per_expert = etn;
-        p.tiles = tiles;
+        p.meta = meta;
         p.hist_ws = (int32_t *)(w + o_hist);
         hipError_t e;
         if (fused_dispatch) {
@@ -1510,6 +1519,13 @@ camStatus camFusedDeepMoeGetWorkspaceSize(const camTensor *x, const camTensor *e
             if (e != hipSuccess) return e;
         }
 
+        // both GEMM schedules from the per-expert counts the plan has just written
+        cam::SchedSpec specs[2] = {sp1, sp2};
+        specs[0].sched = (int32_t *)(w + o_sched1);
+        specs[1].sched = (int32_t *)(w + o_sched2);
+        e = cam::launch_build_sched(etn, 0, iE, A, 2, specs, s);
+        if (e != hipSuccess) return e;
+
         cam::GemmArgs g1{};
         g1.a = x1;
         g1.a_scale = x1s;
@@ -1517,8 +1533,7 @@ camStatus camFusedDeepMoeGetWorkspaceSize(const camTensor *x, const camTensor *e
         g1.w_scale = w1.s;
         g1.per_expert = w1.per_expert;
         g1.list = w1.list;
-        g1.tiles = tiles;
-        g1.max_tiles = max_tiles;
+        g1.sched = specs[0].sched;
         g1.Kd = iH;
         g1.N = 2 * iI;
         g1.gate_up = 1;
@@ -1526,7 +1541,7 @@ camStatus camFusedDeepMoeGetWorkspaceSize(const camTensor *x, const camTensor *e
         g1.out = prod;
         e = cam::launch_gemm(g1, s);
         if (e != hipSuccess) return e;
-        e = cam::launch_requant(prod, A, iI, tiles, x2, x2s, s);
+        e = cam::launch_requant(prod, A, iI, specs[0].sched, x2, x2s, s);
         if (e != hipSuccess) return e;
 
         cam::GemmArgs g2{};
@@ -1536,8 +1551,7 @@ camStatus camFusedDeepMoeGetWorkspaceSize(const camTensor *x, const camTensor *e
         g2.w_scale = w2.s;
         g2.per_expert = w2.per_expert;
         g2.list = w2.list;
-        g2.tiles = tiles;
-        g2.max_tiles = max_tiles;
+        g2.sched = specs[1].sched;
         g2.Kd = iI;
         g2.N = iH;
         g2.gate_up = 0;
@@ -1554,7 +1568,7 @@ camStatus camFusedDeepMoeGetWorkspaceSize(const camTensor *x, const camTensor *e
         cb.K = iK;
         cb.H = iH;
         cb.A = A;
-        cb.t_active = tiles + 2;
+        cb.t_active = meta + 2;
         cb.out = outp;
         return cam::launch_combine(cb, s);
     };

@@ -11,13 +11,24 @@ namespace cam {
 constexpr int kMaxExperts = 512;   // E <= 512 on every CAM operator
 constexpr int kMaxRanks = 384;
 constexpr int kMaxTopk = 16;
-constexpr int kGemmTileM = 128;    // rows per GEMM tile (tile table granularity)
 constexpr int kMaxListExperts = 64;  // per-expert weight tensors that fit in the kernel arguments
-// GEMM tile table: kTileHeader ints {tile count, total rows, active tokens, 0}, then one record of
-// kTileRecord ints per tile: {expert, first row, rows, first tile of the expert, tiles of the expert, 0, 0, 0}.
-// Tiles are listed in expert order; the rows of an expert are split evenly over its tiles.
-constexpr int kTileHeader = 4;
-constexpr int kTileRecord = 8;
+// GEMM schedule (device-built, one per GEMM launch): kSchedHeader ints, then the work items.
+//   [0] item count  [1] total rows  [2], [3] 0
+//   [kSchedQueueStart .. +8]  first item of each of the 8 queues, and the end of the last
+//   [kSchedQueueCount + 32 x] items already taken from queue x (zeroed by the builder, advanced by the GEMM);
+//                             one counter per 128-byte line, so that the queues do not share a line
+constexpr int kSchedHeader = 32 + 8 * 32;
+constexpr int kSchedQueueStart = 4;
+constexpr int kSchedQueueCount = 32;
+constexpr int kSchedQueueStride = 32;
+// One work item: rows [m0, m0 + rows) of expert g times column block nb.  flat != 0: at most 128 rows x 512
+// packed columns, the two wave teams split the columns; flat == 0: at most 256 rows x 256 packed columns, team
+// 0 takes tile rows [0, split), team 1 the rest.
+struct SchedItem {
+    int32_t g, m0, rows, split, nb, flat, pad0, pad1;
+};
+// Run metadata the plan kernels leave for the kernels after them: {0, total rows, active tokens, 0}.
+constexpr int kPlanMeta = 4;
 
 // ---------------------------------------------------------------------------------------------
 // Routing plan: counts, offsets, within-expert ranks, receive bookkeeping, GEMM tile table.
@@ -37,7 +48,7 @@ struct PlanArgs {
     int64_t *total;           // [1]    optional
     int32_t *per_rank_zero;   // [R]    optional: zeroed here so a later kernel can accumulate into it
     int R;
-    int32_t *tiles;           // optional GEMM tile table (layout: kTileHeader / kTileRecord below)
+    int32_t *meta;            // optional run metadata, kPlanMeta ints (see above)
     int32_t *hist_ws;         // required scratch of plan_workspace_bytes(T, K, E) bytes
 };
 uint64_t plan_workspace_bytes(int64_t T, int64_t K, int E);
@@ -60,9 +71,17 @@ hipError_t launch_in_rank(const InRankArgs &a, hipStream_t stream);
 hipError_t launch_notify_scan(const int32_t *cnt, int E, int num_tokens, int32_t *off, int32_t *send_data,
                               int32_t *recv_data, hipStream_t stream);
 
-// Tile table from a group list (cumulative or per-expert counts, int64).
-hipError_t launch_build_tiles(const int64_t *group_list, int cumulative, int G, int64_t max_rows, int max_tiles,
-                              int32_t *tiles, hipStream_t stream);
+// GEMM schedules from a group list (cumulative or per-expert counts, int64): one launch builds the schedule of
+// one or two GEMMs over the same rows (they differ in the number of weight columns).
+struct SchedSpec {
+    int N;             // packed weight columns of the GEMM
+    int max_items;     // capacity of the item table (sched_max_items)
+    int32_t *sched;    // sched_bytes() of device memory
+};
+int sched_max_items(int64_t max_rows, int G, int N);
+uint64_t sched_bytes(int64_t max_rows, int G, int N);
+hipError_t launch_build_sched(const int64_t *group_list, int cumulative, int G, int64_t max_rows, int nspec,
+                              const SchedSpec *specs, hipStream_t stream);
 
 // ---------------------------------------------------------------------------------------------
 // Permute (+ per-token int8 quantisation).
@@ -138,8 +157,7 @@ struct GemmArgs {
     const float *w_scale;  // stacked [G,N]
     int per_expert;        // weights given per expert through `list`
     WeightPtrs list;
-    const int32_t *tiles;  // tile table
-    int max_tiles;         // upper bound on the number of tiles (grid size)
+    int32_t *sched;        // schedule built for this launch (its queue counters are consumed by the launch)
     int Kd, N;             // N = logical columns of the weight
     int gate_up;           // weight prepacked with gate/up pairing
     int epilogue;
@@ -147,8 +165,9 @@ struct GemmArgs {
 };
 hipError_t launch_gemm(const GemmArgs &a, hipStream_t stream);
 
-// fp32 SwiGLU products [rows,I] -> int8 + per-row scale.  rows_dev: optional device count of valid rows.
-hipError_t launch_requant(const float *y, int64_t max_rows, int I, const int32_t *tiles_for_rows, int8_t *q,
+// fp32 SwiGLU products [rows,I] -> int8 + per-row scale.  sched_for_rows: optional schedule whose header holds
+// the number of valid rows.
+hipError_t launch_requant(const float *y, int64_t max_rows, int I, const int32_t *sched_for_rows, int8_t *q,
                           float *scale, hipStream_t stream);
 
 hipError_t launch_prepack(const int8_t *src, int8_t *dst, int G, int Kd, int N, int gate_up, hipStream_t stream);

@@ -104,12 +104,6 @@ __global__ __launch_bounds__(kLocalThreads) void dispatch_fused_kernel(FusedDisp
     int32_t *off_ws = table + (long long)nb * E + 4;     // [E] exclusive offsets
     unsigned long long *ctrl = a.ctrl;
 
-#ifdef CAM_FUSED_PROBE
-    // Timing probes (probe builds only): 100 MHz timestamps into the padding behind the control words.
-    if (tid == 0 && b == 0) ctrl[kFusedCtrlWords + 0] = wall_clock64();
-    if (tid == 0 && b == nb + 1) ctrl[kFusedCtrlWords + 3] = wall_clock64();
-    if (tid == 0 && b == gridDim.x - 1) ctrl[kFusedCtrlWords + 6] = wall_clock64();
-#endif
     if (b < nb) {
         // ---- ranking workgroup
         const int t_active = count_active(a.p.mask, a.p.T, tid, kLocalThreads, &total_s);
@@ -121,9 +115,6 @@ __global__ __launch_bounds__(kLocalThreads) void dispatch_fused_kernel(FusedDisp
         stores_done_barrier();
         if (tid == 0) {
             raise(&ctrl[b]);
-#ifdef CAM_FUSED_PROBE
-            if (b == 0) ctrl[kFusedCtrlWords + 1] = wall_clock64();
-#endif
         }
     } else if (b == nb) {
         // ---- finisher
@@ -178,11 +169,9 @@ __global__ __launch_bounds__(kLocalThreads) void dispatch_fused_kernel(FusedDisp
         const int pair_off = block_exclusive_scan<kLocalWaves>(cnt2[0] + cnt2[1], tid, scan_s, &total_s);
         const int total = total_s;
         const int off2[2] = {pair_off, pair_off + cnt2[0]};
-        int nt2[2];
 #pragma unroll
         for (int h = 0; h < 2; ++h) {
             const int e = 2 * tid + h;
-            nt2[h] = e < E ? (cnt2[h] + kGemmTileM - 1) / kGemmTileM : 0;
             if (e < E) {
                 poke_i32(&off_ws[e], off2[h]);
                 if (a.p.cnt) a.p.cnt[e] = cnt2[h];
@@ -196,22 +185,11 @@ __global__ __launch_bounds__(kLocalThreads) void dispatch_fused_kernel(FusedDisp
         if (tid == 0 && a.p.total) {
             a.p.total[0] = total;
         }
-        if (a.p.tiles != nullptr) {
-            const int pair_tbase = block_exclusive_scan<kLocalWaves>(nt2[0] + nt2[1], tid, scan_s, &total_s);
-            const int tbase2[2] = {pair_tbase, pair_tbase + nt2[0]};
-#pragma unroll
-            for (int h = 0; h < 2; ++h) {
-                const int e = 2 * tid + h;
-                if (e < E) {
-                    write_tile_records(a.p.tiles, e, off2[h], cnt2[h], tbase2[h], nt2[h], 0x7fffffff);
-                }
-            }
-            if (tid == 0) {
-                a.p.tiles[0] = total_s;
-                a.p.tiles[1] = total;
-                a.p.tiles[2] = t_active;
-                a.p.tiles[3] = 0;
-            }
+        if (tid == 0 && a.p.meta != nullptr) {
+            a.p.meta[0] = 0;
+            a.p.meta[1] = total;
+            a.p.meta[2] = t_active;
+            a.p.meta[3] = 0;
         }
         if (tid == 0) {
             __hip_atomic_store(&ctrl[kCtrlDone], 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -219,9 +197,6 @@ __global__ __launch_bounds__(kLocalThreads) void dispatch_fused_kernel(FusedDisp
         stores_done_barrier();
         if (tid == 0) {
             raise(&ctrl[kCtrlFlag]);
-#ifdef CAM_FUSED_PROBE
-            ctrl[kFusedCtrlWords + 2] = wall_clock64();
-#endif
         }
     }
 
@@ -236,17 +211,10 @@ __global__ __launch_bounds__(kLocalThreads) void dispatch_fused_kernel(FusedDisp
             quant_token_row<QUANT, ACT>(r);
         }
     }
-#ifdef CAM_FUSED_PROBE
-    if (tid == 0 && b == nb + 1) ctrl[kFusedCtrlWords + 4] = wall_clock64();
-#endif
     if (tid == 0) {
         ok_s = wait_raised(&ctrl[kCtrlFlag]) ? 1 : 0;
     }
     __syncthreads();
-#ifdef CAM_FUSED_PROBE
-    if (tid == 0 && b == nb + 1) ctrl[kFusedCtrlWords + 5] = wall_clock64();
-    if (tid == 0 && b == gridDim.x - 1) ctrl[kFusedCtrlWords + 7] = wall_clock64();
-#endif
     if (ok_s == 0) {
         if (tid == 0) {
             atomicAdd(&ctrl[kCtrlErr], 1ull);
@@ -280,10 +248,6 @@ __global__ __launch_bounds__(kLocalThreads) void dispatch_fused_kernel(FusedDisp
         }
     }
     __syncthreads();
-#ifdef CAM_FUSED_PROBE
-    if (tid == 0 && b == nb + 1) ctrl[kFusedCtrlWords + 8] = wall_clock64();
-    if (tid == 0 && b == gridDim.x - 1) ctrl[kFusedCtrlWords + 9] = wall_clock64();
-#endif
     if (tid == 0) {
         const unsigned long long token_blocks = gridDim.x;
         if (atomicAdd(&ctrl[kCtrlDone], 1ull) == token_blocks - 1) {

@@ -9,60 +9,60 @@
 //   GMM2 epilogue   FDM/epilogue/block/block_epilogue_per_token_dequant.hpp:665-684
 //
 // Design (not a translation of the cube/vector split above).
-//   * One workgroup = 4 waves = a tile of up to 128 rows of ONE expert x 256 packed weight columns.
-//     Every wave covers all rows of the tile and its own 64 columns (128 int32 accumulators per lane),
-//     and two workgroups share a CU so that one runs MFMAs while the other waits on memory or
-//     writes its epilogue.  The grouped shape is bound by streaming the weights: a tall tile makes
-//     every weight byte fetched feed up to 128 rows, and sibling tiles of one expert are scheduled
-//     next to each other so that they find the same weight panel in L2.
+//   * Persistent kernel, one workgroup of 8 waves per CU.  Work items (one row tile of ONE expert x one
+//     block of packed weight columns) come from eight device-built queues, one per XCD; a workgroup
+//     takes items from the queue of the XCD it runs on and helps the other queues when its own is empty.
+//     The row tiles of an expert that read the same weight columns sit next to each other in one queue,
+//     so the CUs working on them share one L2, and the queues list big experts first, which leaves the
+//     small items for the end, where they even out the finishing times.
+//   * Two tile shapes.  Tall tiles (129..256 rows) x 256 columns: the two teams of four waves split the
+//     rows, every wave owns 64 columns.  Flat tiles (<= 128 rows) x 512 columns: the teams split the
+//     columns, so that the weights, which is all such an expert streams from HBM, feed every wave and
+//     twice as many weight bytes are in flight per CU.  A wave always owns up to 128 rows x 64 columns
+//     (up to 128 int32 accumulators per lane), in 32-row fragments; the fragment count is a template
+//     parameter, so the main loop has no control flow.
 //   * Both operands travel global -> LDS with direct-to-LDS loads (16 bytes per lane, no registers),
-//     three stages deep, two 64-deep K steps ahead of the MFMAs.  Weights were laid out once by the
-//     prepack kernel in the lane order the MFMA wants, so a wave's weight load is 1 KB of contiguous
-//     memory that lands in LDS already in fragment order.  Activation rows are placed with an XOR
-//     swizzle of their 16-byte chunks (chosen on the global side, since a direct-to-LDS load writes
-//     lane i at base + 16*i), which makes the ds_read_b128 fragment reads bank-conflict free.
-//   * The loads are issued from inline assembly and the pipeline's waits are written out by hand.
-//     Left to itself the compiler drains every outstanding load at each workgroup barrier and before
-//     LDS reads it cannot prove independent, which serialises the pipeline.
+//     four (tall) or three (flat) stages of 64 K-bytes each, up to a whole ring ahead of the MFMAs: the
+//     fragments of a stage are read into registers one phase before they are multiplied, which frees the
+//     stage for the next load at once.  Weights were laid out once by the prepack kernel in the lane
+//     order the MFMA wants; activation rows are placed with an XOR swizzle of their 16-byte chunks
+//     (chosen on the global side, since a direct-to-LDS load writes lane i at base + 16*i), which makes
+//     the ds_read_b128 fragment reads bank-conflict free.
+//   * Ping-pong.  Every sub-step has two phases separated by workgroup barriers.  In the first, team 0
+//     issues nothing but its 16 MFMAs while team 1 reads its fragments and issues its loads; in the
+//     second they swap.  A SIMD holds one wave of each team, so its matrix pipe always has a wave that
+//     does nothing else.  Loads are addressed by a scalar base plus a per-lane 32-bit offset computed
+//     once per item: vector ALU work in the load path would queue behind the other wave's MFMAs (64-bit
+//     vector address arithmetic per load made the issue of eight loads take 2.3x as long).
+//   * The loads are issued from inline assembly and the waits are written out by hand: left to itself
+//     the compiler drains every outstanding load at each barrier and before LDS reads it cannot prove
+//     independent, which serialises the pipeline.
 //   * The int32 accumulators stay in registers through the epilogue: dequantisation, SiLU and the
 //     gate*up product are applied in place; the int32 tile never goes to memory.  The MFMAs take the
 //     weights as their first operand, so a lane ends up with ONE activation row and runs of four
-//     consecutive weight columns: one row scale per lane, column scales as 16-byte vectors, 8- or
-//     16-byte pieces into the LDS staging from which whole 128-byte lines are stored.
-//     For GMM1 the prepack pairs gate column c with up column I+c inside one wave.
-//   * Variable rows per expert: a device-built tile table lists, per tile, (expert, first row, rows,
-//     first tile of the expert, tiles of the expert); an expert's rows are split evenly over its
-//     tiles and empty experts own no tile.  The grid is sized for the worst case and surplus
-//     workgroups exit at once.  Work ids are dealt to the 8 XCDs in contiguous runs, tile index
-//     fastest inside an expert, so that the workgroups reading one weight panel run together on one
-//     XCD and share its L2; all workgroups of an expert start their K loop at the same step (which
-//     differs from expert to expert), so that they also find each other's activation rows there.
+//     consecutive weight columns: one row scale per lane, column scales as 16-byte vectors, and each
+//     32-row fragment passes through a small LDS staging slice from which whole 128-byte lines are
+//     stored.  For GMM1 the prepack pairs gate column c with up column I+c inside one wave.
 //   * The K order inside a 32-deep MFMA step is whatever the two operands agree on (an integer dot
 //     product does not care), which is what lets both be loaded as plain 16-byte pieces.
 #include "cam_device.h"
 #include "cam_kernels.h"
+#include "rank_device.h"
 #include "../../include/cam_expf_spec.h"
 
 namespace cam {
 
 namespace {
 
-constexpr int kBM = kGemmTileM;  // rows per tile
-constexpr int kNF = 2;           // 2 column fragments per wave (64 columns)
-constexpr int kBK = 64;          // K bytes per pipeline step
-constexpr int kKK = kBK / 32;    // MFMA sub-steps per step
-constexpr int kThreads = 256;
-constexpr int kWaveCols = 64;
-constexpr int kBlockCols = 4 * kWaveCols;
+constexpr int kBK = 64;                         // K bytes per sub-step
+constexpr int kThreads = 512;                   // two teams of four waves
 constexpr int kNumXcd = 8;
-constexpr int kStages = 3;
-constexpr int kStageA = kBM * kBK;                    // 8 KB of activations per stage
-constexpr int kStageB = 4 * kWaveCols * kBK;          // 16 KB of weights per stage (4 KB per wave)
-constexpr int kStageBytes = kStageA + kStageB;
-constexpr int kBLoads = kKK * kNF;                    // weight loads per wave and step
-constexpr int kEpiRowBytes = 144;                     // epilogue staging: 128 data bytes + 16 of padding per row
-constexpr int kLdsBytes = kStages * kStageBytes > 4 * kBM * kEpiRowBytes ? kStages * kStageBytes
-                                                                         : 4 * kBM * kEpiRowBytes;
+constexpr int kMaxStages = 4;
+constexpr int kStageTall = 256 * kBK + 256 * kBK;   // 16 KB of activations + 16 KB of weights
+constexpr int kStageFlat = 128 * kBK + 512 * kBK;   //  8 KB of activations + 32 KB of weights
+constexpr int kLdsBytes = kMaxStages * kStageTall;  // 128 KB (flat: 3 x 40 KB = 120 KB)
+constexpr int kEpiRowBytes = 144;               // epilogue staging: 128 data bytes + 16 of padding per row
+constexpr int kEpiSlice = 32 * kEpiRowBytes;    // one 32-row fragment per wave
 
 // LDS offset (bytes) inside a stage of the 16-byte chunk `c` (0..3) of activation row `r`.
 __device__ __forceinline__ int a_lds_offset(int r, int c)
@@ -70,11 +70,13 @@ __device__ __forceinline__ int a_lds_offset(int r, int c)
     return r * kBK + ((c ^ ((r >> 2) & 3)) << 4);
 }
 
-// One direct-to-LDS load: lane i of the wave fetches 16 bytes at its own global address `g` and the
-// data lands at LDS byte address lds_base + 16*i.
-__device__ __forceinline__ void dma16(const void *g, unsigned lds_base)
+// One direct-to-LDS load: lane i of the wave fetches 16 bytes at base + voff(i) and the data lands at LDS byte
+// address lds_addr + 16*i.  The base is a scalar register pair, so issuing the load needs no vector ALU work.
+__device__ __forceinline__ void dma16(const void *base, unsigned voff, unsigned lds_addr)
 {
-    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(lds_base), "v"(g)
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+                 :
+                 : "s"(lds_addr), "v"(voff), "s"((unsigned long long)base)
                  : "memory", "m0");
 }
 
@@ -82,6 +84,11 @@ template <int N>
 __device__ __forceinline__ void wait_loads_outstanding()
 {
     asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
+}
+
+__device__ __forceinline__ void wait_lds_reads()
+{
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
 }
 
 // Workgroup barrier without the memory fence of __syncthreads(); the waits are explicit (above).
@@ -92,33 +99,41 @@ __device__ __forceinline__ void barrier_no_fence()
     asm volatile("" ::: "memory");
 }
 
-struct TileCtx {
+// What a wave needs to know about the item it works on (all wave-uniform).
+struct ItemCtx {
     const int8_t *a_tile;   // first activation row of the tile
-    const int8_t *wp;       // this wave's weight stream (+ 16 * lane)
-    const float *sg;        // this expert's per-channel scales
-    int m0, rows, nw, Kd, N;
-    int k_start;            // first K step of this workgroup (the K loop wraps around)
-    bool wave_live;
+    const int8_t *wg;       // the expert's packed weights
+    const float *sg;        // the expert's per-channel scales
+    int m0, rows;           // first row and rows of the tile
+    int a_row0, my_rows;    // first tile row of this wave's fragments, rows of them that exist
+    int bslot;              // this wave's 64-column group inside the stage
+    int nw;                 // this wave's packed 64-column group of the weight (clamped to a valid one)
+    bool wave_live;         // the group exists (ragged last column block)
+    int stage_a, stage_bytes;
+    int Kd, N;
 };
 
-// The whole tile for a compile-time number of 32-row fragments, so that the main loop is branch-free.
-template <int EPI, int MF>
-__device__ __forceinline__ void gemm_tile(const GemmArgs &a, const TileCtx &t, int8_t *lds, const float *row_scale_s)
+// One wave's part of one item.  TEAM 0 multiplies in the first phase of every sub-step, TEAM 1 in the second.
+// FLAT selects the tile shape (it fixes the loads per wave and sub-step); MF is the wave's fragment count.
+template <int MF, int TEAM, bool FLAT>
+__device__ __forceinline__ void run_item(const GemmArgs &a, const ItemCtx &t, int nb, int8_t *lds,
+                                         const float *row_scale_s)
 {
-    constexpr int AI = (MF + 1) / 2;           // activation loads per wave and step (1 KB each)
-    constexpr int PER_STEP = AI + kBLoads;     // loads per wave and step
+    constexpr int NS = FLAT ? 3 : 4;                       // ring of stages
+    constexpr int LPS = FLAT ? (TEAM == 0 ? 6 : 4) : 4;    // loads per wave and sub-step
+    constexpr int MFR = MF > 0 ? MF : 1;
     const int tid = threadIdx.x;
     const int lane = tid & (kWave - 1);
-    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wn = __builtin_amdgcn_readfirstlane((tid >> 6) & 3);
     const int KT = t.Kd / kBK;
     const int last = KT - 1;
     const unsigned lds0 = (unsigned)(unsigned long long)(__attribute__((address_space(3))) int8_t *)lds;
 
-    v16i acc[MF][kNF];
+    v16i acc[MFR][2];
 #pragma unroll
-    for (int mf = 0; mf < MF; ++mf) {
+    for (int mf = 0; mf < MFR; ++mf) {
 #pragma unroll
-        for (int nf = 0; nf < kNF; ++nf) {
+        for (int nf = 0; nf < 2; ++nf) {
 #pragma unroll
             for (int i = 0; i < 16; ++i) {
                 acc[mf][nf][i] = 0;
@@ -126,295 +141,622 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs &a, const TileCtx &t, i
         }
     }
 
-    // Per-lane source addresses of the activation loads (they advance by kBK per step).
-    // Load j of wave w fills the 64-byte LDS rows 16q .. 16q+15 with q = 4j + w (q = w & 1 for a
-    // single-fragment tile, where waves 2 and 3 repeat the loads of waves 0 and 1); lane i brings row
-    // 16q + i/4, and the chunk whose swizzled slot is i%4.  Rows inside the last fragment but beyond
-    // the tile repeat its last row (their results are dropped in the epilogue).
-    const int8_t *a_src[AI];
-    unsigned a_dst[AI];
+    // ---- loads.  Tall: team 0 brings the activations (wave wn: tile rows 64wn .. 64wn+63, four loads of 16
+    // rows), team 1 the weights (wave wn: the 4 KB of column group wn).  Flat: team 0 brings the activations
+    // (wave wn: rows 32wn .. 32wn+31) and column groups 0..3, team 1 column groups 4..7.  Lane i of an
+    // activation load brings row (i / 4) of its 16 and the chunk whose swizzled slot is i % 4; rows beyond the
+    // tile repeat its last row (their results are dropped in the epilogue).
+    constexpr int NA = FLAT ? (TEAM == 0 ? 2 : 0) : (TEAM == 0 ? 4 : 0);
+    constexpr int NB = LPS - NA;
+    unsigned a_voff[NA > 0 ? NA : 1];
+    unsigned a_dst[NA > 0 ? NA : 1];
 #pragma unroll
-    for (int j = 0; j < AI; ++j) {
-        const int q = MF >= 2 ? j * 4 + wave : (wave & 1);  // MF == 3: loads 6, 7 bring rows of a fourth, unused fragment
-        const int r = 16 * q + (lane >> 2);
+    for (int j = 0; j < NA; ++j) {
+        const int r0 = (FLAT ? 32 : 64) * wn + 16 * j;
+        const int r = r0 + (lane >> 2);
         const int c = (lane & 3) ^ ((r >> 2) & 3);
-        a_src[j] = t.a_tile + (long long)min(r, t.rows - 1) * t.Kd + c * 16;
-        a_dst[j] = (unsigned)(q * 1024);
+        a_voff[j] = (unsigned)(min(r, t.rows - 1) * t.Kd + c * 16);
+        a_dst[j] = (unsigned)(r0 * kBK);
     }
-    const unsigned b_dst = (unsigned)(kStageA + wave * (kWaveCols * kBK));
+    const int ngroups = t.N / 64;
+    const int bgroup = FLAT ? TEAM * 4 + wn : wn;  // the column group of the stage this wave loads
+    const int nw_load = min(nb * (FLAT ? 8 : 4) + bgroup, ngroups - 1);
+    const int8_t *b_base = t.wg + (long long)nw_load * t.Kd * 64;
+    const unsigned b_voff = (unsigned)(lane * 16);
+    const unsigned b_dst = (unsigned)(t.stage_a + bgroup * 4096);
 
-    // Step s of the pipeline reads K step (k_start + s) mod KT: an integer dot product does not care
-    // about the order, and workgroups that start at different depths do not all pull on the same
-    // memory channels at the same moment (their weight streams lie a fixed stride apart).
-    // Issues the loads of pipeline step s_idx whose index i (activation loads first, then the weight
-    // loads) satisfies i % nparts == part.
-    auto issue_part = [&](int s_idx, int stage, int part, int nparts) {
-        int step = t.k_start + s_idx;
-        step = step >= KT ? step - KT : step;
-        const unsigned sbase = lds0 + (unsigned)(stage * kStageBytes);
+    auto issue = [&](int s_idx, int slot) {
+        const int s = min(s_idx, last);
+        const unsigned sbase = lds0 + (unsigned)(slot * t.stage_bytes);
+        if (NA > 0) {
+            const int8_t *ab = t.a_tile + (long long)s * kBK;
 #pragma unroll
-        for (int j = 0; j < AI; ++j) {
-            if (j % nparts == part) {
-                dma16(a_src[j] + (long long)step * kBK, sbase + a_dst[j]);
+            for (int j = 0; j < NA; ++j) {
+                dma16(ab, a_voff[j], sbase + a_dst[j]);
             }
         }
-        const int8_t *bp = t.wp + (long long)step * (kBLoads * kWave * 16);
+        if (NB > 0) {
+            const int8_t *bb = b_base + (long long)s * 4096;
 #pragma unroll
-        for (int i = 0; i < kBLoads; ++i) {
-            if ((AI + i) % nparts == part) {
-                dma16(bp + i * (kWave * 16), sbase + b_dst + (unsigned)(i * 1024));
+            for (int j = 0; j < NB; ++j) {
+                dma16(bb + j * 1024, b_voff, sbase + b_dst + j * 1024);
             }
         }
     };
-    auto issue = [&](int s_idx, int stage) { issue_part(s_idx, stage, 0, 1); };
 
+    // ---- fragments: read from LDS one phase before they are multiplied.
+    v4i af[2][MFR];
+    v4i bf[2][2];
     const int a_row = lane & 31;
     const int a_half = lane >> 5;
-    constexpr int HF = MF == 4 ? 2 : MF;        // fragments per half
-    constexpr int NH = MF / HF;                 // halves per sub-step
-
-    // Multiplies one stage.  Fragment reads run one half sub-step ahead of the MFMAs that use them.
-    // The loads of the step two ahead are issued from inside the phases, a few at a time between the
-    // MFMA groups: a wave that issued them all at once would sit at the memory pipe's input while it
-    // drains, with its MFMAs waiting behind the loads in program order.
-    auto compute = [&](const int8_t *stage, int next_idx, int next_stage) {
-        const int8_t *sa = stage;
-        const int8_t *sb = stage + kStageA + wave * (kWaveCols * kBK) + lane * 16;
-        v4i af[2][HF];
-        v4i bf[kKK][kNF];
-        auto load_frags = [&](v4i *dst, int kk, int half) {
+    auto read_frags = [&](int slot) {
+        const int8_t *st = lds + slot * t.stage_bytes;
+        const int8_t *sb = st + t.stage_a + t.bslot * 4096 + lane * 16;
 #pragma unroll
-            for (int f = 0; f < HF; ++f) {
-                dst[f] = *(const v4i *)(sa + a_lds_offset((half * HF + f) * 32 + a_row, kk * 2 + a_half));
+        for (int kk = 0; kk < 2; ++kk) {
+#pragma unroll
+            for (int nf = 0; nf < 2; ++nf) {
+                bf[kk][nf] = *(const v4i *)(sb + (kk * 2 + nf) * 1024);
             }
-        };
 #pragma unroll
-        for (int kk = 0; kk < kKK; ++kk) {
-#pragma unroll
-            for (int nf = 0; nf < kNF; ++nf) {
-                bf[kk][nf] = *(const v4i *)(sb + (kk * kNF + nf) * 1024);
+            for (int mf = 0; mf < MF; ++mf) {
+                af[kk][mf] = *(const v4i *)(st + a_lds_offset(t.a_row0 + mf * 32 + a_row, kk * 2 + a_half));
             }
-        }
-        load_frags(af[0], 0, 0);
-#pragma unroll
-        for (int q = 0; q < kKK * NH; ++q) {
-            const int kk = q / NH;
-            const int half = q % NH;
-            if (q + 1 < kKK * NH) {
-                load_frags(af[(q + 1) & 1], (q + 1) / NH, (q + 1) % NH);
-            }
-            // Keep the LDS reads of the next half ahead of this half's MFMAs: the scheduler would
-            // otherwise sink them to just before their first use and expose the LDS latency.
-            __builtin_amdgcn_sched_barrier(0);
-            issue_part(next_idx, next_stage, q, kKK * NH);
-            __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-            for (int f = 0; f < HF; ++f) {
-#pragma unroll
-                for (int nf = 0; nf < kNF; ++nf) {
-                    // Weights as the first operand: the result tile comes out transposed, i.e. a lane
-                    // holds ONE activation row and 4 consecutive weight columns per register quad.
-                    acc[half * HF + f][nf] = __builtin_amdgcn_mfma_i32_32x32x32_i8(bf[kk][nf], af[q & 1][f],
-                                                                                   acc[half * HF + f][nf], 0, 0, 0);
-                }
-            }
-            __builtin_amdgcn_sched_barrier(0);
         }
     };
-
-    // Pipeline.  Every step issues exactly PER_STEP loads per wave and loads retire in order, so "at
-    // most (kStages-2)*PER_STEP outstanding" means that this wave's part of the current step has
-    // landed; the barrier then makes every wave's part visible and also guarantees that all waves
-    // are done reading the previous stage, which the loads issued next overwrite.  Step indices past
-    // the end are clamped (the last step is fetched again), so the loop body has no control flow.
+    auto multiply = [&]() {
+        __builtin_amdgcn_sched_barrier(0);
+        __builtin_amdgcn_s_setprio(2);
 #pragma unroll
-    for (int p = 0; p < kStages - 1; ++p) {
-        issue(min(p, last), p);
+        for (int kk = 0; kk < 2; ++kk) {
+#pragma unroll
+            for (int mf = 0; mf < MF; ++mf) {
+#pragma unroll
+                for (int nf = 0; nf < 2; ++nf) {
+                    // Weights as the first operand: the result tile comes out transposed, i.e. a lane holds ONE
+                    // activation row and 4 consecutive weight columns per register quad.
+                    acc[mf][nf] = __builtin_amdgcn_mfma_i32_32x32x32_i8(bf[kk][nf], af[kk][mf], acc[mf][nf], 0, 0, 0);
+                }
+            }
+        }
+        __builtin_amdgcn_s_setprio(0);
+        __builtin_amdgcn_sched_barrier(0);
+    };
+
+    // ---- pipeline.  Loads retire in order and every sub-step issues exactly LPS loads per wave, so "at most
+    // n * LPS outstanding" says which sub-steps of this wave's loads have landed; the barrier after the wait
+    // makes that true for the whole workgroup.  Sub-step indices past the end are clamped (the last sub-step
+    // is fetched again into a stage nobody reads), so the loop body has no control flow.
+    //   barrier A(s): every load of stage s+1 has landed; team 1 is done reading stage s
+    //   barrier B(s): team 0 is done reading stage s+1
+    // Stage s is free once both teams have its fragments in registers, i.e. after barrier A(s): team 0 refills
+    // it in the phase that follows, team 1 at the end of its own reading phase.
+#pragma unroll
+    for (int p = 0; p < NS; ++p) {
+        issue(p, p);
     }
-    for (int kt = 0; kt < KT; ++kt) {
-        wait_loads_outstanding<(kStages - 2) * PER_STEP>();
-        barrier_no_fence();
-        compute(lds + (kt % kStages) * kStageBytes, min(kt + kStages - 1, last), (kt + kStages - 1) % kStages);
+    wait_loads_outstanding<(NS - 1) * LPS>();
+    barrier_no_fence();  // stage 0 has landed
+    int slot = 0;        // slot of stage s
+    if (TEAM == 0) {
+        read_frags(0);
+        wait_lds_reads();
+        for (int s = 0; s < KT; ++s) {
+            const int next = slot + 1 == NS ? 0 : slot + 1;
+            multiply();                                   // phase 1: stage s, from registers
+            wait_loads_outstanding<(NS - 2) * LPS>();     // my part of stage s+1 has landed
+            barrier_no_fence();                           // A(s)
+            issue(s + NS, slot);                          // phase 2: refill stage s's slot ...
+            read_frags(next);                             // ... and fetch the fragments of stage s+1
+            wait_lds_reads();
+            barrier_no_fence();                           // B(s)
+            slot = next;
+        }
+    } else {
+        for (int s = 0; s < KT; ++s) {
+            const int next = slot + 1 == NS ? 0 : slot + 1;
+            read_frags(slot);                             // phase 1: fragments of stage s ...
+            wait_lds_reads();
+            issue(s + NS, slot);                          // ... then refill its slot
+            wait_loads_outstanding<(NS - 1) * LPS>();     // my part of stage s+1 has landed
+            barrier_no_fence();                           // A(s)
+            multiply();                                   // phase 2: stage s
+            barrier_no_fence();                           // B(s)
+            slot = next;
+        }
     }
     wait_loads_outstanding<0>();
+    barrier_no_fence();  // nobody reads or fills the stages any more: the epilogue may stage through them
 
     // ---- epilogue, accumulators in registers.
     // Lane l holds activation row (l & 31) of each 32x32 fragment; registers 4j .. 4j+3 hold the four
-    // consecutive weight columns 8j + 4*(l/32) + 0..3.  Dequantisation runs on that layout with one
-    // row scale per lane and fragment and the column scales fetched as 16-byte vectors.  To store
-    // whole 128-byte lines, every wave passes its results through its own slice of LDS (the pipeline
-    // stages are free by now): 128 staged bytes per row, then 16 bytes per lane and 8 rows per store.
-    barrier_no_fence();  // all waves are done with the pipeline stages
-    if (!t.wave_live) {
-        return;
-    }
-    const int rows = t.rows;
-    const int m0 = t.m0;
-    const int N = t.N;
-    const int nw = t.nw;
-    const int row_in = lane & 31;
-    const int col_half = (lane >> 5) * 4;
-    int8_t *slice = lds + wave * (kBM * kEpiRowBytes);
+    // consecutive weight columns 8j + 4*(l/32) + 0..3.  Dequantisation runs on that layout with one row scale
+    // per lane and fragment and the column scales fetched as 16-byte vectors.  To store whole 128-byte lines,
+    // every wave passes one fragment at a time through its own slice of LDS: 128 staged bytes per row, then
+    // 16 bytes per lane and 8 rows per store instruction.
+    auto epilogue = [&]() {
+    if (MF > 0 && t.wave_live) {
+        const int wave = tid >> 6;
+        const int row_in = lane & 31;
+        const int col_half = (lane >> 5) * 4;
+        int8_t *slice = lds + wave * kEpiSlice;
+        const int N = t.N;
+        const int nw = t.nw;
 
-    // Copies the wave's staged rows (128 bytes each) to `dst` + row * row_pitch_bytes.
-    auto flush_rows = [&](int8_t *dst, long long row_pitch_bytes) {
-        const int sub = lane >> 3;    // row inside a group of 8
-        const int piece = lane & 7;   // 16-byte piece of the 128-byte row
+        // Copies rows [0, 32) of the slice (128 bytes each) to dst + (first + row) * row_pitch_bytes.
+        auto flush_fragment = [&](int8_t *dst, long long row_pitch_bytes, int mf) {
+            const int sub = lane >> 3;    // row inside a group of 8
+            const int piece = lane & 7;   // 16-byte piece of the 128-byte row
 #pragma unroll
-        for (int it = 0; it < MF * 4; ++it) {
-            const int row = it * 8 + sub;
-            const v4u v = *(const v4u *)(slice + row * kEpiRowBytes + piece * 16);
-            if (row < rows) {
-                *(v4u *)(dst + (long long)(m0 + row) * row_pitch_bytes + piece * 16) = v;
-            }
-        }
-    };
-
-    if (EPI == kEpiInt32) {
-#pragma unroll
-        for (int nf = 0; nf < kNF; ++nf) {
-            const int col0 = a.gate_up ? (nf * (N / 2) + nw * 32) : (nw * kWaveCols + nf * 32);
-#pragma unroll
-            for (int mf = 0; mf < MF; ++mf) {
-#pragma unroll
-                for (int j = 0; j < 4; ++j) {
-                    const v4i v = {acc[mf][nf][4 * j], acc[mf][nf][4 * j + 1], acc[mf][nf][4 * j + 2],
-                                   acc[mf][nf][4 * j + 3]};
-                    *(v4i *)(slice + (mf * 32 + row_in) * kEpiRowBytes + (8 * j + col_half) * 4) = v;
+            for (int it = 0; it < 4; ++it) {
+                const int row = it * 8 + sub;
+                const v4u v = *(const v4u *)(slice + row * kEpiRowBytes + piece * 16);
+                const int trow = mf * 32 + row;
+                if (trow < t.my_rows) {
+                    *(v4u *)(dst + (long long)(t.m0 + t.a_row0 + trow) * row_pitch_bytes + piece * 16) = v;
                 }
             }
-            flush_rows((int8_t *)a.out + (long long)col0 * 4, (long long)N * 4);
-        }
-    } else if (EPI == kEpiSwiglu) {
-        // t = (float(C) * w_scale[n]) * x_scale[m]; y = silu(t_gate) * t_up
-        const int I = N / 2;
-        v4f sg_gate[4], sg_up[4];
+        };
+
+        if (a.epilogue == kEpiInt32) {
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            sg_gate[j] = *(const v4f *)(t.sg + nw * 32 + 8 * j + col_half);
-            sg_up[j] = *(const v4f *)(t.sg + I + nw * 32 + 8 * j + col_half);
-        }
+            for (int nf = 0; nf < 2; ++nf) {
+                const int col0 = a.gate_up ? (nf * (N / 2) + nw * 32) : (nw * 64 + nf * 32);
 #pragma unroll
-        for (int mf = 0; mf < MF; ++mf) {
-            const float xs = row_scale_s[mf * 32 + row_in];
+                for (int mf = 0; mf < MF; ++mf) {
 #pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                v4f y;
-#pragma unroll
-                for (int e = 0; e < 4; ++e) {
-                    const float tg = __fmul_rn(__fmul_rn((float)acc[mf][0][4 * j + e], sg_gate[j][e]), xs);
-                    const float tu = __fmul_rn(__fmul_rn((float)acc[mf][1][4 * j + e], sg_up[j][e]), xs);
-                    y[e] = __fmul_rn(cam_silu_spec(tg), tu);
+                    for (int j = 0; j < 4; ++j) {
+                        const v4i v = {acc[mf][nf][4 * j], acc[mf][nf][4 * j + 1], acc[mf][nf][4 * j + 2],
+                                       acc[mf][nf][4 * j + 3]};
+                        *(v4i *)(slice + row_in * kEpiRowBytes + (8 * j + col_half) * 4) = v;
+                    }
+                    flush_fragment((int8_t *)a.out + (long long)col0 * 4, (long long)N * 4, mf);
                 }
-                *(v4f *)(slice + (mf * 32 + row_in) * kEpiRowBytes + (8 * j + col_half) * 4) = y;
             }
-        }
-        flush_rows((int8_t *)a.out + (long long)(nw * 32) * 4, (long long)I * 4);
-    } else {
-#pragma unroll
-        for (int nf = 0; nf < kNF; ++nf) {
-            v4f ws[4];
+        } else if (a.epilogue == kEpiSwiglu) {
+            // t = (float(C) * w_scale[n]) * x_scale[m]; y = silu(t_gate) * t_up
+            const int I = N / 2;
+            v4f sg_gate[4], sg_up[4];
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
-                ws[j] = *(const v4f *)(t.sg + nw * kWaveCols + nf * 32 + 8 * j + col_half);
+                sg_gate[j] = *(const v4f *)(t.sg + nw * 32 + 8 * j + col_half);
+                sg_up[j] = *(const v4f *)(t.sg + I + nw * 32 + 8 * j + col_half);
             }
 #pragma unroll
             for (int mf = 0; mf < MF; ++mf) {
-                const float xs = row_scale_s[mf * 32 + row_in];
+                const float xs = row_scale_s[t.a_row0 + mf * 32 + row_in];
 #pragma unroll
                 for (int j = 0; j < 4; ++j) {
-                    uint32_t b[4];
+                    v4f y;
 #pragma unroll
                     for (int e = 0; e < 4; ++e) {
-                        b[e] = f32_to_bf16_bits(__fmul_rn(__fmul_rn((float)acc[mf][nf][4 * j + e], ws[j][e]), xs));
+                        const float tg = __fmul_rn(__fmul_rn((float)acc[mf][0][4 * j + e], sg_gate[j][e]), xs);
+                        const float tu = __fmul_rn(__fmul_rn((float)acc[mf][1][4 * j + e], sg_up[j][e]), xs);
+                        y[e] = __fmul_rn(cam_silu_spec(tg), tu);
                     }
-                    const v2u v = {b[0] | (b[1] << 16), b[2] | (b[3] << 16)};
-                    *(v2u *)(slice + (mf * 32 + row_in) * kEpiRowBytes + (nf * 32 + 8 * j + col_half) * 2) = v;
+                    *(v4f *)(slice + row_in * kEpiRowBytes + (8 * j + col_half) * 4) = y;
+                }
+                flush_fragment((int8_t *)a.out + (long long)(nw * 32) * 4, (long long)I * 4, mf);
+            }
+        } else {
+            v4f ws[2][4];
+#pragma unroll
+            for (int nf = 0; nf < 2; ++nf) {
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    ws[nf][j] = *(const v4f *)(t.sg + nw * 64 + nf * 32 + 8 * j + col_half);
                 }
             }
+#pragma unroll
+            for (int mf = 0; mf < MF; ++mf) {
+                const float xs = row_scale_s[t.a_row0 + mf * 32 + row_in];
+#pragma unroll
+                for (int nf = 0; nf < 2; ++nf) {
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) {
+                        uint32_t b[4];
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) {
+                            b[e] = f32_to_bf16_bits(
+                                __fmul_rn(__fmul_rn((float)acc[mf][nf][4 * j + e], ws[nf][j][e]), xs));
+                        }
+                        const v2u v = {b[0] | (b[1] << 16), b[2] | (b[3] << 16)};
+                        *(v2u *)(slice + row_in * kEpiRowBytes + (nf * 32 + 8 * j + col_half) * 2) = v;
+                    }
+                }
+                flush_fragment((int8_t *)a.out + (long long)(nw * 64) * 2, (long long)N * 2, mf);
+            }
         }
-        flush_rows((int8_t *)a.out + (long long)(nw * kWaveCols) * 2, (long long)N * 2);
+    }
+    };
+
+    epilogue();
+    barrier_no_fence();  // the staging slices are free again before the next item's loads land
+}
+
+template <int TEAM, bool FLAT>
+__device__ __forceinline__ void run_item_mf(int mf, const GemmArgs &a, const ItemCtx &t, int nb, int8_t *lds,
+                                            const float *row_scale_s)
+{
+    switch (mf) {
+        case 0: run_item<0, TEAM, FLAT>(a, t, nb, lds, row_scale_s); break;
+        case 1: run_item<1, TEAM, FLAT>(a, t, nb, lds, row_scale_s); break;
+        case 2: run_item<2, TEAM, FLAT>(a, t, nb, lds, row_scale_s); break;
+        case 3: run_item<3, TEAM, FLAT>(a, t, nb, lds, row_scale_s); break;
+        default: run_item<4, TEAM, FLAT>(a, t, nb, lds, row_scale_s); break;
     }
 }
 
-template <int EPI>
-__global__ __launch_bounds__(kThreads, 2) void gemm_kernel(GemmArgs a)
+__global__ __launch_bounds__(kThreads, 1) void gemm_kernel(GemmArgs a)
 {
     __shared__ __attribute__((aligned(1024))) int8_t lds[kLdsBytes];
-    __shared__ float row_scale_s[kBM];
+    __shared__ float row_scale_s[256];
+    __shared__ int item_s;
 
+    const int tid = threadIdx.x;
+    const int team = __builtin_amdgcn_readfirstlane(tid >> 8);
+    const int wn = __builtin_amdgcn_readfirstlane((tid >> 6) & 3);
+    int32_t *sched = a.sched;
+    const int32_t *qstart = sched + kSchedQueueStart;
+    int32_t *qcount = sched + kSchedQueueCount;
+    const SchedItem *items = (const SchedItem *)(sched + kSchedHeader);
+    const int q = blockIdx.x % kNumXcd;  // workgroup i runs on XCD i % 8
+    bool own_empty = false;
+
+    // Takes the next item (thread 0 only).  A device-scope atomic on a queue counter is a round trip to the
+    // memory side and atomics on one line are served one after the other, so: every queue counter has a line
+    // of its own, the take from the own queue is issued at the START of an item and looked at only when the
+    // item is done (take_begin / take_end), and other queues are tried only after a plain load has shown that
+    // they still hold items.  Every queue runs dry, so every workgroup leaves.
+    auto take_begin = [&]() -> int {
+        return own_empty ? 0 : atomicAdd(&qcount[q * kSchedQueueStride], 1);
+    };
+    auto take_end = [&](int taken) -> int {
+        if (!own_empty) {
+            const int i = qstart[q] + taken;
+            if (i < qstart[q + 1]) {
+                return i;
+            }
+            own_empty = true;
+        }
+        for (int k = 1; k < kNumXcd; ++k) {
+            const int qq = (q + k) % kNumXcd;
+            const int len = qstart[qq + 1] - qstart[qq];
+            if (__hip_atomic_load(&qcount[qq * kSchedQueueStride], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) < len) {
+                const int i = atomicAdd(&qcount[qq * kSchedQueueStride], 1);
+                if (i < len) {
+                    return qstart[qq] + i;
+                }
+            }
+        }
+        return -1;
+    };
+
+    int next = -1;
+    if (tid == 0) {
+        next = take_end(take_begin());
+    }
+    for (;;) {
+        if (tid == 0) {
+            item_s = next;
+        }
+        __syncthreads();
+        const int idx = item_s;
+        if (idx < 0) {
+            return;
+        }
+        int taken = 0;
+        if (tid == 0) {
+            taken = take_begin();  // in flight while this item runs
+        }
+        SchedItem it = items[idx];
+        const int g = __builtin_amdgcn_readfirstlane(it.g);
+        const int m0 = __builtin_amdgcn_readfirstlane(it.m0);
+        const int rows = __builtin_amdgcn_readfirstlane(it.rows);
+        const int split = __builtin_amdgcn_readfirstlane(it.split);
+        const int nb = __builtin_amdgcn_readfirstlane(it.nb);
+        const bool flat = __builtin_amdgcn_readfirstlane(it.flat) != 0;
+
+        ItemCtx t;
+        t.Kd = a.Kd;
+        t.N = a.N;
+        t.m0 = m0;
+        t.rows = rows;
+        t.a_tile = a.a + (long long)m0 * a.Kd;
+        t.wg = a.per_expert ? a.list.w[g] : a.w + (long long)g * a.Kd * a.N;
+        t.sg = a.per_expert ? a.list.s[g] : a.w_scale + (long long)g * a.N;
+        if (flat) {
+            t.a_row0 = 0;
+            t.my_rows = rows;
+            t.bslot = team * 4 + wn;
+            t.stage_a = 128 * kBK;
+            t.stage_bytes = kStageFlat;
+        } else {
+            t.a_row0 = team == 0 ? 0 : split;
+            t.my_rows = team == 0 ? min(split, rows) : rows - split;
+            t.bslot = wn;
+            t.stage_a = 256 * kBK;
+            t.stage_bytes = kStageTall;
+        }
+        const int group = nb * (flat ? 8 : 4) + t.bslot;
+        t.wave_live = group < a.N / 64;
+        t.nw = min(group, a.N / 64 - 1);
+        if (a.epilogue != kEpiInt32 && tid < 256) {
+            row_scale_s[tid] = a.a_scale[m0 + min(tid, rows - 1)];
+        }
+        __syncthreads();  // item_s may be rewritten and the row scales read from here on
+
+        const int mf = t.my_rows <= 0 ? 0 : (t.my_rows + 31) >> 5;
+        if (flat) {
+            if (team == 0) {
+                run_item_mf<0, true>(mf, a, t, nb, lds, row_scale_s);
+            } else {
+                run_item_mf<1, true>(mf, a, t, nb, lds, row_scale_s);
+            }
+        } else {
+            if (team == 0) {
+                run_item_mf<0, false>(mf, a, t, nb, lds, row_scale_s);
+            } else {
+                run_item_mf<1, false>(mf, a, t, nb, lds, row_scale_s);
+            }
+        }
+        if (tid == 0) {
+            next = take_end(taken);
+        }
+    }
+}
+
+// Builds the schedules of up to two GEMMs over the same group list (single workgroup of 1024 threads).
+// Expert g with r rows: r == 0 owns nothing; r <= 128 is "flat": one tile and ceil(N/512) column blocks;
+// otherwise "tall": ceil(r/256) tiles of (nearly) equal height, a multiple of 32, and ceil(N/256) column
+// blocks.  Experts are ranked by rows, largest first.
+//   * Tall experts: the (expert, column block) groups, in rank order, are cut into eight consecutive runs of
+//     equal work (rows x column blocks), one per queue.  A queue therefore holds few experts, each with
+//     neighbouring column blocks: the CUs of an XCD that work side by side share the weight panels (row tiles
+//     of one group) and the activation tiles (column blocks of one expert) through their L2, and an expert's
+//     activations are fetched by as few XCDs as its size requires.
+//   * Flat experts are dealt to the queues whole, in rank order, so that the column blocks of one expert,
+//     which all read the same few activation rows, run on one XCD.
+// A queue lists its flat items first, then its tall items, big experts first.  A flat item streams its weights
+// at the pace one CU can pull them from memory and takes longer than a tall one although it computes less:
+// started first, flat items run beside tall ones, which need the matrix cores rather than the memory, and the
+// queues end with items of even length.
+// The work is laid out so that it needs few workgroup barriers: every prefix sum over the experts is the job
+// of one wave, which walks the ranks 64 at a time.
+struct ExpertShape {
+    int rows, tiles, blocks, units;
+    bool tall, flat;
+};
+
+__device__ __forceinline__ ExpertShape expert_shape(int rows, int nb_tall, int nb_flat)
+{
+    ExpertShape e;
+    e.rows = rows;
+    e.tall = rows > 128;
+    e.flat = rows > 0 && !e.tall;
+    e.tiles = e.tall ? (rows + 255) / 256 : (e.flat ? 1 : 0);
+    e.blocks = e.tall ? nb_tall : (e.flat ? nb_flat : 0);
+    e.units = (rows + 31) / 32;
+    return e;
+}
+
+// Queue of the tall group whose work (in units) starts at `before` and is `units` long: the queue its middle
+// falls into when the total work is cut into eight equal runs.
+__device__ __forceinline__ int queue_of_group(long long before, int units, long long wtotal)
+{
+    const long long mid16 = (2 * before + units) * kNumXcd;  // 2 * middle * 8
+    int x = 0;
+#pragma unroll
+    for (int k = 1; k < kNumXcd; ++k) {
+        x += mid16 >= 2 * wtotal * k ? 1 : 0;
+    }
+    return x;
+}
+
+__global__ __launch_bounds__(1024) void build_sched_kernel(const int64_t *group_list, int cumulative, int G,
+                                                          long long max_rows, int nspec, SchedSpec s0, SchedSpec s1)
+{
+    __shared__ int rows_s[kMaxExperts], off_s[kMaxExperts], order_s[kMaxExperts];
+    __shared__ int first_item_s[kMaxExperts + 1];      // by rank: items of the experts ranked before
+    __shared__ int work_before_s[kMaxExperts];         // by rank: work of the tall experts ranked before
+    __shared__ int flat_rank_s[kMaxExperts];           // by rank: flat experts ranked before
+    __shared__ short ngroups_s[kNumXcd][kMaxExperts];  // by rank: the expert's groups in queue x (tall)
+    __shared__ int qbase_s[kNumXcd][kMaxExperts];      // by rank: items of earlier experts of its kind in queue x
+    __shared__ int qtall_s[kNumXcd], qflat_s[kNumXcd];
+    __shared__ int wtotal_s, total_rows_s;
     const int tid = threadIdx.x;
     const int lane = tid & (kWave - 1);
     const int wave = tid >> 6;
 
-    // ---- which tile, which column block.
-    // Each XCD takes one contiguous run of work ids (workgroup i runs on XCD i % 8).  Inside an expert
-    // with n tiles the ids run: a group of column blocks, and inside the group the column block, and
-    // inside the column block the expert's n tiles.  The workgroups that are resident together on an
-    // XCD (64) then are all the row tiles of an expert for a few column blocks: they stream the same
-    // weight panels at the same depth and find each other's lines in L2, so a panel is fetched once.
-    const int num_tiles = min(a.tiles[0], a.max_tiles);
-    const int nblocks = (a.N + kBlockCols - 1) / kBlockCols;
-    const long long total_work = (long long)num_tiles * nblocks;
-    const long long chunk = (total_work + kNumXcd - 1) / kNumXcd;
-    const long long slot = blockIdx.x / kNumXcd;
-    const long long wid = (long long)(blockIdx.x % kNumXcd) * chunk + slot;
-    if (slot >= chunk || wid >= total_work) {
-        return;
-    }
-    const int32_t *probe = a.tiles + kTileHeader + kTileRecord * (int)(wid / nblocks);
-    const int first = probe[3];
-    const int ntile = max(probe[4], 1);
-    const int local = (int)(wid - (long long)first * nblocks);  // id inside the expert
-    const int tile = first + local % ntile;
-    const int nb = local / ntile;
-    const int32_t *te = a.tiles + kTileHeader + kTileRecord * tile;
-    const int g = te[0];
-    TileCtx t;
-    t.m0 = te[1];
-    t.rows = te[2];
-    if (t.rows <= 0) {
-        return;
-    }
-    t.Kd = a.Kd;
-    t.N = a.N;
-    t.nw = nb * 4 + wave;  // this wave's 64-column group
-    t.wave_live = t.nw * kWaveCols < t.N;
-    const int8_t *wg = a.per_expert ? a.list.w[g] : a.w + (long long)g * t.Kd * t.N;
-    t.sg = a.per_expert ? a.list.s[g] : a.w_scale + (long long)g * t.N;
-    t.wp = wg + (long long)(t.wave_live ? t.nw : 0) * t.Kd * kWaveCols + lane * 16;
-    t.a_tile = a.a + (long long)t.m0 * t.Kd;
-    // The start depth depends on the expert only, so that all workgroups of an expert, which share
-    // activation rows or weight panels, stay in step and find each other's lines in L2.
-    t.k_start = (int)(((long long)g * 37) % (t.Kd / kBK));
-
-    if (EPI != kEpiInt32) {
-        for (int r = tid; r < kBM; r += kThreads) {
-            row_scale_s[r] = a.a_scale[t.m0 + min(r, t.rows - 1)];
+    // rows and first row of every expert (wave 0)
+    if (wave == 0) {
+        long long run = 0;  // rows before this chunk (counts) / unused (cumulative)
+        for (int base = 0; base < G; base += kWave) {
+            const int g = base + lane;
+            long long m0 = 0, m1 = 0;
+            if (cumulative) {
+                if (g < G) {
+                    m0 = g == 0 ? 0 : group_list[g - 1];
+                    m1 = group_list[g];
+                }
+            } else {
+                const int c = g < G ? (int)min(max(group_list[g], (int64_t)0), (int64_t)max_rows) : 0;
+                const int inc = wave_inclusive_scan(c, lane);
+                m0 = run + inc - c;
+                m1 = m0 + c;
+                run += __shfl(inc, kWave - 1, kWave);
+            }
+            // Clamp to the rows that exist so that a corrupt group list cannot index past the tensors.
+            m0 = min(max(m0, 0ll), max_rows);
+            m1 = min(max(m1, m0), max_rows);
+            if (g < G) {
+                rows_s[g] = (int)(m1 - m0);
+                off_s[g] = (int)m0;
+            }
+            const int chunk_rows = wave_sum(g < G ? (int)(m1 - m0) : 0);
+            if (lane == 0) {
+                total_rows_s = (base == 0 ? 0 : total_rows_s) + chunk_rows;
+            }
         }
     }
+    __syncthreads();
+    // rank by rows, largest first (ties: lower index first)
+    if (tid < G) {
+        const int cnt = rows_s[tid];
+        int rank = 0;
+        for (int j = 0; j < G; ++j) {
+            const int rj = rows_s[j];
+            rank += (rj > cnt || (rj == cnt && j < tid)) ? 1 : 0;
+        }
+        order_s[rank] = tid;
+    }
+    __syncthreads();
+    const int total_rows = total_rows_s;
 
-    const int mfrags = (t.rows + 31) >> 5;
-    if (mfrags <= 1) {
-        gemm_tile<EPI, 1>(a, t, lds, row_scale_s);
-    } else if (mfrags <= 2) {
-        gemm_tile<EPI, 2>(a, t, lds, row_scale_s);
-    } else if (mfrags <= 3) {
-        gemm_tile<EPI, 3>(a, t, lds, row_scale_s);
-    } else {
-        gemm_tile<EPI, 4>(a, t, lds, row_scale_s);
+    for (int sp = 0; sp < nspec; ++sp) {
+        const SchedSpec spec = sp == 0 ? s0 : s1;
+        int32_t *sched = spec.sched;
+        SchedItem *items = (SchedItem *)(sched + kSchedHeader);
+        const int nb_tall = (spec.N + 255) / 256;
+        const int nb_flat = (spec.N + 511) / 512;
+
+        // by rank: items, tall work and flat experts before (wave 0)
+        if (wave == 0) {
+            int items_run = 0, work_run = 0, flat_run = 0;
+            for (int base = 0; base < G; base += kWave) {
+                const int rank = base + lane;
+                const ExpertShape e = expert_shape(rank < G ? rows_s[order_s[rank]] : 0, nb_tall, nb_flat);
+                const int vi = e.blocks * e.tiles, vw = e.tall ? e.blocks * e.units : 0, vf = e.flat ? 1 : 0;
+                const int ii = wave_inclusive_scan(vi, lane);
+                const int iw = wave_inclusive_scan(vw, lane);
+                const int jf = wave_inclusive_scan(vf, lane);
+                if (rank < G) {
+                    first_item_s[rank] = items_run + ii - vi;
+                    work_before_s[rank] = work_run + iw - vw;
+                    flat_rank_s[rank] = flat_run + jf - vf;
+                }
+                items_run += __shfl(ii, kWave - 1, kWave);
+                work_run += __shfl(iw, kWave - 1, kWave);
+                flat_run += __shfl(jf, kWave - 1, kWave);
+            }
+            if (lane == 0) {
+                first_item_s[G] = items_run;
+                wtotal_s = max(work_run, 1);
+            }
+        }
+        __syncthreads();
+        const int n_items = first_item_s[G];
+        const long long wtotal = wtotal_s;
+
+        // by rank and queue: items of earlier experts.  Wave x (0..7) counts the tall items of queue x, wave 8 + x
+        // its flat items.
+        {
+            const int x = wave & (kNumXcd - 1);
+            const bool flat_wave = wave >= kNumXcd;
+            int run = 0;
+            for (int base = 0; base < G; base += kWave) {
+                const int rank = base + lane;
+                const ExpertShape e = expert_shape(rank < G ? rows_s[order_s[rank]] : 0, nb_tall, nb_flat);
+                int v = 0;
+                if (flat_wave) {
+                    v = (e.flat && flat_rank_s[rank] % kNumXcd == x) ? e.blocks : 0;
+                } else if (e.tall) {
+                    int mine = 0;
+                    const long long before = work_before_s[rank];
+                    for (int c = 0; c < e.blocks; ++c) {
+                        mine += queue_of_group(before + (long long)c * e.units, e.units, wtotal) == x ? 1 : 0;
+                    }
+                    ngroups_s[x][rank] = (short)mine;
+                    v = mine * e.tiles;
+                }
+                const int inc = wave_inclusive_scan(v, lane);
+                if (rank < G && (flat_wave ? e.flat : e.tall)) {
+                    qbase_s[x][rank] = run + inc - v;
+                }
+                run += __shfl(inc, kWave - 1, kWave);
+            }
+            if (lane == 0) {
+                (flat_wave ? qflat_s : qtall_s)[x] = run;
+            }
+        }
+        __syncthreads();
+        if (tid == 0) {
+            int run = 0;
+            for (int x = 0; x < kNumXcd; ++x) {
+                sched[kSchedQueueStart + x] = run;
+                sched[kSchedQueueCount + x * kSchedQueueStride] = 0;
+                run += qflat_s[x] + qtall_s[x];
+            }
+            sched[kSchedQueueStart + kNumXcd] = run;
+            sched[0] = min(n_items, spec.max_items);
+            sched[1] = total_rows;
+            sched[2] = 0;
+            sched[3] = 0;
+        }
+        // one thread per item, in rank-major order
+        for (int i = tid; i < n_items; i += 1024) {
+            int lo = 0, hi = G;  // largest rank with first_item <= i
+            while (hi - lo > 1) {
+                const int mid = (lo + hi) >> 1;
+                if (first_item_s[mid] <= i) {
+                    lo = mid;
+                } else {
+                    hi = mid;
+                }
+            }
+            const int rank = lo;
+            const int eg = order_s[rank];
+            const ExpertShape e = expert_shape(rows_s[eg], nb_tall, nb_flat);
+            const int local = i - first_item_s[rank];
+            const int c = local / e.tiles;
+            const int j = local - c * e.tiles;
+            int x, qpos;
+            if (e.flat) {
+                x = flat_rank_s[rank] % kNumXcd;
+                qpos = qbase_s[x][rank] + c;  // flat items first
+            } else {
+                x = queue_of_group(work_before_s[rank] + (long long)c * e.units, e.units, wtotal);
+                int cfirst = 0;  // the expert's groups in earlier queues
+                for (int xx = 0; xx < x; ++xx) {
+                    cfirst += ngroups_s[xx][rank];
+                }
+                qpos = qflat_s[x] + qbase_s[x][rank] + (c - cfirst) * e.tiles + j;
+            }
+            int pos = qpos;
+            for (int xx = 0; xx < x; ++xx) {
+                pos += qflat_s[xx] + qtall_s[xx];
+            }
+            if (pos >= spec.max_items) {
+                continue;  // cannot happen with a table sized by sched_bytes(); guards a corrupt list
+            }
+            // tile j of e.tiles: heights are multiples of 32 that differ by at most 32
+            const int base_u = e.units / e.tiles, extra = e.units % e.tiles;
+            const int u0 = j * base_u + min(j, extra);
+            const int uj = base_u + (j < extra ? 1 : 0);
+            SchedItem it;
+            it.g = eg;
+            it.m0 = off_s[eg] + u0 * 32;
+            it.rows = min(uj * 32, e.rows - u0 * 32);
+            it.split = e.flat ? 0 : 32 * ((it.rows + 63) / 64);
+            it.nb = c;
+            it.flat = e.flat ? 1 : 0;
+            it.pad0 = 0;
+            it.pad1 = 0;
+            items[pos] = it;
+        }
+        __syncthreads();
     }
 }
 
 // SwiGLU product rows (fp32) -> int8 rows + per-row scale:
 //   m = max|y|; y_scale = m * (1/127); q = rint((y * 127) * (1/m)).   One workgroup per row.
 __global__ __launch_bounds__(256) void requant_kernel(const float *__restrict__ y, int I,
-                                                      const int32_t *__restrict__ tiles, long long max_rows,
+                                                      const int32_t *__restrict__ sched, long long max_rows,
                                                       int8_t *__restrict__ q, float *__restrict__ scale)
 {
     __shared__ float wave_max_s[4];
     const long long row = blockIdx.x;
-    const long long valid = tiles != nullptr ? min((long long)tiles[1], max_rows) : max_rows;
+    const long long valid = sched != nullptr ? min((long long)sched[1], max_rows) : max_rows;
     if (row >= valid) {
         return;
     }
@@ -494,40 +836,59 @@ __global__ __launch_bounds__(256) void prepack_kernel(const int8_t *__restrict__
     *((v4u *)(dst + (long long)g * Kd * N) + p) = o;
 }
 
+int g_num_cus = 0;  // workgroups of the persistent kernel: one per CU of the current device
+
 }  // namespace
 
-hipError_t launch_gemm(const GemmArgs &a, hipStream_t stream)
+int sched_max_items(int64_t max_rows, int G, int N)
 {
-    if (a.max_tiles <= 0) {
-        return hipSuccess;
-    }
-    if (a.Kd % 128 != 0 || a.N % kWaveCols != 0 || (a.gate_up && a.N % (2 * kWaveCols) != 0)) {
+    // tall tiles hold more than 128 rows each, flat tiles are one per expert
+    const int64_t tiles = max_rows / 129 + G;
+    return (int)(tiles * ((N + 255) / 256));
+}
+
+uint64_t sched_bytes(int64_t max_rows, int G, int N)
+{
+    return (uint64_t)(kSchedHeader + (int64_t)sched_max_items(max_rows, G, N) * (int)(sizeof(SchedItem) / 4)) * 4;
+}
+
+hipError_t launch_build_sched(const int64_t *group_list, int cumulative, int G, int64_t max_rows, int nspec,
+                              const SchedSpec *specs, hipStream_t stream)
+{
+    if (G <= 0 || G > kMaxExperts || nspec < 1 || nspec > 2) {
         return hipErrorInvalidValue;
     }
-    const int nblocks = (a.N + kBlockCols - 1) / kBlockCols;
-    long long work = (long long)a.max_tiles * nblocks;
-    work = (work + kNumXcd - 1) / kNumXcd * kNumXcd;
-    if (work > 0x7fffffffll) {
-        return hipErrorInvalidValue;
-    }
-    dim3 grid((unsigned)work), block(kThreads);
-    switch (a.epilogue) {
-        case kEpiInt32:
-            hipLaunchKernelGGL(gemm_kernel<kEpiInt32>, grid, block, 0, stream, a);
-            break;
-        case kEpiSwiglu:
-            hipLaunchKernelGGL(gemm_kernel<kEpiSwiglu>, grid, block, 0, stream, a);
-            break;
-        case kEpiDequantBf16:
-            hipLaunchKernelGGL(gemm_kernel<kEpiDequantBf16>, grid, block, 0, stream, a);
-            break;
-        default:
-            return hipErrorInvalidValue;
-    }
+    const SchedSpec s0 = specs[0];
+    const SchedSpec s1 = nspec > 1 ? specs[1] : specs[0];
+    hipLaunchKernelGGL(build_sched_kernel, dim3(1), dim3(1024), 0, stream, group_list, cumulative, G,
+                       (long long)max_rows, nspec, s0, s1);
     return hipGetLastError();
 }
 
-hipError_t launch_requant(const float *y, int64_t max_rows, int I, const int32_t *tiles_for_rows, int8_t *q,
+hipError_t launch_gemm(const GemmArgs &a, hipStream_t stream)
+{
+    if (a.sched == nullptr) {
+        return hipErrorInvalidValue;
+    }
+    if (a.Kd % kBK != 0 || a.Kd < kBK || a.N % 64 != 0 || (a.gate_up && a.N % 128 != 0)) {
+        return hipErrorInvalidValue;
+    }
+    if (g_num_cus == 0) {
+        int dev = 0, n = 0;
+        hipError_t e = hipGetDevice(&dev);
+        if (e == hipSuccess) {
+            e = hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev);
+        }
+        if (e != hipSuccess) {
+            return e;
+        }
+        g_num_cus = n > 0 ? n : 256;
+    }
+    hipLaunchKernelGGL(gemm_kernel, dim3((unsigned)g_num_cus), dim3(kThreads), 0, stream, a);
+    return hipGetLastError();
+}
+
+hipError_t launch_requant(const float *y, int64_t max_rows, int I, const int32_t *sched_for_rows, int8_t *q,
                           float *scale, hipStream_t stream)
 {
     if (max_rows <= 0) {
@@ -536,14 +897,14 @@ hipError_t launch_requant(const float *y, int64_t max_rows, int I, const int32_t
     if (I % 4 != 0 || I > 4096) {
         return hipErrorInvalidValue;
     }
-    hipLaunchKernelGGL(requant_kernel, dim3((unsigned)max_rows), dim3(256), 0, stream, y, I, tiles_for_rows,
+    hipLaunchKernelGGL(requant_kernel, dim3((unsigned)max_rows), dim3(256), 0, stream, y, I, sched_for_rows,
                        (long long)max_rows, q, scale);
     return hipGetLastError();
 }
 
 hipError_t launch_prepack(const int8_t *src, int8_t *dst, int G, int Kd, int N, int gate_up, hipStream_t stream)
 {
-    if (Kd % kBK != 0 || N % kWaveCols != 0 || (gate_up && N % (2 * kWaveCols) != 0)) {
+    if (Kd % kBK != 0 || N % 64 != 0 || (gate_up && N % 128 != 0)) {
         return hipErrorInvalidValue;
     }
     const long long pieces = (long long)Kd * N / 16;

@@ -1,5 +1,5 @@
 // Routing plan kernels: per-expert counts, prefix offsets, the stable within-expert rank of every
-// (token, k) entry, receive bookkeeping and the GEMM tile table.
+// (token, k) entry and receive bookkeeping.
 //
 // Reference semantics restated here (paths relative to the reference tree):
 //   counts        src/cam/comm_operator/ascend_kernels/dispatch_layout/op_kernel/dispatch_layout.h:83-134
@@ -23,7 +23,7 @@ namespace cam {
 
 namespace {
 
-constexpr int kScanThreads = 1024;  // single-workgroup scan kernels (notify, tile table)
+constexpr int kScanThreads = 1024;  // single-workgroup scan kernel (notify)
 constexpr int kGlobalThreads = 512; // phase 2: one thread per expert column
 
 // Phase 1.  Workgroup b ranks the flat entries [b*chunk, (b+1)*chunk), chunk = IT*256 (rank_chunk), and
@@ -46,7 +46,7 @@ __global__ __launch_bounds__(kLocalThreads) void plan_local_kernel(PlanArgs a, i
 // Phase 2.  Every workgroup sums the histogram columns (all rows for the per-expert count, the rows
 // before its own for its base), scans the counts into offsets, and finishes its own chunk:
 // pos += base[e], dst_row = off[e] + pos.  Workgroup 0 also writes the per-expert outputs and the
-// GEMM tile table.
+
 template <typename IdT>
 __global__ __launch_bounds__(kGlobalThreads) void plan_global_kernel(PlanArgs a, int chunk, const int32_t *hist_in)
 {
@@ -125,19 +125,11 @@ __global__ __launch_bounds__(kGlobalThreads) void plan_global_kernel(PlanArgs a,
             a.per_rank_zero[r] = 0;
         }
     }
-    // GEMM tile table: expert e owns ceil(cnt/kGemmTileM) tiles, in expert order.
-    if (a.tiles != nullptr) {
-        const int nt = tid < E ? (cnt + kGemmTileM - 1) / kGemmTileM : 0;
-        const int tbase = block_exclusive_scan<NW>(nt, tid, scan_s, &total_s);
-        if (tid < E) {
-            write_tile_records(a.tiles, tid, off, cnt, tbase, nt, 0x7fffffff);
-        }
-        if (tid == 0) {
-            a.tiles[0] = total_s;
-            a.tiles[1] = total;
-            a.tiles[2] = t_active;
-            a.tiles[3] = 0;
-        }
+    if (tid == 0 && a.meta != nullptr) {
+        a.meta[0] = 0;
+        a.meta[1] = total;
+        a.meta[2] = t_active;
+        a.meta[3] = 0;
     }
 }
 
@@ -205,49 +197,6 @@ __global__ __launch_bounds__(kScanThreads) void notify_scan_kernel(const int32_t
             recv_data[3 * tid + 1] = o;
             recv_data[3 * tid + 2] = num_tokens;
         }
-    }
-}
-
-__global__ __launch_bounds__(kScanThreads) void build_tiles_kernel(const int64_t *group_list, int cumulative,
-                                                                  int G, long long max_rows, int max_tiles,
-                                                                  int32_t *tiles)
-{
-    __shared__ int scan_s[kScanThreads / kWave];
-    __shared__ int total_s;
-    const int tid = threadIdx.x;
-    long long m0 = 0, m1 = 0;
-    if (tid < G) {
-        if (cumulative) {
-            m0 = tid == 0 ? 0 : group_list[tid - 1];
-            m1 = group_list[tid];
-        } else {
-            m1 = group_list[tid];  // converted to a cumulative value below
-        }
-    }
-    if (!cumulative) {
-        int c = tid < G ? (int)min(max(m1, 0ll), max_rows) : 0;
-        int o = block_exclusive_scan<kScanThreads / kWave>(c, tid, scan_s, &total_s);
-        m0 = o;
-        m1 = (long long)o + c;
-    }
-    // Clamp to the rows that exist so that a corrupt group list cannot index past the tensors.
-    m0 = min(max(m0, 0ll), max_rows);
-    m1 = min(max(m1, m0), max_rows);
-    int cnt = tid < G ? (int)(m1 - m0) : 0;
-    int nt = (cnt + kGemmTileM - 1) / kGemmTileM;
-    int tbase = block_exclusive_scan<kScanThreads / kWave>(nt, tid, scan_s, &total_s);
-    int num_tiles = min(total_s, max_tiles);
-    if (tid < G) {
-        write_tile_records(tiles, tid, (int)m0, cnt, tbase, nt, max_tiles);  // a corrupt list cannot overrun the table
-    }
-    __syncthreads();
-    int rows_total = block_exclusive_scan<kScanThreads / kWave>(cnt, tid, scan_s, &total_s);
-    (void)rows_total;
-    if (tid == 0) {
-        tiles[0] = num_tiles;
-        tiles[1] = total_s;
-        tiles[2] = 0;
-        tiles[3] = 0;
     }
 }
 
@@ -330,14 +279,6 @@ hipError_t launch_notify_scan(const int32_t *cnt, int E, int num_tokens, int32_t
 {
     hipLaunchKernelGGL(notify_scan_kernel, dim3(1), dim3(kScanThreads), 0, stream, cnt, E, num_tokens, off,
                        send_data, recv_data);
-    return hipGetLastError();
-}
-
-hipError_t launch_build_tiles(const int64_t *group_list, int cumulative, int G, int64_t max_rows, int max_tiles,
-                              int32_t *tiles, hipStream_t stream)
-{
-    hipLaunchKernelGGL(build_tiles_kernel, dim3(1), dim3(kScanThreads), 0, stream, group_list, cumulative, G,
-                       (long long)max_rows, max_tiles, tiles);
     return hipGetLastError();
 }
 

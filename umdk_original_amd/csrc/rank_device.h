@@ -71,25 +71,6 @@ __device__ __forceinline__ int count_active(const uint8_t *mask, int T, int tid,
     return *slot;
 }
 
-// Tile records of one expert: its `cnt` rows from row `off` on, split evenly over `nt` tiles (equal
-// tiles keep the workgroups that stream the same weight panel in step with each other).
-__device__ __forceinline__ void write_tile_records(int32_t *tiles, int expert, int off, int cnt, int tbase, int nt,
-                                                   int max_tiles)
-{
-    const int q = nt > 0 ? (cnt + nt - 1) / nt : 0;
-    for (int j = 0; j < nt && tbase + j < max_tiles; ++j) {
-        int32_t *t = tiles + kTileHeader + kTileRecord * (tbase + j);
-        t[0] = expert;
-        t[1] = off + j * q;
-        t[2] = min(q, cnt - j * q);
-        t[3] = tbase;
-        t[4] = nt;
-        t[5] = 0;
-        t[6] = 0;
-        t[7] = 0;
-    }
-}
-
 // Ranks the chunk of flat entries [b*IT*256, (b+1)*IT*256) of one workgroup of 256 threads.
 // Wave w owns the IT*64 entries from b*chunk + w*IT*64 and each lane keeps its IT ids in registers.
 // 64 ids at a time, lanes holding the same id find each other with one ballot per id bit; the rank
