@@ -517,12 +517,14 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_kernel(GemmArgs a)
 //     activations are fetched by as few XCDs as its size requires.
 //   * Flat experts are dealt to the queues whole, in rank order, so that the column blocks of one expert,
 //     which all read the same few activation rows, run on one XCD.
-// A queue lists its flat items first, then its tall items, big experts first.  A flat item streams its weights
-// at the pace one CU can pull them from memory and takes longer than a tall one although it computes less:
-// started first, flat items run beside tall ones, which need the matrix cores rather than the memory, and the
-// queues end with items of even length.
+// A queue lists its tall items big experts first, with its flat items spread evenly among them except for the
+// last kTallTail places.  A flat item streams its weights at the pace one CU can pull them from memory and takes
+// longer than a tall one although it computes less: spread out, flat items run beside tall ones, which need
+// the matrix cores rather than the memory, and the queues end with items of even length.
 // The work is laid out so that it needs few workgroup barriers: every prefix sum over the experts is the job
 // of one wave, which walks the ranks 64 at a time.
+constexpr int kTallTail = 24;  // tall items a queue ends with (three quarters of a round of its 32 workgroups)
+
 struct ExpertShape {
     int rows, tiles, blocks, units;
     bool tall, flat;
@@ -713,14 +715,30 @@ __global__ __launch_bounds__(1024) void build_sched_kernel(const int64_t *group_
             int x, qpos;
             if (e.flat) {
                 x = flat_rank_s[rank] % kNumXcd;
-                qpos = qbase_s[x][rank] + c;  // flat items first
+                qpos = qbase_s[x][rank] + c;
             } else {
                 x = queue_of_group(work_before_s[rank] + (long long)c * e.units, e.units, wtotal);
                 int cfirst = 0;  // the expert's groups in earlier queues
                 for (int xx = 0; xx < x; ++xx) {
                     cfirst += ngroups_s[xx][rank];
                 }
-                qpos = qflat_s[x] + qbase_s[x][rank] + (c - cfirst) * e.tiles + j;
+                qpos = qbase_s[x][rank] + (c - cfirst) * e.tiles + j;
+            }
+            {
+                // Queue order: the flat items spread evenly among the tall ones (flat item j has key (2j+1)/(2F),
+                // tall item i key (2i+1)/(2T), smaller keys first, a tall item first on a tie), except that the
+                // last kTallTail tall items follow the last flat one.
+                const long long F = qflat_s[x];
+                const long long T = max(qtall_s[x] - kTallTail, 0);
+                if (e.flat) {
+                    const long long num = (2ll * qpos + 1) * T - F;
+                    qpos += (int)(num < 0 ? 0 : min(T, num / (2 * F) + 1));
+                } else if (qpos < T) {
+                    const long long num = (2ll * qpos + 1) * F - T;
+                    qpos += (int)(num <= 0 ? 0 : min(F, (num + 2 * T - 1) / (2 * T)));
+                } else {
+                    qpos += (int)F;
+                }
             }
             int pos = qpos;
             for (int xx = 0; xx < x; ++xx) {
