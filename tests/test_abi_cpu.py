@@ -196,6 +196,9 @@ def test_fused_deep_moe_validation():
     a[1] = _t((5, 2), torch.int32)
     assert _lib.phase1("FusedDeepMoe", a)[0] == CAM_ERR_SHAPE
     a = _fused_args()
+    a[15] = 7  # quantMode
+    assert _lib.phase1("FusedDeepMoe", a)[0] == CAM_ERR_RANGE
+    a = _fused_args()
     a[2] = [_packed((4, 1024, 512))]  # wrong 2I
     assert _lib.phase1("FusedDeepMoe", a)[0] == CAM_ERR_SHAPE
     a = _fused_args()
@@ -225,6 +228,17 @@ def test_gemm_and_prepack_validation():
     assert _lib.phase1("GroupedMatmulInt32", [x, [_packed((2, 128, 128))], 0, gl, 2, out])[0] == CAM_ERR_RANGE
     assert _lib.phase1("GroupedMatmulInt32", [x, [_packed((2, 128, 128))], 0, _t((2,), torch.int32), 0, out])[0] == \
         CAM_ERR_DTYPE
+    # outputs and weight scales are written and read 16 bytes at a time
+    skewed = _t((10 * 128 + 1,), torch.int32)[1:].view(10, 128)
+    assert _lib.phase1("GroupedMatmulInt32", [x, [_packed((2, 128, 128))], 0, gl, 0, skewed])[0] == CAM_ERR_ALIGN
+    xs, bf = _t((10,), torch.float32), _t((10, 128), torch.bfloat16)
+    deq = [x, xs, [_packed((2, 128, 128))], [_t((2, 128), torch.float32)], gl, 0, bf]
+    assert _lib.phase1("GroupedMatmulDequant", deq)[0] == CAM_OK
+    deq[3] = [_t((2 * 128 + 1,), torch.float32)[1:].view(2, 128)]
+    assert _lib.phase1("GroupedMatmulDequant", deq)[0] == CAM_ERR_ALIGN
+    deq[3] = [_t((2, 128), torch.float32)]
+    deq[6] = _t((10 * 128 + 1,), torch.bfloat16)[1:].view(10, 128)
+    assert _lib.phase1("GroupedMatmulDequant", deq)[0] == CAM_ERR_ALIGN
 
 
 def test_phase2_rejects_wrong_executor_and_small_workspace():

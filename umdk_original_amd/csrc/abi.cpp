@@ -244,6 +244,10 @@ camStatus resolve_weights(const camTensorList *wl, const camTensorList *sl, cons
             if (s->dtype != CAM_DT_FLOAT) {
                 return fail(CAM_ERR_DTYPE, "%s scale must be float32", wname);
             }
+            if (((uintptr_t)s->data) % 16 != 0) {
+                return fail(CAM_ERR_ALIGN, "%s scale[%llu] data must be 16-byte aligned", wname,
+                            (unsigned long long)i);
+            }
             int64_t want = stacked ? G * N : N;
             if (numel(s) != want || !is_contiguous(s)) {
                 return fail(CAM_ERR_SHAPE, "%s scale[%llu] must hold %lld contiguous values", wname,
@@ -1242,6 +1246,7 @@ camStatus camGroupedMatmulDequantGetWorkspaceSize(const camTensor *x, const camT
         return fail(CAM_ERR_SHAPE, "out must have one row per row of x");
     }
     CAM_TRY(check_gemm_dims("GroupedMatmulDequant", gc.Kd, N, false));
+    CAM_TRY(check_aligned(out, "out", 16));
     WeightSet ws{};
     CAM_TRY(resolve_weights(weight, weightScale, "weight", gc.G, gc.Kd, N, true, &ws));
     cam::SchedSpec sp = sched_spec(gc.A, gc.G, N);
@@ -1290,6 +1295,7 @@ camStatus camGroupedMatmulInt32GetWorkspaceSize(const camTensor *x, const camTen
         return fail(CAM_ERR_SHAPE, "out must have one row per row of x");
     }
     CAM_TRY(check_gemm_dims("GroupedMatmulInt32", gc.Kd, N, gateUp != 0));
+    CAM_TRY(check_aligned(out, "out", 16));
     WeightSet ws{};
     CAM_TRY(resolve_weights(weight, nullptr, "weight", gc.G, gc.Kd, N, false, &ws));
     cam::SchedSpec sp = sched_spec(gc.A, gc.G, N);
@@ -1338,7 +1344,12 @@ camStatus camFusedDeepMoeGetWorkspaceSize(const camTensor *x, const camTensor *e
                                           camOpExecutor **executor)
 {
     (void)groupEp;
-    (void)quantMode;
+    // The fused operator always quantises per token (the only path the reference kernel has); quantMode is
+    // carried into the tiling data unchecked there (AK/fused_deep_moe/op_host/fused_deep_moe_tiling.cpp:356).
+    // Values no dispatch operator knows are rejected here instead of being ignored.
+    if (quantMode < 0 || quantMode > 3) {
+        return fail(CAM_ERR_RANGE, "quantMode %lld outside [0, 3]", (long long)quantMode);
+    }
     CAM_TRY(check_tensor(x, "x", 2, CAM_DT_BF16, CAM_DT_FLOAT16));
     CAM_TRY(check_tensor(expertIds, "expertIds", 2, CAM_DT_INT32));
     CAM_TRY(check_tensor(expertScales, "expertScales", 2, CAM_DT_FLOAT));
