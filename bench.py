@@ -91,7 +91,8 @@ def main():
     ap.add_argument("--skip-gemm", action="store_true")
     ap.add_argument("--skip-layer", action="store_true")
     ap.add_argument("--skip-cpu", action="store_true")
-    ap.add_argument("--only", default="", help="comma list of sections: step,dispatch,combine,gemm,layer,copy")
+    ap.add_argument("--only", default="", help="comma list of sections: step (the timed dispatch + combine step and its two kernels), "
+                         "dispatch / combine (those plus the other operator forms of each), gemm, layer, copy")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build is single-GPU; every figure is measured on one MI355X. "
@@ -213,6 +214,7 @@ def main():
                                              note="MoeDispatchPrefill: plan + permute + int8 quant, one launch")
             log("dispatch (one launch): %.1f us -> %.0f GB/s = %.1f%% of HBM peak"
                 % (t_disp * 1e6, disp_bytes / t_disp / 1e9, 100 * disp_bytes / t_disp / HBM_PEAK))
+        if want("dispatch"):
             # the same work as the reference's operator pair: plan, then aclnn-shaped permute (3 launches)
             plan_bufs = [dict(pos=torch.empty((T, K), **i32), cnt=torch.empty(E, **i32), off=torch.empty(E, **i32),
                               roff=torch.empty(E, **i32), rcnt=torch.empty(E, **i32),
@@ -246,6 +248,7 @@ def main():
                                              note="MoeCombineGather with the dispatch's (token, k) -> row map")
             log("combine (gather with the dispatch's map): %.1f us -> %.0f GB/s = %.1f%% of HBM peak"
                 % (t_comb * 1e6, comb_bytes / t_comb / 1e9, 100 * comb_bytes / t_comb / HBM_PEAK))
+        if want("combine"):
             wss = [torch.empty(T * K * 4 + 256, dtype=torch.uint8, device=dev) for _ in range(NBUF)]
 
             def normal_rot():
@@ -384,6 +387,32 @@ def main():
         except cam.CamError as ex:  # the slice lost its format tag
             log("uniform-expert GEMM skipped: %s" % ex)
         del gsets, ws1, ws2
+        torch.cuda.empty_cache()
+        # Calibration only, never a product path: what the vendor's dense int8 GEMM (hipBLASLt behind
+        # torch._int_mm) sustains on this box at GMM1's shape with random operands.  It fixes what "MFMA-bound"
+        # can mean here: the matrix cores run below their nominal clock once operands toggle and LDS is busy.
+        try:
+            ca = torch.randint(-127, 128, (rows, H), dtype=torch.int8, device=dev)
+            cb = torch.randint(-127, 128, (2 * I, H), dtype=torch.int8, device=dev).t()  # column-major B
+            for _ in range(3):
+                torch._int_mm(ca, cb)
+            torch.cuda.synchronize()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            for _ in range(20):
+                torch._int_mm(ca, cb)
+            e1.record()
+            torch.cuda.synchronize()
+            t_c = e0.elapsed_time(e1) * 1e-3 / 20
+            result["calibration_dense_int8"] = dict(what="torch._int_mm (hipBLASLt), M 8192 x K 7168 x N 4096, "
+                                                         "random int8 operands, column-major B; calibration only",
+                                                    us=t_c * 1e6, tops=ops1 / t_c / 1e12,
+                                                    frac_int8_peak=ops1 / t_c / INT8_PEAK)
+            log("calibration: dense int8 GEMM through torch._int_mm %.1f us -> %.0f TOPS" % (t_c * 1e6,
+                                                                                            ops1 / t_c / 1e12))
+            del ca, cb
+        except Exception as ex:  # noqa: BLE001 - the calibration is optional
+            log("dense int8 calibration skipped: %s" % ex)
         torch.cuda.empty_cache()
 
     # ------------------------------------------------------------------ whole fused layers
