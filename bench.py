@@ -282,6 +282,33 @@ def main():
             result["combine_decode"] = dict(tokens=Td, us=us(s_cd), gb_per_s=cd_bytes / s_cd["mean"] / 1e9,
                                             bytes=cd_bytes)
             del wss, yd, od
+            # rows quantised for the wire (int8 + one bf16 scale per 8 columns): the gather reads 1.25 bytes per
+            # element instead of 2 and rebuilds the bf16 value before weighting it
+            gen = torch.Generator(device=dev).manual_seed(49)
+            wire = []
+            for i in range(NBUF):
+                q = torch.randint(-127, 128, (A, H), generator=gen, dtype=torch.int8, device=dev)
+                sc = (torch.rand((A, H // 8), generator=gen, device=dev) * 0.02 + 0.001).bfloat16()
+                wire.append(torch.cat([q.view(torch.uint8), sc.view(torch.uint8).reshape(A, H // 4)], dim=1)
+                            .view(torch.int8).contiguous())
+                del q, sc
+
+            def comb_wire():
+                for i in range(ROT):
+                    d = dsets[i % NBUF]
+                    _lib.call("MoeCombineGather", [wire[i % NBUF], None, d["slot"], d["rcnt"], gw, couts[i % NBUF]])
+
+            s_cw = spread(graph_of(comb_wire), ROT, SPREAD_REPLAYS)
+            wire_bytes = A * (H + H // 4) + A * 4 + A * 4 + T * H * 2
+            kernels["combine_gather_wire_rows"] = dict(bound="hbm", us=us(s_cw), bytes=wire_bytes,
+                                                       achieved=wire_bytes / s_cw["mean"] / 1e9,
+                                                       peak=HBM_PEAK / 1e9, unit="GB/s",
+                                                       frac=wire_bytes / s_cw["mean"] / HBM_PEAK,
+                                                       note="MoeCombineGather over int8 wire rows (8-column blocks, "
+                                                            "bf16 block scales): 1.25 bytes per element read")
+            log("combine from wire rows: %.1f us -> %.0f GB/s of its own %.1f MB"
+                % (s_cw["mean"] * 1e6, wire_bytes / s_cw["mean"] / 1e9, wire_bytes / 1e6))
+            del wire
         del xs, ys, dsets, couts
         torch.cuda.empty_cache()
 

@@ -249,7 +249,12 @@ CAM_API camStatus camMoeCombineNormal(void *workspace, uint64_t workspaceSize, c
  *   names points back at that slot, so a slotRow built by MoeCombineIndex needs no initialisation; when NULL,
  *   slotRow is trusted (entries < 0 are skipped), which is what the dispatch operators' slotRow output is for.
  *   epRecvCountsOptional int32 [E]: when given, rows at or past its last element are never read.
- *   Same arithmetic and limits as MoeCombineNormal. */
+ *   Same arithmetic and limits as MoeCombineNormal.
+ *   recvX may instead hold rows quantised for the wire, int8 [A, H + H/4] (H = out's columns): H int8 values,
+ *   then one bf16 scale per block of 8 columns -- the int8 communication quantisation of
+ *   AK/moe_combine_shmem/op_kernel/moe_combine_shmem.h:564-592.  Each value is rebuilt as
+ *   bf16(float(q) * float(scale)) (:755-773) before it is weighted and summed.  GroupedMatmulDequant writes
+ *   such rows when its out tensor is int8. */
 CAM_API camStatus camMoeCombineIndexGetWorkspaceSize(const camTensor *tokenSrcInfo, int64_t numRows,
                                                      const camTensor *slotRow, uint64_t *workspaceSize,
                                                      camOpExecutor **executor);
@@ -295,7 +300,12 @@ CAM_API camStatus camGroupedMatmulSwigluQuant(void *workspace, uint64_t workspac
  * FDM/gemm/kernel/grouped_matmul_slice_m_per_token_dequant_multistage_workspace.h:24-378; epilogue
  * FDM/epilogue/block/block_epilogue_per_token_dequant.hpp:572-703).
  * x int8 [A,I]; xScale fp32 [A]; weight list [G,I,H] / G x [I,H], CAM_FORMAT_MFMA_B with gateUp=0;
- * weightScale fp32 [G,H] -> out bf16 [A,H] = bf16((float(acc) * weightScale[g][h]) * xScale[m]). */
+ * weightScale fp32 [G,H] -> out bf16 [A,H] = bf16((float(acc) * weightScale[g][h]) * xScale[m]).
+ * out int8 [A, H + H/4] selects wire rows instead: every bf16 row above is quantised in blocks of 8 columns as
+ * AK/moe_combine_shmem/op_kernel/moe_combine_shmem.h:567-592 does before a row leaves the rank:
+ *   m = max |x| over the block; s = m * (1/127); q = int8(half(x / s)) (both casts round to nearest even);
+ *   the row is the H values q followed by the H/8 scales bf16(s); an all-zero block gives q = 0, scale 0
+ *   (0/0 in the reference).  The workspace then also holds the bf16 rows. */
 CAM_API camStatus camGroupedMatmulDequantGetWorkspaceSize(
     const camTensor *x, const camTensor *xScale, const camTensorList *weight, const camTensorList *weightScale,
     const camTensor *groupList, int64_t groupListType, const camTensor *out, uint64_t *workspaceSize,

@@ -428,6 +428,101 @@ ORACLE_API void cam_oracle_combine(const uint16_t *y, const int32_t *row_of, con
     }
 }
 
+/* ---------------------------------------------------------------- A.10b combine rows quantised for the wire
+ * AK/moe_combine_shmem/op_kernel/moe_combine_shmem.h (IsQuant instantiation).
+ * A quantised row is H int8 values followed by H/8 scales in the activation type (:564, :570-571, :781):
+ * blocks of 8 columns (one BlockReduceMax result per 32-byte block of fp32, :301-305, :577).
+ *   quantise (:567-592):  xf = float(x);  m = max |xf| over the block;  s = m * (1/127) (:300, :579);
+ *     stored scale = bf16_rne(s) (:581);  q = int8_rne(fp16_rne(xf / s)) with the UNROUNDED s (:583-589).
+ *   dequantise (:755-773):  v = bf16_rne(float(q) * float(stored scale)).
+ * Deliberate definitions: an all-zero block (0/0 in the reference) gives q = 0 and scale 0; Div is taken to be
+ * the IEEE correctly rounded quotient ("parity unpinned" against the Ascend Div instruction bit for bit). */
+static inline uint16_t f32_to_fp16(float f)
+{
+    uint32_t u;
+    memcpy(&u, &f, 4);
+    uint32_t sign = (u >> 16) & 0x8000u;
+    uint32_t absu = u & 0x7fffffffu;
+    if (absu >= 0x7f800000u) { /* inf / nan */
+        return (uint16_t)(sign | 0x7c00u | ((absu > 0x7f800000u) ? 0x200u : 0u));
+    }
+    if (absu >= 0x477ff000u) { /* rounds to 65520 or more: overflow to inf */
+        return (uint16_t)(sign | 0x7c00u);
+    }
+    if (absu < 0x33000001u) { /* at most half the smallest subnormal (2^-25): rounds to zero */
+        return (uint16_t)sign;
+    }
+    int32_t e = (int32_t)(absu >> 23) - 127;
+    uint32_t man = (absu & 0x7fffffu) | 0x800000u; /* 24-bit significand */
+    int shift;                                     /* bits dropped from the significand */
+    uint32_t base;
+    if (e < -14) { /* subnormal result: value = man * 2^(e-23), unit 2^-24 */
+        shift = -e - 1;  /* (e - 23) - (-24) = e + 1 -> drop -(e+1) bits */
+        base = 0;
+    } else {
+        shift = 13;
+        base = (uint32_t)(e + 15) << 10;
+        man &= 0x7fffffu;
+    }
+    uint32_t kept = man >> shift;
+    uint32_t rem = man & ((1u << shift) - 1u);
+    uint32_t half = 1u << (shift - 1);
+    if (rem > half || (rem == half && (kept & 1u))) {
+        ++kept; /* a carry out of the mantissa moves into the exponent field, which is what is wanted */
+    }
+    return (uint16_t)(sign | (base + kept));
+}
+
+ORACLE_API uint16_t cam_oracle_f32_to_fp16(float x) { return f32_to_fp16(x); }
+
+#define CAM_COMMQ_BLOCK 8
+
+/* x [A,H] bf16 bits -> out [A, H + H/4] bytes */
+ORACLE_API void cam_oracle_comm_quant_rows(const uint16_t *x, int64_t A, int64_t H, uint8_t *out)
+{
+    const int64_t pitch = H + H / 4;
+#pragma omp parallel for schedule(static)
+    for (int64_t r = 0; r < A; ++r) {
+        const uint16_t *xr = x + r * H;
+        int8_t *q = (int8_t *)(out + r * pitch);
+        uint16_t *sc = (uint16_t *)(out + r * pitch + H);
+        for (int64_t b = 0; b < H / CAM_COMMQ_BLOCK; ++b) {
+            float m = 0.0f;
+            for (int j = 0; j < CAM_COMMQ_BLOCK; ++j) {
+                float a = fabsf(bf16_to_f32(xr[b * CAM_COMMQ_BLOCK + j]));
+                m = a > m ? a : m;
+            }
+            if (m == 0.0f) {
+                sc[b] = 0;
+                for (int j = 0; j < CAM_COMMQ_BLOCK; ++j) {
+                    q[b * CAM_COMMQ_BLOCK + j] = 0;
+                }
+                continue;
+            }
+            float s = m * (1.0f / 127.0f);
+            sc[b] = f32_to_bf16(s);
+            for (int j = 0; j < CAM_COMMQ_BLOCK; ++j) {
+                float v = bf16_to_f32(xr[b * CAM_COMMQ_BLOCK + j]) / s;
+                q[b * CAM_COMMQ_BLOCK + j] = (int8_t)nearbyintf(fp16_to_f32(f32_to_fp16(v)));
+            }
+        }
+    }
+}
+
+/* packed [A, H + H/4] -> bf16 bits [A,H] */
+ORACLE_API void cam_oracle_comm_dequant_rows(const uint8_t *packed, int64_t A, int64_t H, uint16_t *out)
+{
+    const int64_t pitch = H + H / 4;
+#pragma omp parallel for schedule(static)
+    for (int64_t r = 0; r < A; ++r) {
+        const int8_t *q = (const int8_t *)(packed + r * pitch);
+        const uint16_t *sc = (const uint16_t *)(packed + r * pitch + H);
+        for (int64_t h = 0; h < H; ++h) {
+            out[r * H + h] = f32_to_bf16((float)q[h] * bf16_to_f32(sc[h / CAM_COMMQ_BLOCK]));
+        }
+    }
+}
+
 /* row_of for the fused op: off[e] + pos (cam_moe_distribute_combine.h:737-742), -1 where idx < 0. */
 ORACLE_API void cam_oracle_rows_from_pos(const int64_t *idx, const int32_t *off, const int32_t *pos,
                                          int64_t n, int64_t E, int32_t *row_of)

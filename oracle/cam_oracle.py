@@ -228,6 +228,33 @@ def combine(y_bits, row_of, w):
     return out
 
 
+def f32_to_fp16_bits(a):
+    a = _c(a, np.float32)
+    f = lib().cam_oracle_f32_to_fp16
+    f.restype = ctypes.c_uint16
+    f.argtypes = [ctypes.c_float]
+    return np.array([f(float(v)) for v in a.ravel()], np.uint16).reshape(a.shape)
+
+
+def comm_quant_rows(y_bits):
+    """bf16 rows [A,H] -> wire rows [A, H + H/4] uint8: H int8 values, then H/8 bf16 block scales."""
+    y_bits = _c(y_bits, np.uint16)
+    A, H = y_bits.shape
+    assert H % 8 == 0
+    out = np.zeros((A, H + H // 4), np.uint8)
+    lib().cam_oracle_comm_quant_rows(_p(y_bits), _i64(A), _i64(H), _p(out))
+    return out
+
+
+def comm_dequant_rows(packed, H):
+    packed = _c(packed, np.uint8)
+    A = packed.shape[0]
+    assert packed.shape[1] == H + H // 4
+    out = np.zeros((A, H), np.uint16)
+    lib().cam_oracle_comm_dequant_rows(_p(packed), _i64(A), _i64(H), _p(out))
+    return out
+
+
 def fused_layer(x_bits, idx, topk_w, w1, w1_scale, w2, w2_scale, n_active=None, debug=False):
     """One rank's whole layer. w1 [E,H,2I] int8, w2 [E,I,H] int8. Returns (out bits, expert_token_nums[, dbg])."""
     x_bits = _c(x_bits, np.uint16)

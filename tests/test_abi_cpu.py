@@ -163,6 +163,12 @@ def test_combine_gather_validation():
     a = list(ok)
     a[2] = _t((T, K + 1), torch.int32)
     assert _lib.phase1("MoeCombineGather", a)[0] == CAM_ERR_SHAPE
+    # rows quantised for the wire: int8 [A, H + H/4]
+    a = list(ok)
+    a[0] = _t((A, H + H // 4), torch.int8)
+    assert _lib.phase1("MoeCombineGather", a)[0] == CAM_OK
+    a[0] = _t((A, H), torch.int8)
+    assert _lib.phase1("MoeCombineGather", a)[0] == CAM_ERR_SHAPE
 
 
 def _packed(shape):
@@ -239,6 +245,11 @@ def test_gemm_and_prepack_validation():
     deq[3] = [_t((2, 128), torch.float32)]
     deq[6] = _t((10 * 128 + 1,), torch.bfloat16)[1:].view(10, 128)
     assert _lib.phase1("GroupedMatmulDequant", deq)[0] == CAM_ERR_ALIGN
+    deq[6] = _t((10, 160), torch.int8)  # wire rows: N + N/4 columns of int8
+    st, ws_wire, _ = _lib.phase1("GroupedMatmulDequant", deq)
+    assert st == CAM_OK and ws_wire >= 10 * 128 * 2
+    deq[6] = _t((10, 128), torch.int8)
+    assert _lib.phase1("GroupedMatmulDequant", deq)[0] == CAM_ERR_SHAPE
 
 
 def test_phase2_rejects_wrong_executor_and_small_workspace():

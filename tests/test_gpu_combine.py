@@ -54,6 +54,43 @@ def test_combine_full_size_config(gpu, oracle):
     assert torch.isfinite(got.float()).all()
 
 
+def _wire_case(gpu, oracle, T, K, E, H, seed):
+    ids, w = synth.sigmoid_zipf_routing(T, E, K, seed=seed)
+    idx_np = ids.numpy()
+    cnt, off, pos, _ = plan_oracle(oracle, idx_np, E)
+    A = T * K
+    y = synth.normal_bf16(A, H, seed=seed + 1)
+    y[0] = 0  # an all-zero row: q = 0, scale 0
+    if A > 2:   # tiny and huge rows: scales and rebuilt values at both ends of the bf16 range
+        y[1] = (y[1].float() * 1e-37).bfloat16()
+        y[2] = (y[2].float() * 1e36).bfloat16()
+    packed = oracle.comm_quant_rows(synth.bf16_bits(y))
+    row_of = oracle.rows_from_pos(idx_np, off, pos, E)
+    want = oracle.combine(oracle.comm_dequant_rows(packed, H), row_of, w.numpy())
+    got = cam.moe_combine_gather(torch.from_numpy(packed.view(np.int8)).to(gpu), None,
+                                 torch.from_numpy(row_of.reshape(T, K)).to(gpu), w.to(gpu))
+    assert got.dtype == torch.bfloat16 and got.shape == (T, H)
+    assert_bits_equal(to_np(got), want, "combined x from wire rows")
+    return y, packed, row_of, w, got
+
+
+@pytest.mark.parametrize("T,K,E,H", [(1, 1, 2, 1024), (33, 8, 64, 7168), (57, 16, 32, 4096), (21, 3, 8, 1032)])
+def test_combine_from_wire_rows_bit_exact(gpu, oracle, T, K, E, H):
+    """Rows quantised for the wire (int8 + bf16 scale per 8 columns) are dequantised inside the gather."""
+    announce("combine from wire rows T=%d K=%d E=%d H=%d" % (T, K, E, H))
+    _wire_case(gpu, oracle, T, K, E, H, seed=T + K + 5)
+
+
+def test_combine_from_wire_rows_full_size(gpu, oracle):
+    """C4 shape with wire rows: bit-exact against the oracle, and close to the combine of the unquantised rows."""
+    announce("combine from wire rows, C4 full size")
+    T, K, E, H = 4096, 8, 256, 7168
+    y, packed, row_of, w, got = _wire_case(gpu, oracle, T, K, E, H, seed=46)
+    exact = cam.moe_combine_gather(y.to(gpu), None, torch.from_numpy(row_of.reshape(T, K)).to(gpu), w.to(gpu))
+    diff = (got.float() - exact.float()).abs().max().item()
+    assert diff <= 0.02 * exact.float().abs().max().item() + 1e-3
+
+
 def test_combine_identity_and_linearity(gpu, oracle):
     announce("combine properties")
     T, K, E, H = 256, 1, 16, 1024

@@ -98,6 +98,23 @@ def test_gmm2_dequant_bit_exact(gpu, oracle, sizes, I, H):
     assert_bits_equal(to_np(out)[:A], want[:A], "bf16 output")
 
 
+@pytest.mark.parametrize("sizes,I,H", [([4, 0, 131, 60], 128, 256), ([300, 77], 512, 1024)])
+def test_gmm2_wire_rows_bit_exact(gpu, oracle, sizes, I, H):
+    """GroupedMatmulDequant with an int8 output: the bf16 rows quantised for the wire in 8-column blocks."""
+    announce("gmm2 wire rows sizes=%s I=%d H=%d" % (sizes, I, H))
+    a, w, gl, A = _inputs(sizes, I, H, seed=I + H + 1, wrange=16)
+    G = len(sizes)
+    ws = synth.channel_scales((G, H), seed=35)
+    xs = synth.channel_scales((max(A, 1),), seed=36, lo=0.001, hi=0.01)
+    wp = cam.prepack_weight(w.to(gpu), False)
+    packed = cam.grouped_matmul_dequant(a.to(gpu), xs.to(gpu), wp, ws.to(gpu), gl.to(gpu), wire_rows=True)
+    assert packed.dtype == torch.int8 and packed.shape == (max(A, 1), H + H // 4)
+    c = oracle.gmm_int32(a.numpy(), w.numpy(), gl.numpy())
+    rows = oracle.gmm2_epilogue(c, ws.numpy(), xs.numpy(), gl.numpy())
+    want = oracle.comm_quant_rows(rows[:A])
+    assert np.array_equal(packed.cpu().numpy().view(np.uint8)[:A], want), "wire rows"
+
+
 def test_full_size_grouped_gemm_sampled_rows(gpu):
     """One GPU's 32 local experts at the benchmark shape; sampled rows against an exact CPU integer matmul."""
     announce("gemm C3 full size, sampled rows")

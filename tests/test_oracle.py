@@ -416,6 +416,86 @@ def test_combine_identity_mean_and_no_fma(oracle):
     assert (oracle.bf16_bits_to_f32(out) == 0.0).all()  # fused arithmetic would leave a residue
 
 
+# ------------------------------------------------------------------ rows quantised for the wire
+def test_f32_to_fp16_matches_numpy(oracle):
+    rng = np.random.default_rng(11)
+    f = rng.integers(0, 2 ** 32, size=60000, dtype=np.uint64).astype(np.uint32).view(np.float32)
+    f = f[np.isfinite(f)]
+    edge = np.array([0.0, -0.0, 65504.0, 65519.99, 65520.0, 65536.0, 6.1e-5, 5.96e-8, 2.98e-8, 2.9802322e-8,
+                     2.9802326e-8, 1.4999, 1.5, 2.5, 0.5, 1e-10, -1.49999, 127.03125, 100.3], np.float32)
+    f = np.concatenate([f, edge, rng.uniform(-130, 130, 40000).astype(np.float32)])
+    with np.errstate(over="ignore"):
+        want = f.astype(np.float16).view(np.uint16)
+    assert np.array_equal(oracle.f32_to_fp16_bits(f), want)
+
+
+def _comm_quant_numpy(x_bits):
+    """The wire quantisation with numpy's own float32 / float16 arithmetic (independent of the C code)."""
+    xf = oracle_bits_to_f32(x_bits)
+    A, H = xf.shape
+    blk = xf.reshape(A, H // 8, 8)
+    m = np.max(np.abs(blk), axis=2).astype(np.float32)
+    s = (m * np.float32(1.0 / 127.0)).astype(np.float32)
+    with np.errstate(divide="ignore", invalid="ignore"):
+        v = (blk / s[:, :, None]).astype(np.float32)
+    q = np.rint(v.astype(np.float16).astype(np.float32))
+    q[m == 0] = 0
+    return q.astype(np.int8).reshape(A, H), s
+
+
+def oracle_bits_to_f32(bits):
+    return (bits.astype(np.uint32) << 16).view(np.float32)
+
+
+def test_comm_quant_rows_definition_and_layout(oracle):
+    A, H = 37, 1024
+    x = synth.normal_bf16(A, H, seed=71)
+    x[3] = 0                      # all-zero row: every block q = 0, scale 0
+    x[4, :8] = 0                  # one zero block in a live row
+    x[5, 8:16] = torch.tensor([2.0, -2.0, 2.0, 2.0, -2.0, 2.0, 2.0, -2.0])  # equal magnitudes -> +-127
+    x[6, 16:24] = torch.tensor([1.0, 0.5, 0.25, -0.125, 0.0, 1.0, -1.0, 0.0625])
+    bits = synth.bf16_bits(x)
+    packed = oracle.comm_quant_rows(bits)
+    assert packed.shape == (A, H + H // 4) and packed.dtype == np.uint8
+    q = packed[:, :H].view(np.int8)
+    sc_bits = np.ascontiguousarray(packed[:, H:]).view(np.uint16)
+    assert sc_bits.shape == (A, H // 8)
+    want_q, s = _comm_quant_numpy(bits)
+    assert np.array_equal(q, want_q)
+    assert np.array_equal(sc_bits, oracle.f32_to_bf16_bits(s))
+    assert not q[3].any() and not sc_bits[3].any() and not q[4, :8].any() and sc_bits[4, 0] == 0
+    assert np.array_equal(q[5, 8:16], np.array([127, -127, 127, 127, -127, 127, 127, -127], np.int8))
+    # every live block reaches +-127 at its largest element and nothing exceeds it
+    live = s > 0
+    assert (np.abs(q.astype(np.int32)).reshape(A, H // 8, 8).max(axis=2)[live] == 127).all()
+    # dequantised values: bf16(q * bf16(scale)), within one quantisation step (plus bf16 rounding) of the input
+    back = oracle.comm_dequant_rows(packed, H)
+    scf = oracle_bits_to_f32(sc_bits)
+    want_back = oracle.f32_to_bf16_bits((q.astype(np.float32).reshape(A, H // 8, 8) * scf[:, :, None]).reshape(A, H))
+    assert np.array_equal(back, want_back)
+    err = np.abs(oracle_bits_to_f32(back) - oracle_bits_to_f32(bits)).reshape(A, H // 8, 8)
+    assert (err <= scf[:, :, None] * 0.51 + np.abs(oracle_bits_to_f32(bits)).reshape(A, H // 8, 8) * 2 ** -6 + 1e-30).all()
+
+
+def test_comm_quant_double_rounding_is_kept(oracle):
+    """x / s just below a half-integer rounds up to it in fp16 and then to the even neighbour: the reference casts
+    float -> half -> int8 (moe_combine_shmem.h:587-589), and so must a restatement."""
+    # block maximum 127 makes s = 127 * (1/127), which is 1 up to rounding; 1.4990234375 is a bf16 value whose fp16
+    # image is itself, so pick a neighbour scale instead: search a few blocks for a case where the two roundings differ.
+    rng = np.random.default_rng(5)
+    x = synth.bf16_bits(torch.from_numpy(rng.uniform(-3, 3, size=(4000, 8)).astype(np.float32)).bfloat16())
+    xf = oracle_bits_to_f32(x)
+    m = np.max(np.abs(xf), axis=1).astype(np.float32)
+    s = (m * np.float32(1.0 / 127.0)).astype(np.float32)
+    v = (xf / s[:, None]).astype(np.float32)
+    direct = np.rint(v)
+    via_half = np.rint(v.astype(np.float16).astype(np.float32))
+    rows = np.nonzero((direct != via_half).any(axis=1))[0]
+    assert len(rows) > 0, "the sample holds no double-rounding case"
+    packed = oracle.comm_quant_rows(x[rows])
+    assert np.array_equal(packed[:, :8].view(np.int8), via_half[rows].astype(np.int8))
+
+
 def test_rows_from_src_info_inverts_dispatch(oracle):
     T, K, E, H = 31, 3, 6, 16
     ids, _ = synth.softmax_topk_routing(T, E, K, seed=16)

@@ -1026,12 +1026,18 @@ camStatus camMoeCombineGatherGetWorkspaceSize(const camTensor *recvX, const camT
                                               const camTensor *recvTopkWeights, const camTensor *out,
                                               uint64_t *workspaceSize, camOpExecutor **executor)
 {
-    CAM_TRY(check_tensor(recvX, "recvX", 2, CAM_DT_BF16));
+    // recvX: bf16 rows [A,H], or rows quantised for the wire, int8 [A, H + H/4] (the int8 communication
+    // quantisation of AK/moe_combine_shmem/op_kernel/moe_combine_shmem.h:564-592, dequantised as :755-773).
+    CAM_TRY(check_tensor(recvX, "recvX", 2, CAM_DT_BF16, CAM_DT_INT8));
     CAM_TRY(check_tensor(slotRow, "slotRow", 2, CAM_DT_INT32));
     CAM_TRY(check_tensor(recvTopkWeights, "recvTopkWeights", 2, CAM_DT_FLOAT));
     CAM_TRY(check_tensor(out, "out", 2, CAM_DT_BF16));
-    const int64_t A = recvX->sizes[0], H = recvX->sizes[1];
+    const bool wire = recvX->dtype == CAM_DT_INT8;
+    const int64_t A = recvX->sizes[0], H = out->sizes[1];
     const int64_t T = recvTopkWeights->sizes[0], K = recvTopkWeights->sizes[1];
+    if (recvX->sizes[1] != (wire ? H + H / 4 : H)) {
+        return fail(CAM_ERR_SHAPE, "recvX must be [A,H] bf16 or [A, H + H/4] int8 wire rows, H = out's columns");
+    }
     if (H < 1024 || H > 7168) {
         return fail(CAM_ERR_RANGE, "hidden size %lld outside [1024, 7168]", (long long)H);
     }
@@ -1076,6 +1082,7 @@ camStatus camMoeCombineGatherGetWorkspaceSize(const camTensor *recvX, const camT
     g.K = (int)K;
     g.H = (int)H;
     g.A = A;
+    g.wire_rows = wire ? 1 : 0;
     g.out = (uint16_t *)out->data;
     auto run = [g](void *, hipStream_t s) -> hipError_t { return cam::launch_combine(g, s); };
     return finish_phase1(kOpCombGather, 0, run, workspaceSize, executor);
@@ -1240,8 +1247,14 @@ camStatus camGroupedMatmulDequantGetWorkspaceSize(const camTensor *x, const camT
 {
     GemmCommon gc{};
     CAM_TRY(check_gemm_inputs("GroupedMatmulDequant", x, xScale, true, groupList, groupListType, &gc));
-    CAM_TRY(check_tensor(out, "out", 2, CAM_DT_BF16));
-    const int64_t N = out->sizes[1];
+    // out: bf16 [A,N], or int8 [A, N + N/4]: the bf16 rows quantised for the wire on their way out (blocks of 8
+    // columns, AK/moe_combine_shmem/op_kernel/moe_combine_shmem.h:564-592), which MoeCombineGather reads back.
+    CAM_TRY(check_tensor(out, "out", 2, CAM_DT_BF16, CAM_DT_INT8));
+    const bool wire = out->dtype == CAM_DT_INT8;
+    if (wire && out->sizes[1] % 10 != 0) {
+        return fail(CAM_ERR_SHAPE, "int8 out must be [A, N + N/4] with N a multiple of 8");
+    }
+    const int64_t N = wire ? out->sizes[1] / 5 * 4 : out->sizes[1];
     if (out->sizes[0] != gc.A) {
         return fail(CAM_ERR_SHAPE, "out must have one row per row of x");
     }
@@ -1252,6 +1265,7 @@ camStatus camGroupedMatmulDequantGetWorkspaceSize(const camTensor *x, const camT
     cam::SchedSpec sp = sched_spec(gc.A, gc.G, N);
     Carver c;
     const uint64_t o_sched = c.take(cam::sched_bytes(gc.A, (int)gc.G, (int)N));
+    const uint64_t o_rows = wire ? c.take((uint64_t)gc.A * N * 2) : 0;  // the bf16 rows before quantisation
     cam::GemmArgs g{};
     g.a = (const int8_t *)x->data;
     g.a_scale = (const float *)xScale->data;
@@ -1264,6 +1278,7 @@ camStatus camGroupedMatmulDequantGetWorkspaceSize(const camTensor *x, const camT
     g.gate_up = 0;
     g.epilogue = cam::kEpiDequantBf16;
     g.out = out->data;
+    uint8_t *wire_out = (uint8_t *)out->data;
     auto run = [=](void *wsp, hipStream_t s) mutable -> hipError_t {
         sp.sched = (int32_t *)((char *)wsp + o_sched);
         hipError_t e = cam::launch_build_sched(gc.group_list, gc.cumulative, (int)gc.G, gc.A, 1, &sp, s);
@@ -1271,7 +1286,16 @@ camStatus camGroupedMatmulDequantGetWorkspaceSize(const camTensor *x, const camT
             return e;
         }
         g.sched = sp.sched;
-        return cam::launch_gemm(g, s);
+        if (!wire) {
+            return cam::launch_gemm(g, s);
+        }
+        uint16_t *rows = (uint16_t *)((char *)wsp + o_rows);
+        g.out = rows;
+        e = cam::launch_gemm(g, s);
+        if (e != hipSuccess) {
+            return e;
+        }
+        return cam::launch_comm_quant(rows, gc.A, g.N, sp.sched + 1, wire_out, s);  // sched[1]: rows that exist
     };
     return finish_phase1(kOpGmm2, c.off, run, workspaceSize, executor);
 }

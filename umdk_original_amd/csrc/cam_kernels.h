@@ -131,7 +131,8 @@ hipError_t launch_dispatch_fused(FusedDispatchArgs a, hipStream_t stream);
 hipError_t launch_invert_src_info(const int32_t *src_info, int64_t A, const int32_t *row_limit, int T, int K,
                                   int32_t *slot_row, hipStream_t stream);
 struct CombineArgs {
-    const uint16_t *y;        // [A,H] bf16 bits
+    const uint16_t *y;        // [A,H] bf16 bits, or wire rows [A, H + H/4] bytes (wire_rows != 0)
+    int wire_rows;            // rows are H int8 values + H/8 bf16 block scales (launch_comm_quant's output)
     const int32_t *slot_row;  // [T,K] row of slot (t,k) (<0: skip)
     const int32_t *src_info;  // optional: when set, slot_row entries are verified against the triples
     const float *w;           // [T,K]
@@ -142,6 +143,10 @@ struct CombineArgs {
     uint16_t *out;            // [T,H]
 };
 hipError_t launch_combine(const CombineArgs &a, hipStream_t stream);
+// bf16 rows [A,H] -> wire rows [A, H + H/4] bytes: per block of 8 columns int8 values and one bf16 scale.
+// row_limit: optional device scalar; rows >= *row_limit are left untouched.
+hipError_t launch_comm_quant(const uint16_t *y, int64_t A, int H, const int32_t *row_limit, uint8_t *out,
+                             hipStream_t stream);
 
 // ---------------------------------------------------------------------------------------------
 // Grouped int8 GEMM.
