@@ -482,6 +482,47 @@ def main():
                                 dtype="int8 weights and activations (w8a8)")
             del w1, w2, wsl, xl, outl
             torch.cuda.empty_cache()
+        # the same two shapes with block-scaled FP8 weights and activations (E4M3, E8M0 scales per 128 / 128 x 128)
+        for name, (Tl, Hl, El, Kl, Il) in {
+            "qwen3_235b_shape_prefill_fp8": (8192, 4096, 128, 8, 1536),
+            "qwen3_235b_shape_decode_fp8": (128, 4096, 128, 8, 1536),
+        }.items():
+            idl, gl_w = synth.sigmoid_zipf_routing(Tl, El, Kl, seed=47)
+            gen = torch.Generator(device=dev).manual_seed(475)
+
+            def fp8_weight(shape):
+                # random E4M3 bit patterns below the NaN code, both signs
+                b = torch.randint(0, 0x78, shape, generator=gen, dtype=torch.uint8, device=dev)
+                b |= (torch.randint(0, 2, shape, generator=gen, dtype=torch.uint8, device=dev) << 7)
+                return b.view(torch.float8_e4m3fn)
+
+            w1 = cam.prepack_weight(fp8_weight((El, Hl, 2 * Il)), True)
+            w2 = cam.prepack_weight(fp8_weight((El, Il, Hl)), False)
+            w1s = torch.randint(112, 118, (El, Hl // 128, 2 * Il // 128), generator=gen, dtype=torch.uint8, device=dev)
+            w2s = torch.randint(112, 118, (El, Il // 128, Hl // 128), generator=gen, dtype=torch.uint8, device=dev)
+            xl = synth.normal_bf16(Tl, Hl, seed=474).to(dev)
+            idl32 = idl.to(torch.int32).to(dev)
+            gl_w = gl_w.to(dev)
+            outl = torch.empty((Tl, Hl), dtype=torch.bfloat16, device=dev)
+            etn = torch.empty(El, dtype=torch.int64, device=dev)
+            fargs = [xl, idl32, w1, w1s, w2, w2s, gl_w, None, El, outl, etn]
+            st, ws_bytes, msg = _lib.phase1("FusedDeepMoeFp8", fargs)
+            assert st == 0, msg
+            wsl = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
+
+            def layer8():
+                _lib.call("FusedDeepMoeFp8", fargs, workspace=wsl)
+
+            s_l = spread(graph_of(layer8), 1, max(10, min(SPREAD_REPLAYS, K_STEPS // 4)))
+            ops = synth.gemm_ops(Tl * Kl, Hl, Il)
+            log("fused layer %s: %.1f us (median %.1f; %.0f TFLOP/s)" % (name, s_l["mean"] * 1e6, s_l["median"] * 1e6,
+                                                                         ops / s_l["mean"] / 1e12))
+            layers[name] = dict(us=s_l["mean"] * 1e6, us_spread=us(s_l), tokens=Tl, hidden=Hl, experts=El, top_k=Kl,
+                                intermediate=Il, tops=ops / s_l["mean"] / 1e12, workspace_bytes=ws_bytes,
+                                dtype="fp8 e4m3 weights and activations, e8m0 scales per 128 (activations) and "
+                                      "128 x 128 (weights), fp32 accumulation")
+            del w1, w2, wsl, xl, outl, fargs
+            torch.cuda.empty_cache()
         result["fused_layer_us"] = layers
 
     # ------------------------------------------------------------------ CPU baseline (the oracle on the host cores)

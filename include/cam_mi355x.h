@@ -60,7 +60,8 @@ enum {
     CAM_DT_UINT8 = 4,
     CAM_DT_INT64 = 9,
     CAM_DT_BOOL = 12,
-    CAM_DT_BF16 = 27
+    CAM_DT_BF16 = 27,
+    CAM_DT_FLOAT8_E4M3FN = 36      /* OCP FP8 E4M3 (block-scaled FP8 operators only) */
 };
 
 /* Storage formats.  CAM_FORMAT_ND is plain row-major.  CAM_FORMAT_MFMA_B is the weight layout
@@ -347,6 +348,44 @@ CAM_API camStatus camFusedDeepMoeGetWorkspaceSize(
     const camTensor *expertTokenNums, uint64_t *workspaceSize, camOpExecutor **executor);
 CAM_API camStatus camFusedDeepMoe(void *workspace, uint64_t workspaceSize, camOpExecutor *executor,
                                   camStream_t stream);
+
+/* ------------------------------------------------------------------------------------------------
+ * Block-scaled FP8 variant of the layer.  No counterpart in the reference, whose fused operator is W8A8 int8
+ * only (src/cam/README.md:20-21); the arithmetic is defined in cam_fp8_spec.h: OCP E4M3 values, one E8M0
+ * (power-of-two) scale per activation row and 128 columns of K and per 128 x 128 block of a weight, fp32
+ * accumulation.  Results are compared with a tolerance (bf16 outputs within 1e-2 relative), not bit for bit;
+ * the quantised activations themselves are exact.
+ *
+ * MoeDispatchPrefill with quantMode 4 produces the quantised rows (recvX E4M3 [A,H], recvXScales uint8 [A,H/128]).
+ *
+ * GroupedMatmulFp8: x E4M3 [A,K]; xScale uint8 [A,K/128]; weight E4M3 [G,K,N], CAM_FORMAT_MFMA_B (PrepackWeight
+ *   with the same gateUp); weightScale uint8 [G,K/128,N/128]; groupList int64 [G] as for the int8 operators.
+ *   gateUp == 0: out fp32 [A,N] (the sums) or bf16 [A,N];  gateUp != 0: out fp32 [A,N/2] = silu(gate) * up with
+ *   gate = columns [0,N/2) and up = [N/2,N) of the logical weight, as in the int8 layer.
+ * QuantRowsFp8: x fp32 [A,I] -> q E4M3 [A,I], scale uint8 [A,I/128] (the re-quantisation between the two GEMMs).
+ * FusedDeepMoeFp8: x bf16 [bs,H]; expertIds int32 [bs,K]; gmm1Weight E4M3 [E,H,2I] (MFMA_B, gateUp=1) with
+ *   gmm1WeightScale uint8 [E,H/128,2I/128]; gmm2Weight E4M3 [E,I,H] (MFMA_B, gateUp=0) with gmm2WeightScale
+ *   uint8 [E,I/128,H/128]; expertScales fp32 [bs,K]; xActiveMaskOptional as FusedDeepMoe
+ *   -> output bf16 [bs,H], expertTokenNums int64 [E].  One rank; 1024 <= H <= 7168, H and I multiples of 128,
+ *   K <= 16. */
+CAM_API camStatus camGroupedMatmulFp8GetWorkspaceSize(const camTensor *x, const camTensor *xScale,
+                                                      const camTensor *weight, const camTensor *weightScale,
+                                                      int64_t gateUp, const camTensor *groupList,
+                                                      int64_t groupListType, const camTensor *out,
+                                                      uint64_t *workspaceSize, camOpExecutor **executor);
+CAM_API camStatus camGroupedMatmulFp8(void *workspace, uint64_t workspaceSize, camOpExecutor *executor,
+                                      camStream_t stream);
+CAM_API camStatus camQuantRowsFp8GetWorkspaceSize(const camTensor *x, const camTensor *q, const camTensor *scale,
+                                                  uint64_t *workspaceSize, camOpExecutor **executor);
+CAM_API camStatus camQuantRowsFp8(void *workspace, uint64_t workspaceSize, camOpExecutor *executor,
+                                  camStream_t stream);
+CAM_API camStatus camFusedDeepMoeFp8GetWorkspaceSize(
+    const camTensor *x, const camTensor *expertIds, const camTensor *gmm1Weight, const camTensor *gmm1WeightScale,
+    const camTensor *gmm2Weight, const camTensor *gmm2WeightScale, const camTensor *expertScales,
+    const camTensor *xActiveMaskOptional, int64_t moeExpertNum, const camTensor *output,
+    const camTensor *expertTokenNums, uint64_t *workspaceSize, camOpExecutor **executor);
+CAM_API camStatus camFusedDeepMoeFp8(void *workspace, uint64_t workspaceSize, camOpExecutor *executor,
+                                     camStream_t stream);
 
 #ifdef __cplusplus
 }

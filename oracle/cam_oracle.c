@@ -27,6 +27,7 @@
 #include <math.h>
 
 #include "../include/cam_expf_spec.h"
+#include "../include/cam_fp8_spec.h"
 
 #ifdef _OPENMP
 #include <omp.h>
@@ -613,4 +614,112 @@ ORACLE_API int cam_oracle_fused_layer(const uint16_t *x, const int64_t *idx, con
     free(cnt); free(off); free(in_rank); free(gl); free(pos); free(row_of); free(x1); free(x1s);
     free(c1); free(d); free(x2); free(x2s); free(c2); free(y);
     return 0;
+}
+
+/* ================================================================ block-scaled FP8 layer
+ * No counterpart in the reference (W8A8 only, src/cam/README.md:20-21): these functions evaluate the definition
+ * in include/cam_fp8_spec.h.  The matrix products accumulate in double and round once to fp32, which is what a
+ * tolerance test of an fp32-accumulating kernel should be measured against. */
+ORACLE_API float cam_oracle_e4m3_to_f32(uint8_t v) { return cam_e4m3_to_f32(v); }
+ORACLE_API uint8_t cam_oracle_f32_to_e4m3(float x) { return cam_f32_to_e4m3(x); }
+ORACLE_API int cam_oracle_fp8_block_scale_exp(float amax) { return cam_fp8_block_scale_exp(amax); }
+
+/* x [A,H] fp32 -> q [A,H] e4m3 bytes, scale [A, H/128] e8m0 bytes.  H % 128 == 0. */
+ORACLE_API void cam_oracle_fp8_quant_rows_f32(const float *x, int64_t A, int64_t H, uint8_t *q, uint8_t *scale)
+{
+    const int64_t nb = H / CAM_FP8_BLOCK;
+#pragma omp parallel for schedule(static)
+    for (int64_t r = 0; r < A; ++r) {
+        for (int64_t b = 0; b < nb; ++b) {
+            const float *xb = x + r * H + b * CAM_FP8_BLOCK;
+            float m = 0.0f;
+            for (int j = 0; j < CAM_FP8_BLOCK; ++j) {
+                float a = fabsf(xb[j]);
+                m = a > m ? a : m;
+            }
+            const int e = cam_fp8_block_scale_exp(m);
+            scale[r * nb + b] = cam_e8m0_from_exp(e);
+            /* x * 2^-e in two exact steps so that neither factor leaves the normal range */
+            const float f1 = cam_exp2_int(-(e / 2)), f2 = cam_exp2_int(-(e - e / 2));
+            for (int j = 0; j < CAM_FP8_BLOCK; ++j) {
+                q[r * H + b * CAM_FP8_BLOCK + j] = cam_f32_to_e4m3((xb[j] * f1) * f2);
+            }
+        }
+    }
+}
+
+/* the same from bf16 (act == 0) or fp16 (act == 1) activations */
+ORACLE_API void cam_oracle_fp8_quant_rows(const uint16_t *x, int act, int64_t A, int64_t H, uint8_t *q,
+                                          uint8_t *scale)
+{
+    float *xf = (float *)malloc((size_t)(A > 0 ? A : 1) * (size_t)H * 4);
+    for (int64_t i = 0; i < A * H; ++i) {
+        xf[i] = act_to_f32(x[i], act);
+    }
+    cam_oracle_fp8_quant_rows_f32(xf, A, H, q, scale);
+    free(xf);
+}
+
+/* out[m, n] = sum_kb 2^(sa[m,kb] + sw[g,kb,n/128] - 254) * sum_{k in kb} a[m,k] * w[g,k,n]   (double, then fp32)
+ * a [A,K] e4m3, sa [A,K/128] e8m0, w [G,K,N] e4m3 row-major, sw [G,K/128,N/128] e8m0, group_list cumulative. */
+ORACLE_API void cam_oracle_fp8_gemm(const uint8_t *a, const uint8_t *sa, const uint8_t *w, const uint8_t *sw,
+                                    const int64_t *group_list, int64_t G, int64_t K, int64_t N, float *out)
+{
+    float lut[256];
+    for (int i = 0; i < 256; ++i) {
+        lut[i] = cam_e4m3_to_f32((uint8_t)i);
+    }
+    const int64_t kb_n = K / CAM_FP8_BLOCK, nb_n = N / CAM_FP8_BLOCK;
+    for (int64_t g = 0; g < G; ++g) {
+        const int64_t m0 = g == 0 ? 0 : group_list[g - 1], m1 = group_list[g];
+        const uint8_t *wg = w + g * K * N;
+        const uint8_t *swg = sw + g * kb_n * nb_n;
+#pragma omp parallel for schedule(dynamic, 4)
+        for (int64_t m = m0; m < m1; ++m) {
+            double *acc = (double *)calloc((size_t)N, sizeof(double));
+            double *part = (double *)malloc((size_t)N * sizeof(double));
+            for (int64_t kb = 0; kb < kb_n; ++kb) {
+                memset(part, 0, (size_t)N * sizeof(double));
+                for (int64_t k = kb * CAM_FP8_BLOCK; k < (kb + 1) * CAM_FP8_BLOCK; ++k) {
+                    const double av = lut[a[m * K + k]];
+                    if (av == 0.0) {
+                        continue;
+                    }
+                    const uint8_t *wr = wg + k * N;
+                    for (int64_t n = 0; n < N; ++n) {
+                        part[n] += av * (double)lut[wr[n]];
+                    }
+                }
+                const int ea = (int)sa[m * kb_n + kb] - 127;
+                for (int64_t n = 0; n < N; ++n) {
+                    const int eb = (int)swg[kb * nb_n + n / CAM_FP8_BLOCK] - 127;
+                    acc[n] += ldexp(part[n], ea + eb);
+                }
+            }
+            for (int64_t n = 0; n < N; ++n) {
+                out[m * N + n] = (float)acc[n];
+            }
+            free(acc);
+            free(part);
+        }
+    }
+}
+
+/* y[m, i] = silu(c[m, i]) * c[m, I + i]: gate = columns [0, I), up = [I, 2I), as in the int8 layer
+ * (FDM/epilogue/block/block_epilogue_per_token_dequant_swiglu.h:178, :253-264). */
+ORACLE_API void cam_oracle_fp8_swiglu(const float *c, int64_t M, int64_t I, float *y)
+{
+#pragma omp parallel for schedule(static)
+    for (int64_t m = 0; m < M; ++m) {
+        for (int64_t i = 0; i < I; ++i) {
+            y[m * I + i] = cam_silu_spec(c[m * 2 * I + i]) * c[m * 2 * I + I + i];
+        }
+    }
+}
+
+ORACLE_API void cam_oracle_f32_rows_to_bf16(const float *x, int64_t n, uint16_t *out)
+{
+    for (int64_t i = 0; i < n; ++i) {
+        out[i] = f32_to_bf16(x[i]);
+    }
 }

@@ -287,3 +287,100 @@ def fused_layer(x_bits, idx, topk_w, w1, w1_scale, w2, w2_scale, n_active=None, 
     if debug:
         return out, etn, dbg
     return out, etn
+
+
+# ------------------------------------------------------------------ block-scaled FP8 layer (a definition of this
+# build: include/cam_fp8_spec.h; the reference is W8A8 only)
+def e4m3_to_f32(b):
+    b = _c(b, np.uint8)
+    f = lib().cam_oracle_e4m3_to_f32
+    f.restype = ctypes.c_float
+    f.argtypes = [ctypes.c_uint8]
+    return np.array([f(int(v)) for v in b.ravel()], np.float32).reshape(b.shape)
+
+
+def f32_to_e4m3(x):
+    x = _c(x, np.float32)
+    f = lib().cam_oracle_f32_to_e4m3
+    f.restype = ctypes.c_uint8
+    f.argtypes = [ctypes.c_float]
+    return np.array([f(float(v)) for v in x.ravel()], np.uint8).reshape(x.shape)
+
+
+def fp8_block_scale_exp(amax):
+    f = lib().cam_oracle_fp8_block_scale_exp
+    f.restype = ctypes.c_int
+    f.argtypes = [ctypes.c_float]
+    return int(f(float(amax)))
+
+
+def fp8_quant_rows_f32(x):
+    """fp32 rows [A,H] -> (e4m3 bytes [A,H], e8m0 scales [A,H/128])."""
+    x = _c(x, np.float32)
+    A, H = x.shape
+    assert H % 128 == 0
+    q = np.zeros((A, H), np.uint8)
+    sc = np.zeros((A, H // 128), np.uint8)
+    lib().cam_oracle_fp8_quant_rows_f32(_p(x), _i64(A), _i64(H), _p(q), _p(sc))
+    return q, sc
+
+
+def fp8_quant_rows(x_bits, fp16=False):
+    x_bits = _c(x_bits, np.uint16)
+    A, H = x_bits.shape
+    assert H % 128 == 0
+    q = np.zeros((A, H), np.uint8)
+    sc = np.zeros((A, H // 128), np.uint8)
+    lib().cam_oracle_fp8_quant_rows(_p(x_bits), ctypes.c_int(1 if fp16 else 0), _i64(A), _i64(H), _p(q), _p(sc))
+    return q, sc
+
+
+def fp8_gemm(a, sa, w, sw, group_list):
+    """a [A,K] e4m3, sa [A,K/128] e8m0, w [G,K,N] e4m3, sw [G,K/128,N/128] e8m0 -> fp32 [A,N]."""
+    a = _c(a, np.uint8)
+    sa = _c(sa, np.uint8)
+    w = _c(w, np.uint8)
+    sw = _c(sw, np.uint8)
+    gl = _c(group_list, np.int64)
+    G, K, N = w.shape
+    out = np.zeros((a.shape[0], N), np.float32)
+    lib().cam_oracle_fp8_gemm(_p(a), _p(sa), _p(w), _p(sw), _p(gl), _i64(G), _i64(K), _i64(N), _p(out))
+    return out
+
+
+def fp8_swiglu(c):
+    c = _c(c, np.float32)
+    M, N = c.shape
+    y = np.zeros((M, N // 2), np.float32)
+    lib().cam_oracle_fp8_swiglu(_p(c), _i64(M), _i64(N // 2), _p(y))
+    return y
+
+
+def fp8_fused_layer(x_bits, idx, topk_w, w1, sw1, w2, sw2, debug=False):
+    """The FP8 layer on one rank as the composition of the stage functions.
+    w1 [E,H,2I] e4m3, sw1 [E,H/128,2I/128]; w2 [E,I,H], sw2 [E,I/128,H/128].  Returns bf16 bits [T,H]."""
+    idx = _c(idx, np.int64)
+    T, K = idx.shape
+    E = w1.shape[0]
+    _, cnt, _ = layout(idx, E, 1)
+    off, _ = offsets(cnt, T)
+    pos = send_token_idx(idx, E)
+    row_of = rows_from_pos(idx, off, pos, E)
+    A = int(cnt.sum())
+    H = x_bits.shape[1]
+    rows = np.zeros((max(A, 1), H), np.uint16)
+    flat = row_of.reshape(-1)
+    src = np.repeat(np.arange(T), K)
+    ok = flat >= 0
+    rows[flat[ok]] = x_bits[src[ok]]
+    x1, s1 = fp8_quant_rows(rows[:A] if A else rows[:0])
+    gl = np.cumsum(cnt).astype(np.int64)
+    c1 = fp8_gemm(x1, s1, w1, sw1, gl)
+    y = fp8_swiglu(c1)
+    x2, s2 = fp8_quant_rows_f32(y)
+    c2 = fp8_gemm(x2, s2, w2, sw2, gl)
+    ybits = f32_to_bf16_bits(c2)
+    out = combine(ybits if A else np.zeros((1, H), np.uint16), row_of.reshape(T, K), topk_w)
+    if debug:
+        return out, dict(x1=x1, s1=s1, c1=c1, y=y, x2=x2, s2=s2, c2=c2, row_of=row_of, cnt=cnt)
+    return out

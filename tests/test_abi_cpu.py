@@ -291,3 +291,53 @@ def test_torch_ops_registered_with_reference_schemas():
         torch.empty(4, 1024, device="meta", dtype=torch.bfloat16), torch.empty(4, 2, device="meta", dtype=torch.int32),
         [], [], [], [], torch.empty(4, 2, device="meta"), None, None, "g", 1, 0, 8, 1, 0, 0, 0)
     assert out[0].shape == (4, 1024) and out[1].shape == (8,) and out[1].dtype == torch.int64
+
+
+def test_fp8_operator_validation():
+    f8, u8 = torch.float8_e4m3fn, torch.uint8
+
+    def packed8(shape):
+        w = _t(shape, f8)
+        w._cam_format = CAM_FORMAT_MFMA_B
+        return w
+
+    gl = _t((2,), torch.int64)
+    ok = [_t((10, 256), f8), _t((10, 2), u8), packed8((2, 256, 512)), _t((2, 2, 4), u8), 0, gl, 0,
+          _t((10, 512), torch.float32)]
+    assert _lib.phase1("GroupedMatmulFp8", ok)[0] == CAM_OK
+    a = list(ok)
+    a[7] = _t((10, 512), torch.bfloat16)
+    assert _lib.phase1("GroupedMatmulFp8", a)[0] == CAM_OK
+    a = list(ok)
+    a[4], a[7] = 1, _t((10, 256), torch.float32)      # SwiGLU product: N/2 columns
+    assert _lib.phase1("GroupedMatmulFp8", a)[0] == CAM_OK
+    a[7] = _t((10, 256), torch.bfloat16)
+    assert _lib.phase1("GroupedMatmulFp8", a)[0] == CAM_ERR_DTYPE
+    a = list(ok)
+    a[1] = _t((10, 3), u8)
+    assert _lib.phase1("GroupedMatmulFp8", a)[0] == CAM_ERR_SHAPE
+    a = list(ok)
+    a[2] = _t((2, 256, 512), f8)                       # not prepacked
+    assert _lib.phase1("GroupedMatmulFp8", a)[0] == CAM_ERR_UNSUPPORTED
+    a = list(ok)
+    a[0], a[1], a[2], a[3] = _t((10, 192), f8), _t((10, 1), u8), packed8((2, 192, 512)), _t((2, 1, 4), u8)
+    assert _lib.phase1("GroupedMatmulFp8", a)[0] == CAM_ERR_RANGE   # K not a multiple of 128
+    assert _lib.phase1("QuantRowsFp8", [_t((4, 256), torch.float32), _t((4, 256), f8), _t((4, 2), u8)])[0] == CAM_OK
+    assert _lib.phase1("QuantRowsFp8", [_t((4, 200), torch.float32), _t((4, 200), f8), _t((4, 1), u8)])[0] == \
+        CAM_ERR_ALIGN
+    T, K, E, H, I = 4, 2, 4, 1024, 512
+    fused = [_t((T, H), torch.bfloat16), _t((T, K), torch.int32), packed8((E, H, 2 * I)), _t((E, H // 128, 2 * I // 128), u8),
+             packed8((E, I, H)), _t((E, I // 128, H // 128), u8), _t((T, K), torch.float32), None, E,
+             _t((T, H), torch.bfloat16), _t((E,), torch.int64)]
+    st, ws, _ = _lib.phase1("FusedDeepMoeFp8", fused)
+    assert st == CAM_OK and ws > 0
+    a = list(fused)
+    a[3] = _t((E, H // 128, 2 * I // 128 + 1), u8)
+    assert _lib.phase1("FusedDeepMoeFp8", a)[0] == CAM_ERR_SHAPE
+    a = list(fused)
+    a[8] = 513
+    assert _lib.phase1("FusedDeepMoeFp8", a)[0] == CAM_ERR_RANGE
+    # quantMode 4 of MoeDispatchPrefill: FP8 rows with uint8 block scales
+    pre = _prefill_args()
+    pre[5] = 4
+    assert _lib.phase1("MoeDispatchPrefill", pre)[0] != CAM_OK          # int8 rows / fp32 scales do not fit

@@ -550,3 +550,115 @@ def test_fused_layer_active_mask_prefix(oracle):
     assert np.array_equal(part[:6], full[:6])  # tokens are independent
     assert (part[6:] == 0).all()
     assert etn.sum() == 6 * 2
+
+
+# ------------------------------------------------------------------ block-scaled FP8 (definition: include/cam_fp8_spec.h)
+def _e4m3_closed_form(code):
+    s = -1.0 if code & 0x80 else 1.0
+    e, m = (code >> 3) & 0xf, code & 7
+    if e == 0xf and m == 7:
+        return float("nan")
+    if e == 0:
+        return s * math.ldexp(m / 8.0, -6)
+    return s * math.ldexp(1.0 + m / 8.0, e - 7)
+
+
+def test_e4m3_decode_table_closed_form_and_torch(oracle):
+    codes = np.arange(256, dtype=np.uint8)
+    got = oracle.e4m3_to_f32(codes)
+    want = np.array([_e4m3_closed_form(int(c)) for c in codes], np.float32)
+    assert np.array_equal(got, want, equal_nan=True)
+    assert got[0x7e] == 448.0 and got[0x08] == 2.0 ** -6 and got[0x01] == 2.0 ** -9
+    via_torch = torch.from_numpy(codes).view(torch.float8_e4m3fn).float().numpy()
+    assert np.array_equal(got, via_torch, equal_nan=True)
+
+
+def test_e4m3_encode_is_nearest_even_and_saturates(oracle):
+    rng = np.random.default_rng(21)
+    table = oracle.e4m3_to_f32(np.arange(256, dtype=np.uint8)).astype(np.float64)
+    finite = np.array([c for c in range(256) if not math.isnan(table[c])])
+    x = np.concatenate([rng.uniform(-470, 470, 3000), rng.normal(0, 1, 3000), rng.uniform(-0.02, 0.02, 2000),
+                        table[finite], (table[finite[:-1]] + table[finite[1:]]) / 2,   # representable values and ties
+                        [448.0, 449.0, 463.9, 464.0, 1e9, -1e9, 2.0 ** -10, 2.0 ** -10 * 1.0001, 0.0]]).astype(np.float32)
+    got = oracle.f32_to_e4m3(x)
+    # brute force: the nearest finite value, ties to the even code, everything above 448 clamped
+    for xv, g in zip(x.tolist(), got.tolist()):
+        c = min(max(xv, -448.0), 448.0)
+        d = np.abs(table[finite] - c)
+        best = finite[np.nonzero(d == d.min())[0]]
+        if len(best) > 1:
+            best = [b for b in best if (b & 1) == 0] if c != 0 else [0x80 if math.copysign(1, xv) < 0 else 0]
+        assert table[g] == table[best[0]], (xv, g, best)
+    # and torch's conversion wherever it is defined the same way (no saturation there)
+    inr = np.abs(x) <= 448
+    via_torch = torch.from_numpy(x[inr]).to(torch.float8_e4m3fn).view(torch.uint8).numpy()
+    assert np.array_equal(got[inr], via_torch)
+    assert oracle.f32_to_e4m3(np.array([np.inf, -np.inf], np.float32)).tolist() == [0x7e, 0xfe]
+
+
+def test_fp8_block_scale_is_the_smallest_power_of_two(oracle):
+    from fractions import Fraction
+    rng = np.random.default_rng(22)
+    vals = np.concatenate([np.exp(rng.uniform(-60, 60, 2000)), [448.0, 448.0001, 447.99, 224.0, 1.0, 1.75, 1.7500001,
+                                                                 3.5, 2.0 ** -100, 7 * 2.0 ** 40]]).astype(np.float32)
+    for v in vals.tolist():
+        x = oracle.fp8_block_scale_exp(v)
+        fv = Fraction(v)
+        assert fv / Fraction(2) ** x <= 448, (v, x)
+        assert fv / Fraction(2) ** (x - 1) > 448, (v, x)
+    assert oracle.fp8_block_scale_exp(0.0) == 0
+
+
+def test_fp8_quant_rows_matches_torch_conversion_of_scaled_values(oracle):
+    x = torch.randn(19, 512, generator=torch.Generator().manual_seed(23)) * 5
+    x[0] = 0
+    x[1] *= 1e-12
+    x[2, :128] = 448.0
+    xb = x.bfloat16()
+    q, sc = oracle.fp8_quant_rows(synth.bf16_bits(xb))
+    xf = xb.float().reshape(19, 4, 128)
+    amax = xf.abs().amax(dim=2)
+    exps = torch.tensor([[oracle.fp8_block_scale_exp(float(v)) for v in row] for row in amax])
+    assert np.array_equal(sc, (exps + 127).to(torch.uint8).numpy())
+    scaled = xf * torch.pow(2.0, -exps.float())[:, :, None]
+    assert float(scaled.abs().max()) <= 448.0
+    want = scaled.to(torch.float8_e4m3fn).view(torch.uint8).reshape(19, 512).numpy()
+    assert np.array_equal(q, want)
+    # the largest scaled value of a live block lies in (224, 448]; rounding keeps it within [224, 448]
+    deq = oracle.e4m3_to_f32(q).reshape(19, 4, 128)
+    big = np.abs(deq).max(axis=2)
+    live = amax.numpy() > 0
+    assert ((big[live] >= 224) & (big[live] <= 448)).all()
+    pre = scaled.abs().amax(dim=2).numpy()
+    assert ((pre[live] > 224) & (pre[live] <= 448)).all()
+    q32, sc32 = oracle.fp8_quant_rows_f32(xb.float().numpy())
+    assert np.array_equal(q32, q) and np.array_equal(sc32, sc)
+
+
+def test_fp8_gemm_against_float64_and_swiglu(oracle):
+    g = torch.Generator().manual_seed(24)
+    sizes = [3, 0, 5]
+    G, K, N = 3, 256, 256
+    A = sum(sizes)
+    a = (torch.randn(A, K, generator=g) * 2).to(torch.float8_e4m3fn)
+    w = torch.randn(G, K, N, generator=g).to(torch.float8_e4m3fn)
+    sa = (torch.randint(-5, 4, (A, K // 128), generator=g) + 127).to(torch.uint8)
+    sw = (torch.randint(-5, 4, (G, K // 128, N // 128), generator=g) + 127).to(torch.uint8)
+    gl = np.cumsum(sizes).astype(np.int64)
+    got = oracle.fp8_gemm(a.view(torch.uint8).numpy(), sa.numpy(), w.view(torch.uint8).numpy(), sw.numpy(), gl)
+    af = a.double() * torch.pow(2.0, sa.double() - 127).repeat_interleave(128, dim=1)
+    want = np.zeros((A, N))
+    m0 = 0
+    for e, n in enumerate(sizes):
+        wf = w[e].double() * torch.pow(2.0, sw[e].double() - 127).repeat_interleave(128, dim=0).repeat_interleave(128, dim=1)
+        want[m0:m0 + n] = (af[m0:m0 + n] @ wf).numpy()
+        m0 += n
+    assert np.array_equal(got, want.astype(np.float32))
+    # scaling every operand block by a power of two scales the result exactly
+    got2 = oracle.fp8_gemm(a.view(torch.uint8).numpy(), (sa + 3).numpy(), w.view(torch.uint8).numpy(), (sw - 1).numpy(), gl)
+    assert np.array_equal(got2, got * 4.0)
+    c = torch.randn(7, 64, generator=g).numpy() * 3
+    y = oracle.fp8_swiglu(c.astype(np.float32))
+    c64 = c.astype(np.float32).astype(np.float64)
+    ref = c64[:, :32] / (1 + np.exp(-c64[:, :32])) * c64[:, 32:]
+    assert np.allclose(y, ref, rtol=3e-6, atol=1e-7)

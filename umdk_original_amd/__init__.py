@@ -5,7 +5,8 @@ include/cam_mi355x.h); this package is the thin Python host side that mirrors th
 `umdk_cam_op_lib` operators.
 """
 from . import _lib
-from .ops import (CamError, fused_deep_moe, get_dispatch_layout, grouped_matmul_dequant, grouped_matmul_int32,
+from .ops import (CamError, fused_deep_moe, fused_deep_moe_fp8, get_dispatch_layout, grouped_matmul_dequant,
+                  grouped_matmul_fp8, grouped_matmul_int32, quant_rows_fp8,
                   grouped_matmul_swiglu_quant, moe_combine_gather, moe_combine_index, moe_combine_normal,
                   moe_combine_prefill, moe_dispatch_fused, moe_dispatch_normal,
                   moe_dispatch_plan, moe_dispatch_prefill, notify_dispatch, prepack_weight, register_torch_ops)

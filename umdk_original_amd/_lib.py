@@ -36,6 +36,7 @@ CAM_DT_UINT8 = 4
 CAM_DT_INT64 = 9
 CAM_DT_BOOL = 12
 CAM_DT_BF16 = 27
+CAM_DT_FLOAT8_E4M3FN = 36
 
 CAM_FORMAT_ND = 2
 CAM_FORMAT_MFMA_B = 100
@@ -49,6 +50,7 @@ _DTYPES = {
     torch.int64: CAM_DT_INT64,
     torch.bool: CAM_DT_BOOL,
     torch.bfloat16: CAM_DT_BF16,
+    torch.float8_e4m3fn: CAM_DT_FLOAT8_E4M3FN,
 }
 
 
@@ -103,6 +105,9 @@ SIGNATURES = {
     "GroupedMatmulInt32": [_TP, _LP, _I64, _TP, _I64, _TP],
     "FusedDeepMoe": [_TP, _TP, _LP, _LP, _LP, _LP, _TP, _TP, _TP, _STR, _I64, _I64, _I64, _I64, _I64, _I64, _I64,
                      _TP, _TP],
+    "GroupedMatmulFp8": [_TP, _TP, _TP, _TP, _I64, _TP, _I64, _TP],
+    "QuantRowsFp8": [_TP, _TP, _TP],
+    "FusedDeepMoeFp8": [_TP, _TP, _TP, _TP, _TP, _TP, _TP, _TP, _I64, _TP, _TP],
 }
 
 # Single-call entry points (no executor, no workspace): name -> argument types before the stream.

@@ -50,7 +50,10 @@ enum OpTag {
     kOpGmm1 = 0x474d4d31,
     kOpGmm2 = 0x474d4d32,
     kOpGmmI32 = 0x474d4d49,
-    kOpFused = 0x46555345
+    kOpFused = 0x46555345,
+    kOpGmmFp8 = 0x474d4638,
+    kOpQuantFp8 = 0x51544638,
+    kOpFusedFp8 = 0x46554638
 };
 
 constexpr uint64_t kAlign = 256;
@@ -752,8 +755,9 @@ camStatus camMoeDispatchPrefillGetWorkspaceSize(const camTensor *x, const camTen
     if (numRanks != 1) {
         return fail(CAM_ERR_UNSUPPORTED, "MoeDispatchPrefill: numRanks must be 1 (single-GPU library)");
     }
-    if (quantMode < 0 || quantMode > 3) {
-        return fail(CAM_ERR_RANGE, "quantMode %lld outside [0, 3]", (long long)quantMode);
+    // quantMode 4 is this library's block-scaled FP8 (include/cam_fp8_spec.h); 0..3 are the reference's values
+    if (quantMode < 0 || quantMode > 4) {
+        return fail(CAM_ERR_RANGE, "quantMode %lld outside [0, 4]", (long long)quantMode);
     }
     if (quantMode == 1) {
         return fail(CAM_ERR_UNSUPPORTED, "quantMode 1 (static quantisation) is not built");
@@ -778,14 +782,27 @@ camStatus camMoeDispatchPrefillGetWorkspaceSize(const camTensor *x, const camTen
         return fail(CAM_ERR_RANGE, "tokens * top-k does not fit 32 bits");
     }
     const bool quant = quantMode != 0;
-    CAM_TRY(check_tensor(recvX, "recvX", 2, quant ? CAM_DT_INT8 : x->dtype));
+    const bool fp8 = quantMode == 4;
+    if (fp8 && H % 128 != 0) {
+        return fail(CAM_ERR_ALIGN, "FP8 block scales need a hidden size that is a multiple of 128");
+    }
+    if (fp8) {
+        CAM_TRY(check_tensor(recvX, "recvX", 2, CAM_DT_FLOAT8_E4M3FN, CAM_DT_UINT8));
+    } else {
+        CAM_TRY(check_tensor(recvX, "recvX", 2, quant ? CAM_DT_INT8 : x->dtype));
+    }
     if (recvX->sizes[1] != H) {
         return fail(CAM_ERR_SHAPE, "recvX dimension 1 must equal the hidden size");
     }
     const int64_t A = recvX->sizes[0];
     CAM_TRY(check_aligned(x, "x", 16));
     CAM_TRY(check_aligned(recvX, "recvX", 16));
-    if (quant) {
+    if (fp8) {
+        CAM_TRY(check_tensor(recvXScalesOptional, "recvXScales", 2, CAM_DT_UINT8));
+        if (recvXScalesOptional->sizes[0] < A || recvXScalesOptional->sizes[1] != H / 128) {
+            return fail(CAM_ERR_SHAPE, "recvXScales must be uint8 [rows, H/128] (E8M0)");
+        }
+    } else if (quant) {
         CAM_TRY(check_tensor(recvXScalesOptional, "recvXScales", 1, CAM_DT_FLOAT));
         if (recvXScalesOptional->sizes[0] < A) {
             return fail(CAM_ERR_SHAPE, "recvXScales must hold one value per recvX row");
@@ -846,7 +863,7 @@ camStatus camMoeDispatchPrefillGetWorkspaceSize(const camTensor *x, const camTen
     f.x_is_fp16 = x->dtype == CAM_DT_FLOAT16;
     f.H = (int)H;
     f.A = A;
-    f.quant = quantMode == 0 ? 0 : (quantMode == 2 ? 1 : 2);
+    f.quant = quantMode == 0 ? 0 : (quantMode == 2 ? 1 : (quantMode == 4 ? 3 : 2));
     f.out = recvX->data;
     f.scales = quant ? (float *)recvXScalesOptional->data : nullptr;
     f.src_info = (int32_t *)expandIdx->data;
@@ -1103,8 +1120,12 @@ camStatus camPrepackWeightGetWorkspaceSize(const camTensor *src, int64_t gateUp,
     if (src->ndim != 2 && src->ndim != 3) {
         return fail(CAM_ERR_SHAPE, "src must be [Kd,N] or [G,Kd,N]");
     }
-    CAM_TRY(check_tensor(src, "src", src->ndim, CAM_DT_INT8));
-    CAM_TRY(check_tensor(dst, "dst", src->ndim, CAM_DT_INT8));
+    // the layout moves bytes: int8 weights, or FP8 E4M3 weights of the block-scaled operators
+    CAM_TRY(check_tensor(src, "src", src->ndim, CAM_DT_INT8, CAM_DT_FLOAT8_E4M3FN, CAM_DT_UINT8));
+    CAM_TRY(check_tensor(dst, "dst", src->ndim, CAM_DT_INT8, CAM_DT_FLOAT8_E4M3FN, CAM_DT_UINT8));
+    if (src->dtype != dst->dtype) {
+        return fail(CAM_ERR_DTYPE, "src and dst must have the same dtype");
+    }
     for (int d = 0; d < src->ndim; ++d) {
         if (src->sizes[d] != dst->sizes[d]) {
             return fail(CAM_ERR_SHAPE, "src and dst must have the same extents");
@@ -1613,6 +1634,352 @@ camStatus camFusedDeepMoeGetWorkspaceSize(const camTensor *x, const camTensor *e
 camStatus camFusedDeepMoe(void *workspace, uint64_t workspaceSize, camOpExecutor *executor, camStream_t stream)
 {
     return run_phase2(kOpFused, "camFusedDeepMoe", workspace, workspaceSize, executor, stream);
+}
+
+// ------------------------------------------------------------------------------------------------
+// Block-scaled FP8 operators (include/cam_fp8_spec.h).  No counterpart in the reference, whose fused operator
+// is W8A8 only (src/cam/README.md:20-21).
+namespace {
+
+struct Fp8Weight {
+    const int8_t *w;
+    const uint8_t *s;
+};
+
+camStatus check_fp8_weight(const camTensor *w, const camTensor *ws, const char *name, int64_t G, int64_t Kd,
+                           int64_t N, Fp8Weight *out)
+{
+    CAM_TRY(check_tensor(w, name, 3, CAM_DT_FLOAT8_E4M3FN, CAM_DT_UINT8));
+    if (w->format != CAM_FORMAT_MFMA_B) {
+        return fail(CAM_ERR_UNSUPPORTED, "%s must be converted once with camPrepackWeight (format CAM_FORMAT_MFMA_B)",
+                    name);
+    }
+    if (w->sizes[0] != G || w->sizes[1] != Kd || w->sizes[2] != N) {
+        return fail(CAM_ERR_SHAPE, "%s must be [%lld,%lld,%lld]", name, (long long)G, (long long)Kd, (long long)N);
+    }
+    CAM_TRY(check_tensor(ws, "weight scale", 3, CAM_DT_UINT8));
+    if (ws->sizes[0] != G || ws->sizes[1] != Kd / 128 || ws->sizes[2] != N / 128) {
+        return fail(CAM_ERR_SHAPE, "%s scale must be uint8 [%lld,%lld,%lld] (E8M0 per 128 x 128 block)", name,
+                    (long long)G, (long long)(Kd / 128), (long long)(N / 128));
+    }
+    CAM_TRY(check_aligned(w, name, 16));
+    out->w = (const int8_t *)w->data;
+    out->s = (const uint8_t *)ws->data;
+    return CAM_OK;
+}
+
+camStatus check_fp8_dims(const char *op, int64_t Kd, int64_t N, bool gate_up)
+{
+    if (Kd < 128 || Kd % 128 != 0 || Kd > 8192) {
+        return fail(CAM_ERR_RANGE, "%s: K %lld must be a multiple of 128 in [128, 8192]", op, (long long)Kd);
+    }
+    if (N < 128 || N % (gate_up ? 256 : 128) != 0) {
+        return fail(CAM_ERR_RANGE, "%s: N %lld must be a multiple of %d", op, (long long)N, gate_up ? 256 : 128);
+    }
+    return CAM_OK;
+}
+
+}  // namespace
+
+camStatus camGroupedMatmulFp8GetWorkspaceSize(const camTensor *x, const camTensor *xScale, const camTensor *weight,
+                                              const camTensor *weightScale, int64_t gateUp,
+                                              const camTensor *groupList, int64_t groupListType,
+                                              const camTensor *out, uint64_t *workspaceSize,
+                                              camOpExecutor **executor)
+{
+    CAM_TRY(check_tensor(x, "x", 2, CAM_DT_FLOAT8_E4M3FN, CAM_DT_UINT8));
+    CAM_TRY(check_aligned(x, "x", 16));
+    CAM_TRY(check_tensor(groupList, "groupList", 1, CAM_DT_INT64));
+    if (groupListType != 0 && groupListType != 1) {
+        return fail(CAM_ERR_RANGE, "GroupedMatmulFp8: groupListType must be 0 (cumulative) or 1 (counts)");
+    }
+    const int64_t A = x->sizes[0], Kd = x->sizes[1], G = groupList->sizes[0];
+    if (G <= 0 || G > cam::kMaxExperts) {
+        return fail(CAM_ERR_RANGE, "GroupedMatmulFp8: %lld experts outside (0, %d]", (long long)G, cam::kMaxExperts);
+    }
+    if (A > 0x3fffffffll) {
+        return fail(CAM_ERR_RANGE, "GroupedMatmulFp8: too many rows");
+    }
+    CAM_TRY(check_tensor(xScale, "xScale", 2, CAM_DT_UINT8));
+    if (xScale->sizes[0] < A || xScale->sizes[1] != Kd / 128) {
+        return fail(CAM_ERR_SHAPE, "xScale must be uint8 [rows, K/128] (E8M0)");
+    }
+    CAM_TRY(check_tensor(out, "out", 2, CAM_DT_FLOAT, CAM_DT_BF16));
+    if (out->sizes[0] != A) {
+        return fail(CAM_ERR_SHAPE, "out must have one row per row of x");
+    }
+    const bool gate_up = gateUp != 0;
+    if (gate_up && out->dtype != CAM_DT_FLOAT) {
+        return fail(CAM_ERR_DTYPE, "the SwiGLU product (gateUp != 0) is written as float32");
+    }
+    const int64_t N = gate_up ? 2 * out->sizes[1] : out->sizes[1];
+    CAM_TRY(check_fp8_dims("GroupedMatmulFp8", Kd, N, gate_up));
+    CAM_TRY(check_aligned(out, "out", 16));
+    Fp8Weight fw{};
+    CAM_TRY(check_fp8_weight(weight, weightScale, "weight", G, Kd, N, &fw));
+    cam::SchedSpec sp = sched_spec(A, G, N);
+    Carver c;
+    const uint64_t o_sched = c.take(cam::sched_bytes(A, (int)G, (int)N));
+    cam::GemmArgs g{};
+    g.a = (const int8_t *)x->data;
+    g.w = fw.w;
+    g.fp8 = 1;
+    g.a_scale8 = (const uint8_t *)xScale->data;
+    g.w_scale8 = fw.s;
+    g.Kd = (int)Kd;
+    g.N = (int)N;
+    g.gate_up = gate_up;
+    g.epilogue = gate_up ? cam::kEpiSwiglu : (out->dtype == CAM_DT_BF16 ? cam::kEpiDequantBf16 : cam::kEpiInt32);
+    g.out = out->data;
+    const int64_t *gl = (const int64_t *)groupList->data;
+    const int cumulative = groupListType == 0;
+    auto run = [=](void *wsp, hipStream_t s) mutable -> hipError_t {
+        sp.sched = (int32_t *)((char *)wsp + o_sched);
+        hipError_t e = cam::launch_build_sched(gl, cumulative, (int)G, A, 1, &sp, s);
+        if (e != hipSuccess) {
+            return e;
+        }
+        g.sched = sp.sched;
+        return cam::launch_gemm(g, s);
+    };
+    return finish_phase1(kOpGmmFp8, c.off, run, workspaceSize, executor);
+}
+
+camStatus camGroupedMatmulFp8(void *workspace, uint64_t workspaceSize, camOpExecutor *executor, camStream_t stream)
+{
+    return run_phase2(kOpGmmFp8, "camGroupedMatmulFp8", workspace, workspaceSize, executor, stream);
+}
+
+camStatus camQuantRowsFp8GetWorkspaceSize(const camTensor *x, const camTensor *q, const camTensor *scale,
+                                          uint64_t *workspaceSize, camOpExecutor **executor)
+{
+    CAM_TRY(check_tensor(x, "x", 2, CAM_DT_FLOAT));
+    CAM_TRY(check_tensor(q, "q", 2, CAM_DT_FLOAT8_E4M3FN, CAM_DT_UINT8));
+    CAM_TRY(check_tensor(scale, "scale", 2, CAM_DT_UINT8));
+    const int64_t A = x->sizes[0], I = x->sizes[1];
+    if (I < 128 || I % 128 != 0) {
+        return fail(CAM_ERR_ALIGN, "the row length %lld must be a multiple of 128", (long long)I);
+    }
+    if (q->sizes[0] != A || q->sizes[1] != I || scale->sizes[0] != A || scale->sizes[1] != I / 128) {
+        return fail(CAM_ERR_SHAPE, "q must be [rows, I] and scale uint8 [rows, I/128]");
+    }
+    if (A > 0x7fffffffll) {
+        return fail(CAM_ERR_RANGE, "too many rows");
+    }
+    CAM_TRY(check_aligned(x, "x", 16));
+    CAM_TRY(check_aligned(q, "q", 16));
+    const float *xp = (const float *)x->data;
+    uint8_t *qp = (uint8_t *)q->data;
+    uint8_t *sp = (uint8_t *)scale->data;
+    const int iI = (int)I;
+    auto run = [=](void *, hipStream_t s) -> hipError_t {
+        return cam::launch_requant_fp8(xp, A, iI, nullptr, qp, sp, s);
+    };
+    return finish_phase1(kOpQuantFp8, 0, run, workspaceSize, executor);
+}
+
+camStatus camQuantRowsFp8(void *workspace, uint64_t workspaceSize, camOpExecutor *executor, camStream_t stream)
+{
+    return run_phase2(kOpQuantFp8, "camQuantRowsFp8", workspace, workspaceSize, executor, stream);
+}
+
+camStatus camFusedDeepMoeFp8GetWorkspaceSize(const camTensor *x, const camTensor *expertIds,
+                                             const camTensor *gmm1Weight, const camTensor *gmm1WeightScale,
+                                             const camTensor *gmm2Weight, const camTensor *gmm2WeightScale,
+                                             const camTensor *expertScales, const camTensor *xActiveMaskOptional,
+                                             int64_t moeExpertNum, const camTensor *output,
+                                             const camTensor *expertTokenNums, uint64_t *workspaceSize,
+                                             camOpExecutor **executor)
+{
+    CAM_TRY(check_tensor(x, "x", 2, CAM_DT_BF16, CAM_DT_FLOAT16));
+    CAM_TRY(check_tensor(expertIds, "expertIds", 2, CAM_DT_INT32));
+    CAM_TRY(check_tensor(expertScales, "expertScales", 2, CAM_DT_FLOAT));
+    if (moeExpertNum <= 0 || moeExpertNum > cam::kMaxExperts) {
+        return fail(CAM_ERR_RANGE, "moeExpertNum %lld outside (0, %d]", (long long)moeExpertNum, cam::kMaxExperts);
+    }
+    const int64_t T = x->sizes[0], H = x->sizes[1], K = expertIds->sizes[1], E = moeExpertNum;
+    if (T < 1 || expertIds->sizes[0] != T || expertScales->sizes[0] != T || expertScales->sizes[1] != K) {
+        return fail(CAM_ERR_SHAPE, "x, expertIds and expertScales must agree on [bs] and [bs,K]");
+    }
+    if (H < 1024 || H > 7168) {
+        return fail(CAM_ERR_RANGE, "hidden size %lld outside [1024, 7168]", (long long)H);
+    }
+    if (K <= 0 || K > cam::kMaxTopk) {
+        return fail(CAM_ERR_RANGE, "top-k %lld outside (0, %d]", (long long)K, cam::kMaxTopk);
+    }
+    if (T * K > 0x3fffffffll) {
+        return fail(CAM_ERR_RANGE, "tokens * top-k too large");
+    }
+    CAM_TRY(check_tensor(gmm2Weight, "gmm2Weight", 3, CAM_DT_FLOAT8_E4M3FN, CAM_DT_UINT8));
+    const int64_t I = gmm2Weight->sizes[1];
+    CAM_TRY(check_fp8_dims("FusedDeepMoeFp8 GMM1", H, 2 * I, true));
+    CAM_TRY(check_fp8_dims("FusedDeepMoeFp8 GMM2", I, H, false));
+    Fp8Weight w1{}, w2{};
+    CAM_TRY(check_fp8_weight(gmm1Weight, gmm1WeightScale, "gmm1Weight", E, H, 2 * I, &w1));
+    CAM_TRY(check_fp8_weight(gmm2Weight, gmm2WeightScale, "gmm2Weight", E, I, H, &w2));
+    if (xActiveMaskOptional != nullptr) {
+        CAM_TRY(check_tensor(xActiveMaskOptional, "xActiveMask", 1, CAM_DT_BOOL, CAM_DT_UINT8));
+        if (xActiveMaskOptional->sizes[0] != T) {
+            return fail(CAM_ERR_SHAPE, "xActiveMask must be [bs]");
+        }
+    }
+    CAM_TRY(check_tensor(output, "output", 2, CAM_DT_BF16));
+    if (output->sizes[0] != T || output->sizes[1] != H) {
+        return fail(CAM_ERR_SHAPE, "output must be [bs, H]");
+    }
+    CAM_TRY(check_tensor(expertTokenNums, "expertTokenNums", 1, CAM_DT_INT64));
+    if (expertTokenNums->sizes[0] != E) {
+        return fail(CAM_ERR_SHAPE, "expertTokenNums must hold one value per expert");
+    }
+    CAM_TRY(check_aligned(x, "x", 16));
+    CAM_TRY(check_aligned(output, "output", 16));
+
+    const int64_t A = T * K;
+    cam::SchedSpec sp1 = sched_spec(A, E, 2 * I);
+    cam::SchedSpec sp2 = sched_spec(A, E, H);
+    Carver c;
+    const uint64_t o_pos = c.take((uint64_t)A * 4);
+    const uint64_t o_row = c.take((uint64_t)A * 4);
+    const uint64_t o_meta = c.take(cam::kPlanMeta * 4);
+    const uint64_t o_sched1 = c.take(cam::sched_bytes(A, (int)E, (int)(2 * I)));
+    const uint64_t o_sched2 = c.take(cam::sched_bytes(A, (int)E, (int)H));
+    const bool fused_dispatch = cam::fused_dispatch_fits(T, K);
+    const uint64_t o_hist = c.take(fused_dispatch ? cam::fused_dispatch_table_bytes(T, K, (int)E)
+                                                  : cam::plan_workspace_bytes(T, K, (int)E));
+    const uint64_t o_ctrl = c.take(cam::fused_dispatch_ctrl_bytes());
+    // as in the int8 layer, the bf16 rows of GMM2 overlay the quantised input rows and the fp32 products
+    const uint64_t x1_bytes = align_up((uint64_t)A * H);
+    const uint64_t shared_bytes = std::max<uint64_t>((uint64_t)A * H * 2, x1_bytes + (uint64_t)A * I * 4);
+    const uint64_t o_x1 = c.take(shared_bytes);
+    const uint64_t o_prod = o_x1 + x1_bytes;
+    const uint64_t o_y = o_x1;
+    const uint64_t o_x1s = c.take((uint64_t)A * (H / 128));
+    const uint64_t o_x2 = c.take((uint64_t)A * I);
+    const uint64_t o_x2s = c.take((uint64_t)A * (I / 128));
+
+    const uint16_t *xp = (const uint16_t *)x->data;
+    const int x_is_fp16 = x->dtype == CAM_DT_FLOAT16;
+    const int32_t *ids = (const int32_t *)expertIds->data;
+    const float *gates = (const float *)expertScales->data;
+    const uint8_t *mask = xActiveMaskOptional ? (const uint8_t *)xActiveMaskOptional->data : nullptr;
+    uint16_t *outp = (uint16_t *)output->data;
+    int64_t *etn = (int64_t *)expertTokenNums->data;
+    const int iT = (int)T, iK = (int)K, iE = (int)E, iH = (int)H, iI = (int)I;
+
+    auto run = [=](void *wsp, hipStream_t s) -> hipError_t {
+        char *w = (char *)wsp;
+        int32_t *pos = (int32_t *)(w + o_pos);
+        int32_t *row = (int32_t *)(w + o_row);
+        int32_t *meta = (int32_t *)(w + o_meta);
+        uint8_t *x1 = (uint8_t *)(w + o_x1);
+        uint8_t *x1s = (uint8_t *)(w + o_x1s);
+        float *prod = (float *)(w + o_prod);
+        uint8_t *x2 = (uint8_t *)(w + o_x2);
+        uint8_t *x2s = (uint8_t *)(w + o_x2s);
+        uint16_t *y = (uint16_t *)(w + o_y);
+
+        cam::PlanArgs p{};
+        p.idx = ids;
+        p.idx_is64 = 0;
+        p.mask = mask;
+        p.T = iT;
+        p.K = iK;
+        p.E = iE;
+        p.R = 1;
+        p.pos = pos;
+        p.dst_row = row;
+        p.tokens_per_expert = etn;
+        p.meta = meta;
+        p.hist_ws = (int32_t *)(w + o_hist);
+        hipError_t e;
+        if (fused_dispatch) {
+            cam::FusedDispatchArgs f{};
+            f.p = p;
+            f.x = xp;
+            f.x_is_fp16 = x_is_fp16;
+            f.H = iH;
+            f.A = A;
+            f.quant = 3;
+            f.out = x1;
+            f.scales = (float *)x1s;
+            f.ctrl = (unsigned long long *)(w + o_ctrl);
+            e = cam::launch_dispatch_fused(f, s);
+            if (e != hipSuccess) return e;
+        } else {
+            e = cam::launch_plan(p, s);
+            if (e != hipSuccess) return e;
+            cam::DispatchArgs d{};
+            d.x = xp;
+            d.x_is_fp16 = x_is_fp16;
+            d.idx = ids;
+            d.dst_row = row;
+            d.T = iT;
+            d.K = iK;
+            d.H = iH;
+            d.E = iE;
+            d.A = A;
+            d.quant = 3;
+            d.out = x1;
+            d.scales = (float *)x1s;
+            e = cam::launch_dispatch(d, s);
+            if (e != hipSuccess) return e;
+        }
+        cam::SchedSpec specs[2] = {sp1, sp2};
+        specs[0].sched = (int32_t *)(w + o_sched1);
+        specs[1].sched = (int32_t *)(w + o_sched2);
+        e = cam::launch_build_sched(etn, 0, iE, A, 2, specs, s);
+        if (e != hipSuccess) return e;
+
+        cam::GemmArgs g1{};
+        g1.a = (const int8_t *)x1;
+        g1.w = w1.w;
+        g1.fp8 = 1;
+        g1.a_scale8 = x1s;
+        g1.w_scale8 = w1.s;
+        g1.sched = specs[0].sched;
+        g1.Kd = iH;
+        g1.N = 2 * iI;
+        g1.gate_up = 1;
+        g1.epilogue = cam::kEpiSwiglu;
+        g1.out = prod;
+        e = cam::launch_gemm(g1, s);
+        if (e != hipSuccess) return e;
+        e = cam::launch_requant_fp8(prod, A, iI, specs[0].sched, x2, x2s, s);
+        if (e != hipSuccess) return e;
+
+        cam::GemmArgs g2{};
+        g2.a = (const int8_t *)x2;
+        g2.w = w2.w;
+        g2.fp8 = 1;
+        g2.a_scale8 = x2s;
+        g2.w_scale8 = w2.s;
+        g2.sched = specs[1].sched;
+        g2.Kd = iI;
+        g2.N = iH;
+        g2.gate_up = 0;
+        g2.epilogue = cam::kEpiDequantBf16;
+        g2.out = y;
+        e = cam::launch_gemm(g2, s);
+        if (e != hipSuccess) return e;
+
+        cam::CombineArgs cb{};
+        cb.y = y;
+        cb.slot_row = row;
+        cb.w = gates;
+        cb.T = iT;
+        cb.K = iK;
+        cb.H = iH;
+        cb.A = A;
+        cb.t_active = meta + 2;
+        cb.out = outp;
+        return cam::launch_combine(cb, s);
+    };
+    return finish_phase1(kOpFusedFp8, c.off, run, workspaceSize, executor);
+}
+
+camStatus camFusedDeepMoeFp8(void *workspace, uint64_t workspaceSize, camOpExecutor *executor, camStream_t stream)
+{
+    return run_phase2(kOpFusedFp8, "camFusedDeepMoeFp8", workspace, workspaceSize, executor, stream);
 }
 
 }  // extern "C"

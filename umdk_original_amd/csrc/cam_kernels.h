@@ -92,7 +92,8 @@ struct DispatchArgs {
     const int32_t *dst_row;  // if non-null, used instead of the four arrays above
     int T, K, H, E;
     int64_t A;           // rows in the outputs
-    int quant;           // 0 copy, 1 = epsilon variant, 2 = no-epsilon variant
+    int quant;           // 0 copy, 1 = epsilon variant, 2 = no-epsilon variant (int8, one fp32 scale per row),
+                         // 3 = FP8 E4M3 with one E8M0 scale per row and 128 columns (scales: uint8 [A, H/128])
     int x_is_fp16;       // activations are IEEE fp16 instead of bf16 (matters only when quantising)
     void *out;           // [A,H] bf16 bits or int8
     float *scales;       // [A]   (quant only)
@@ -163,6 +164,13 @@ struct GemmArgs {
     int per_expert;        // weights given per expert through `list`
     WeightPtrs list;
     int32_t *sched;        // schedule built for this launch (its queue counters are consumed by the launch)
+    // Block-scaled FP8 (fp8 != 0; include/cam_fp8_spec.h): a and w hold E4M3 bytes, the fp32 scales above are
+    // unused, and every 128 bytes of K carry a power-of-two scale (E8M0 byte) per activation row and per 128
+    // weight columns.  Stacked weights only.  Epilogues: kEpiInt32 stores the fp32 sums, kEpiSwiglu stores
+    // silu(gate) * up as fp32, kEpiDequantBf16 stores bf16(sum).
+    int fp8;
+    const uint8_t *a_scale8;  // [A, Kd/128]
+    const uint8_t *w_scale8;  // [G, Kd/128, N/128]
     int Kd, N;             // N = logical columns of the weight
     int gate_up;           // weight prepacked with gate/up pairing
     int epilogue;
@@ -176,6 +184,11 @@ hipError_t launch_requant(const float *y, int64_t max_rows, int I, const int32_t
                           float *scale, hipStream_t stream);
 
 hipError_t launch_prepack(const int8_t *src, int8_t *dst, int G, int Kd, int N, int gate_up, hipStream_t stream);
+
+// fp32 rows [rows, I] -> E4M3 bytes + one E8M0 scale per row and 128 columns (I % 128 == 0).  sched_for_rows as
+// for launch_requant.
+hipError_t launch_requant_fp8(const float *y, int64_t max_rows, int I, const int32_t *sched_for_rows, uint8_t *q,
+                              uint8_t *scale, hipStream_t stream);
 
 }  // namespace cam
 

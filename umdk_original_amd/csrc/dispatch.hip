@@ -67,7 +67,7 @@ hipError_t launch_dispatch(const DispatchArgs &a, hipStream_t stream)
     if (a.T <= 0) {
         return hipSuccess;
     }
-    if (a.H % 8 != 0 || a.H / 8 > kDispMaxChunks * kWave) {
+    if (a.H % 8 != 0 || a.H / 8 > kDispMaxChunks * kWave || (a.quant == 3 && a.H % 128 != 0)) {
         return hipErrorInvalidValue;
     }
     dim3 grid((a.T + kDispWaves - 1) / kDispWaves), block(kDispWaves * kWave);
@@ -78,6 +78,12 @@ hipError_t launch_dispatch(const DispatchArgs &a, hipStream_t stream)
             hipLaunchKernelGGL((dispatch_kernel<1, 1>), grid, block, 0, stream, a);
         } else {
             hipLaunchKernelGGL((dispatch_kernel<1, 0>), grid, block, 0, stream, a);
+        }
+    } else if (a.quant == 3) {
+        if (a.x_is_fp16) {
+            hipLaunchKernelGGL((dispatch_kernel<3, 1>), grid, block, 0, stream, a);
+        } else {
+            hipLaunchKernelGGL((dispatch_kernel<3, 0>), grid, block, 0, stream, a);
         }
     } else {
         if (a.x_is_fp16) {

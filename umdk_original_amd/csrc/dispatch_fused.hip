@@ -272,6 +272,12 @@ hipError_t launch_t(const FusedDispatchArgs &a, dim3 grid, hipStream_t stream)
         } else {
             hipLaunchKernelGGL((dispatch_fused_kernel<IdT, 1, 0>), grid, blk, 0, stream, a);
         }
+    } else if (a.quant == 3) {
+        if (a.x_is_fp16) {
+            hipLaunchKernelGGL((dispatch_fused_kernel<IdT, 3, 1>), grid, blk, 0, stream, a);
+        } else {
+            hipLaunchKernelGGL((dispatch_fused_kernel<IdT, 3, 0>), grid, blk, 0, stream, a);
+        }
     } else {
         if (a.x_is_fp16) {
             hipLaunchKernelGGL((dispatch_fused_kernel<IdT, 2, 1>), grid, blk, 0, stream, a);
@@ -302,7 +308,7 @@ hipError_t launch_dispatch_fused(FusedDispatchArgs a, hipStream_t stream)
     if (!fused_dispatch_fits(a.p.T, a.p.K) || a.p.hist_ws == nullptr || a.ctrl == nullptr || a.p.pos == nullptr) {
         return hipErrorInvalidValue;
     }
-    if (a.H % 8 != 0 || a.H / 8 > kDispMaxChunks * kWave) {
+    if (a.H % 8 != 0 || a.H / 8 > kDispMaxChunks * kWave || (a.quant == 3 && a.H % 128 != 0)) {
         return hipErrorInvalidValue;
     }
     const long long n_all = (long long)a.p.T * a.p.K;

@@ -48,6 +48,7 @@
 #include "cam_device.h"
 #include "cam_kernels.h"
 #include "rank_device.h"
+#include "permute_device.h"
 #include "../../include/cam_expf_spec.h"
 
 namespace cam {
@@ -61,6 +62,7 @@ constexpr int kMaxStages = 4;
 constexpr int kStageTall = 256 * kBK + 256 * kBK;   // 16 KB of activations + 16 KB of weights
 constexpr int kStageFlat = 128 * kBK + 512 * kBK;   //  8 KB of activations + 32 KB of weights
 constexpr int kLdsBytes = kMaxStages * kStageTall;  // 128 KB (flat: 3 x 40 KB = 120 KB)
+constexpr int kScaleKb = 64;                    // FP8: K-blocks of 128 bytes an item may span (Kd <= 8192)
 constexpr int kEpiRowBytes = 144;               // epilogue staging: 128 data bytes + 16 of padding per row
 constexpr int kEpiSlice = 32 * kEpiRowBytes;    // one 32-row fragment per wave
 
@@ -115,9 +117,27 @@ struct ItemCtx {
 
 // One wave's part of one item.  TEAM 0 multiplies in the first phase of every sub-step, TEAM 1 in the second.
 // FLAT selects the tile shape (it fixes the loads per wave and sub-step); MF is the wave's fragment count.
-template <int MF, int TEAM, bool FLAT>
+__device__ __forceinline__ int acc_bits(int v) { return v; }
+__device__ __forceinline__ int acc_bits(float v) { return __float_as_int(v); }
+
+template <bool FP8>
+struct AccType {
+    typedef v16i type;
+};
+template <>
+struct AccType<true> {
+    typedef v16f type;
+};
+
+// FP8 items (FP8 = true) run the same pipeline with v_mfma_scale_f32_32x32x64_f8f6f4: one instruction covers
+// the 64 K bytes of a sub-step (the two 16-byte pieces a lane holds), takes the E8M0 scale of the lane's weight
+// column block and of its activation row for the current 128-byte K block, and accumulates in fp32.  The
+// scales of the item wait in LDS (a_scale8_s[kb * 256 + tile row], w_scale8_s[column group * kScaleKb + kb]) and
+// are read with the fragments.
+template <int MF, int TEAM, bool FLAT, bool FP8>
 __device__ __forceinline__ void run_item(const GemmArgs &a, const ItemCtx &t, int nb, int8_t *lds,
-                                         const float *row_scale_s)
+                                         const float *row_scale_s, const uint8_t *a_scale8_s,
+                                         const uint8_t *w_scale8_s)
 {
     constexpr int NS = FLAT ? 3 : 4;                       // ring of stages
     constexpr int LPS = FLAT ? (TEAM == 0 ? 6 : 4) : 4;    // loads per wave and sub-step
@@ -129,7 +149,7 @@ __device__ __forceinline__ void run_item(const GemmArgs &a, const ItemCtx &t, in
     const int last = KT - 1;
     const unsigned lds0 = (unsigned)(unsigned long long)(__attribute__((address_space(3))) int8_t *)lds;
 
-    v16i acc[MFR][2];
+    typename AccType<FP8>::type acc[MFR][2];
 #pragma unroll
     for (int mf = 0; mf < MFR; ++mf) {
 #pragma unroll
@@ -185,37 +205,60 @@ __device__ __forceinline__ void run_item(const GemmArgs &a, const ItemCtx &t, in
     };
 
     // ---- fragments: read from LDS one phase before they are multiplied.
-    v4i af[2][MFR];
-    v4i bf[2][2];
+    v8i af[MFR];  // .lo: the K bytes of the first 32-byte half of the sub-step, .hi: of the second
+    v8i bf[2];
+    int sa[MFR];  // FP8: E8M0 scales of this lane's activation rows, and of its two weight column fragments
+    int sw[2] = {0, 0};
     const int a_row = lane & 31;
     const int a_half = lane >> 5;
-    auto read_frags = [&](int slot) {
+    auto read_frags = [&](int slot, int s_idx) {
         const int8_t *st = lds + slot * t.stage_bytes;
         const int8_t *sb = st + t.stage_a + t.bslot * 4096 + lane * 16;
 #pragma unroll
-        for (int kk = 0; kk < 2; ++kk) {
+        for (int nf = 0; nf < 2; ++nf) {
+            bf[nf].lo = *(const v4i *)(sb + nf * 1024);
+            bf[nf].hi = *(const v4i *)(sb + (2 + nf) * 1024);
+        }
 #pragma unroll
-            for (int nf = 0; nf < 2; ++nf) {
-                bf[kk][nf] = *(const v4i *)(sb + (kk * 2 + nf) * 1024);
-            }
+        for (int mf = 0; mf < MF; ++mf) {
+            af[mf].lo = *(const v4i *)(st + a_lds_offset(t.a_row0 + mf * 32 + a_row, a_half));
+            af[mf].hi = *(const v4i *)(st + a_lds_offset(t.a_row0 + mf * 32 + a_row, 2 + a_half));
+        }
+        if (FP8) {
+            const int kb = min(s_idx, last) >> 1;
+            sw[0] = w_scale8_s[(t.bslot * 2 + 0) * kScaleKb + kb];
+            sw[1] = w_scale8_s[(t.bslot * 2 + 1) * kScaleKb + kb];
 #pragma unroll
             for (int mf = 0; mf < MF; ++mf) {
-                af[kk][mf] = *(const v4i *)(st + a_lds_offset(t.a_row0 + mf * 32 + a_row, kk * 2 + a_half));
+                sa[mf] = a_scale8_s[kb * 256 + t.a_row0 + mf * 32 + a_row];
             }
         }
     };
     auto multiply = [&]() {
         __builtin_amdgcn_sched_barrier(0);
         __builtin_amdgcn_s_setprio(2);
-#pragma unroll
-        for (int kk = 0; kk < 2; ++kk) {
+        // Weights as the first operand: the result tile comes out transposed, i.e. a lane holds ONE
+        // activation row and 4 consecutive weight columns per register quad.
+        if constexpr (FP8) {
 #pragma unroll
             for (int mf = 0; mf < MF; ++mf) {
 #pragma unroll
                 for (int nf = 0; nf < 2; ++nf) {
-                    // Weights as the first operand: the result tile comes out transposed, i.e. a lane holds ONE
-                    // activation row and 4 consecutive weight columns per register quad.
-                    acc[mf][nf] = __builtin_amdgcn_mfma_i32_32x32x32_i8(bf[kk][nf], af[kk][mf], acc[mf][nf], 0, 0, 0);
+                    acc[mf][nf] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(bf[nf], af[mf], acc[mf][nf], 0, 0, 0,
+                                                                                 sw[nf], 0, sa[mf]);
+                }
+            }
+        } else {
+#pragma unroll
+            for (int kk = 0; kk < 2; ++kk) {
+#pragma unroll
+                for (int mf = 0; mf < MF; ++mf) {
+#pragma unroll
+                    for (int nf = 0; nf < 2; ++nf) {
+                        acc[mf][nf] = __builtin_amdgcn_mfma_i32_32x32x32_i8(kk == 0 ? bf[nf].lo : bf[nf].hi,
+                                                                            kk == 0 ? af[mf].lo : af[mf].hi,
+                                                                            acc[mf][nf], 0, 0, 0);
+                    }
                 }
             }
         }
@@ -239,7 +282,7 @@ __device__ __forceinline__ void run_item(const GemmArgs &a, const ItemCtx &t, in
     barrier_no_fence();  // stage 0 has landed
     int slot = 0;        // slot of stage s
     if (TEAM == 0) {
-        read_frags(0);
+        read_frags(0, 0);
         wait_lds_reads();
         for (int s = 0; s < KT; ++s) {
             const int next = slot + 1 == NS ? 0 : slot + 1;
@@ -247,7 +290,7 @@ __device__ __forceinline__ void run_item(const GemmArgs &a, const ItemCtx &t, in
             wait_loads_outstanding<(NS - 2) * LPS>();     // my part of stage s+1 has landed
             barrier_no_fence();                           // A(s)
             issue(s + NS, slot);                          // phase 2: refill stage s's slot ...
-            read_frags(next);                             // ... and fetch the fragments of stage s+1
+            read_frags(next, s + 1);                      // ... and fetch the fragments of stage s+1
             wait_lds_reads();
             barrier_no_fence();                           // B(s)
             slot = next;
@@ -255,7 +298,7 @@ __device__ __forceinline__ void run_item(const GemmArgs &a, const ItemCtx &t, in
     } else {
         for (int s = 0; s < KT; ++s) {
             const int next = slot + 1 == NS ? 0 : slot + 1;
-            read_frags(slot);                             // phase 1: fragments of stage s ...
+            read_frags(slot, s);                          // phase 1: fragments of stage s ...
             wait_lds_reads();
             issue(s + NS, slot);                          // ... then refill its slot
             wait_loads_outstanding<(NS - 1) * LPS>();     // my part of stage s+1 has landed
@@ -306,8 +349,9 @@ __device__ __forceinline__ void run_item(const GemmArgs &a, const ItemCtx &t, in
                 for (int mf = 0; mf < MF; ++mf) {
 #pragma unroll
                     for (int j = 0; j < 4; ++j) {
-                        const v4i v = {acc[mf][nf][4 * j], acc[mf][nf][4 * j + 1], acc[mf][nf][4 * j + 2],
-                                       acc[mf][nf][4 * j + 3]};
+                        // int32 sums, or the bits of the fp32 sums of an FP8 item
+                        const v4i v = {acc_bits(acc[mf][nf][4 * j]), acc_bits(acc[mf][nf][4 * j + 1]),
+                                       acc_bits(acc[mf][nf][4 * j + 2]), acc_bits(acc[mf][nf][4 * j + 3])};
                         *(v4i *)(slice + row_in * kEpiRowBytes + (8 * j + col_half) * 4) = v;
                     }
                     flush_fragment((int8_t *)a.out + (long long)col0 * 4, (long long)N * 4, mf);
@@ -317,21 +361,29 @@ __device__ __forceinline__ void run_item(const GemmArgs &a, const ItemCtx &t, in
             // t = (float(C) * w_scale[n]) * x_scale[m]; y = silu(t_gate) * t_up
             const int I = N / 2;
             v4f sg_gate[4], sg_up[4];
+            if (!FP8) {
 #pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                sg_gate[j] = *(const v4f *)(t.sg + nw * 32 + 8 * j + col_half);
-                sg_up[j] = *(const v4f *)(t.sg + I + nw * 32 + 8 * j + col_half);
+                for (int j = 0; j < 4; ++j) {
+                    sg_gate[j] = *(const v4f *)(t.sg + nw * 32 + 8 * j + col_half);
+                    sg_up[j] = *(const v4f *)(t.sg + I + nw * 32 + 8 * j + col_half);
+                }
             }
 #pragma unroll
             for (int mf = 0; mf < MF; ++mf) {
-                const float xs = row_scale_s[t.a_row0 + mf * 32 + row_in];
+                const float xs = FP8 ? 1.0f : row_scale_s[t.a_row0 + mf * 32 + row_in];
 #pragma unroll
                 for (int j = 0; j < 4; ++j) {
                     v4f y;
 #pragma unroll
                     for (int e = 0; e < 4; ++e) {
-                        const float tg = __fmul_rn(__fmul_rn((float)acc[mf][0][4 * j + e], sg_gate[j][e]), xs);
-                        const float tu = __fmul_rn(__fmul_rn((float)acc[mf][1][4 * j + e], sg_up[j][e]), xs);
+                        float tg, tu;
+                        if constexpr (FP8) {  // the sums carry their scales already
+                            tg = acc[mf][0][4 * j + e];
+                            tu = acc[mf][1][4 * j + e];
+                        } else {
+                            tg = __fmul_rn(__fmul_rn((float)acc[mf][0][4 * j + e], sg_gate[j][e]), xs);
+                            tu = __fmul_rn(__fmul_rn((float)acc[mf][1][4 * j + e], sg_up[j][e]), xs);
+                        }
                         y[e] = __fmul_rn(cam_silu_spec(tg), tu);
                     }
                     *(v4f *)(slice + row_in * kEpiRowBytes + (8 * j + col_half) * 4) = y;
@@ -340,16 +392,18 @@ __device__ __forceinline__ void run_item(const GemmArgs &a, const ItemCtx &t, in
             }
         } else {
             v4f ws[2][4];
+            if (!FP8) {
 #pragma unroll
-            for (int nf = 0; nf < 2; ++nf) {
+                for (int nf = 0; nf < 2; ++nf) {
 #pragma unroll
-                for (int j = 0; j < 4; ++j) {
-                    ws[nf][j] = *(const v4f *)(t.sg + nw * 64 + nf * 32 + 8 * j + col_half);
+                    for (int j = 0; j < 4; ++j) {
+                        ws[nf][j] = *(const v4f *)(t.sg + nw * 64 + nf * 32 + 8 * j + col_half);
+                    }
                 }
             }
 #pragma unroll
             for (int mf = 0; mf < MF; ++mf) {
-                const float xs = row_scale_s[t.a_row0 + mf * 32 + row_in];
+                const float xs = FP8 ? 1.0f : row_scale_s[t.a_row0 + mf * 32 + row_in];
 #pragma unroll
                 for (int nf = 0; nf < 2; ++nf) {
 #pragma unroll
@@ -357,8 +411,12 @@ __device__ __forceinline__ void run_item(const GemmArgs &a, const ItemCtx &t, in
                         uint32_t b[4];
 #pragma unroll
                         for (int e = 0; e < 4; ++e) {
-                            b[e] = f32_to_bf16_bits(
-                                __fmul_rn(__fmul_rn((float)acc[mf][nf][4 * j + e], ws[nf][j][e]), xs));
+                            if constexpr (FP8) {
+                                b[e] = f32_to_bf16_bits(acc[mf][nf][4 * j + e]);
+                            } else {
+                                b[e] = f32_to_bf16_bits(
+                                    __fmul_rn(__fmul_rn((float)acc[mf][nf][4 * j + e], ws[nf][j][e]), xs));
+                            }
                         }
                         const v2u v = {b[0] | (b[1] << 16), b[2] | (b[3] << 16)};
                         *(v2u *)(slice + row_in * kEpiRowBytes + (nf * 32 + 8 * j + col_half) * 2) = v;
@@ -374,23 +432,27 @@ __device__ __forceinline__ void run_item(const GemmArgs &a, const ItemCtx &t, in
     barrier_no_fence();  // the staging slices are free again before the next item's loads land
 }
 
-template <int TEAM, bool FLAT>
+template <int TEAM, bool FLAT, bool FP8>
 __device__ __forceinline__ void run_item_mf(int mf, const GemmArgs &a, const ItemCtx &t, int nb, int8_t *lds,
-                                            const float *row_scale_s)
+                                            const float *row_scale_s, const uint8_t *a_scale8_s,
+                                            const uint8_t *w_scale8_s)
 {
     switch (mf) {
-        case 0: run_item<0, TEAM, FLAT>(a, t, nb, lds, row_scale_s); break;
-        case 1: run_item<1, TEAM, FLAT>(a, t, nb, lds, row_scale_s); break;
-        case 2: run_item<2, TEAM, FLAT>(a, t, nb, lds, row_scale_s); break;
-        case 3: run_item<3, TEAM, FLAT>(a, t, nb, lds, row_scale_s); break;
-        default: run_item<4, TEAM, FLAT>(a, t, nb, lds, row_scale_s); break;
+        case 0: run_item<0, TEAM, FLAT, FP8>(a, t, nb, lds, row_scale_s, a_scale8_s, w_scale8_s); break;
+        case 1: run_item<1, TEAM, FLAT, FP8>(a, t, nb, lds, row_scale_s, a_scale8_s, w_scale8_s); break;
+        case 2: run_item<2, TEAM, FLAT, FP8>(a, t, nb, lds, row_scale_s, a_scale8_s, w_scale8_s); break;
+        case 3: run_item<3, TEAM, FLAT, FP8>(a, t, nb, lds, row_scale_s, a_scale8_s, w_scale8_s); break;
+        default: run_item<4, TEAM, FLAT, FP8>(a, t, nb, lds, row_scale_s, a_scale8_s, w_scale8_s); break;
     }
 }
 
+template <bool FP8>
 __global__ __launch_bounds__(kThreads, 1) void gemm_kernel(GemmArgs a)
 {
     __shared__ __attribute__((aligned(1024))) int8_t lds[kLdsBytes];
     __shared__ float row_scale_s[256];
+    __shared__ uint8_t a_scale8_s[FP8 ? kScaleKb * 256 : 4];
+    __shared__ uint8_t w_scale8_s[FP8 ? 16 * kScaleKb : 4];
     __shared__ int item_s;
 
     const int tid = threadIdx.x;
@@ -481,7 +543,25 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_kernel(GemmArgs a)
         const int group = nb * (flat ? 8 : 4) + t.bslot;
         t.wave_live = group < a.N / 64;
         t.nw = min(group, a.N / 64 - 1);
-        if (a.epilogue != kEpiInt32 && tid < 256) {
+        if (FP8) {
+            // the item's scales: activation rows x K blocks (transposed, so that the lanes of a fragment read
+            // neighbouring bytes), and one row of K blocks per 64-column group of the item
+            const int KB = a.Kd >> 7;
+            for (int i = tid; i < 256 * KB; i += kThreads) {
+                const int r = i / KB, kb = i - r * KB;
+                a_scale8_s[kb * 256 + r] = a.a_scale8[(long long)(m0 + min(r, rows - 1)) * KB + kb];
+            }
+            const int ngr = flat ? 8 : 4;
+            const int nblk = a.N >> 7;
+            for (int i = tid; i < ngr * 2 * KB; i += kThreads) {
+                const int gf = i / KB, kb = i - gf * KB;  // gf = column group of the item * 2 + fragment
+                const int grp = min(nb * ngr + (gf >> 1), a.N / 64 - 1);  // packed 64-column group of the weight
+                const int nf = gf & 1;
+                // first logical column of the fragment (a paired group holds 32 gate and 32 up columns)
+                const int col = a.gate_up ? nf * (a.N / 2) + grp * 32 : grp * 64 + nf * 32;
+                w_scale8_s[gf * kScaleKb + kb] = a.w_scale8[((long long)g * KB + kb) * nblk + (col >> 7)];
+            }
+        } else if (a.epilogue != kEpiInt32 && tid < 256) {
             row_scale_s[tid] = a.a_scale[m0 + min(tid, rows - 1)];
         }
         __syncthreads();  // item_s may be rewritten and the row scales read from here on
@@ -489,15 +569,15 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_kernel(GemmArgs a)
         const int mf = t.my_rows <= 0 ? 0 : (t.my_rows + 31) >> 5;
         if (flat) {
             if (team == 0) {
-                run_item_mf<0, true>(mf, a, t, nb, lds, row_scale_s);
+                run_item_mf<0, true, FP8>(mf, a, t, nb, lds, row_scale_s, a_scale8_s, w_scale8_s);
             } else {
-                run_item_mf<1, true>(mf, a, t, nb, lds, row_scale_s);
+                run_item_mf<1, true, FP8>(mf, a, t, nb, lds, row_scale_s, a_scale8_s, w_scale8_s);
             }
         } else {
             if (team == 0) {
-                run_item_mf<0, false>(mf, a, t, nb, lds, row_scale_s);
+                run_item_mf<0, false, FP8>(mf, a, t, nb, lds, row_scale_s, a_scale8_s, w_scale8_s);
             } else {
-                run_item_mf<1, false>(mf, a, t, nb, lds, row_scale_s);
+                run_item_mf<1, false, FP8>(mf, a, t, nb, lds, row_scale_s, a_scale8_s, w_scale8_s);
             }
         }
         if (tid == 0) {
@@ -820,6 +900,66 @@ __global__ __launch_bounds__(256) void requant_kernel(const float *__restrict__ 
     }
 }
 
+// fp32 rows -> FP8 E4M3 with one E8M0 scale per row and 128 columns (include/cam_fp8_spec.h).  A wave takes 512
+// columns of a row: lane l the 8 columns from 8 l, so a block of 128 columns is a quarter of the wave.
+__global__ __launch_bounds__(256) void requant_fp8_kernel(const float *__restrict__ y, int I,
+                                                          const int32_t *__restrict__ sched, long long max_rows,
+                                                          uint8_t *__restrict__ q, uint8_t *__restrict__ scale)
+{
+    const long long row = blockIdx.x;
+    const long long valid = sched != nullptr ? min((long long)sched[1], max_rows) : max_rows;
+    if (row >= valid) {
+        return;
+    }
+    const int lane = threadIdx.x & (kWave - 1);
+    const int wave = threadIdx.x >> 6;
+    for (int c0 = wave * 512; c0 < I; c0 += 4 * 512) {
+        const int col = c0 + lane * 8;
+        const bool live = col < I;
+        float x[8];
+        float m = 0.0f;
+        if (live) {
+            const v4f lo = __builtin_nontemporal_load((const v4f *)(y + row * I + col));
+            const v4f hi = __builtin_nontemporal_load((const v4f *)(y + row * I + col + 4));
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                x[e] = lo[e];
+                x[4 + e] = hi[e];
+            }
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                m = fmaxf(m, fabsf(x[e]));
+            }
+        } else {
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                x[e] = 0.0f;
+            }
+        }
+#pragma unroll
+        for (int off = 1; off < 16; off <<= 1) {
+            m = fmaxf(m, __shfl_xor(m, off, kWave));
+        }
+        const int ex = fp8_block_scale_exp(m);
+        const float f1 = exp2_int(-(ex / 2)), f2 = exp2_int(-(ex - ex / 2));
+        int lo = 0, hi = 0;
+        lo = __builtin_amdgcn_cvt_pk_fp8_f32(__fmul_rn(__fmul_rn(x[0], f1), f2), __fmul_rn(__fmul_rn(x[1], f1), f2), lo,
+                                             false);
+        lo = __builtin_amdgcn_cvt_pk_fp8_f32(__fmul_rn(__fmul_rn(x[2], f1), f2), __fmul_rn(__fmul_rn(x[3], f1), f2), lo,
+                                             true);
+        hi = __builtin_amdgcn_cvt_pk_fp8_f32(__fmul_rn(__fmul_rn(x[4], f1), f2), __fmul_rn(__fmul_rn(x[5], f1), f2), hi,
+                                             false);
+        hi = __builtin_amdgcn_cvt_pk_fp8_f32(__fmul_rn(__fmul_rn(x[6], f1), f2), __fmul_rn(__fmul_rn(x[7], f1), f2), hi,
+                                             true);
+        if (live) {
+            *(v2u *)(q + row * I + col) = v2u{(uint32_t)lo, (uint32_t)hi};
+            if ((lane & 15) == 0) {
+                scale[row * (I >> 7) + (col >> 7)] = (uint8_t)(ex + 127);
+            }
+        }
+    }
+}
+
 // Row-major [G,Kd,N] int8 -> MFMA operand order.  One thread writes one 16-byte piece:
 //   piece index = (((g*NW + nw)*KS + ks)*2 + nf)*64 + lane, holding K rows ks*32 + (lane/32)*16 + 0..15 of
 //   logical column  gate_up ? nf*(N/2) + nw*32 + lane%32 : nw*64 + nf*32 + lane%32.
@@ -902,7 +1042,15 @@ hipError_t launch_gemm(const GemmArgs &a, hipStream_t stream)
         }
         g_num_cus = n > 0 ? n : 256;
     }
-    hipLaunchKernelGGL(gemm_kernel, dim3((unsigned)g_num_cus), dim3(kThreads), 0, stream, a);
+    if (a.fp8) {
+        if (a.Kd % 128 != 0 || a.N % 128 != 0 || (a.gate_up && a.N % 256 != 0) || a.Kd / 128 > kScaleKb ||
+            a.per_expert || a.a_scale8 == nullptr || a.w_scale8 == nullptr) {
+            return hipErrorInvalidValue;
+        }
+        hipLaunchKernelGGL(gemm_kernel<true>, dim3((unsigned)g_num_cus), dim3(kThreads), 0, stream, a);
+    } else {
+        hipLaunchKernelGGL(gemm_kernel<false>, dim3((unsigned)g_num_cus), dim3(kThreads), 0, stream, a);
+    }
     return hipGetLastError();
 }
 
@@ -916,6 +1064,20 @@ hipError_t launch_requant(const float *y, int64_t max_rows, int I, const int32_t
         return hipErrorInvalidValue;
     }
     hipLaunchKernelGGL(requant_kernel, dim3((unsigned)max_rows), dim3(256), 0, stream, y, I, sched_for_rows,
+                       (long long)max_rows, q, scale);
+    return hipGetLastError();
+}
+
+hipError_t launch_requant_fp8(const float *y, int64_t max_rows, int I, const int32_t *sched_for_rows, uint8_t *q,
+                              uint8_t *scale, hipStream_t stream)
+{
+    if (max_rows <= 0) {
+        return hipSuccess;
+    }
+    if (I % 128 != 0) {
+        return hipErrorInvalidValue;
+    }
+    hipLaunchKernelGGL(requant_fp8_kernel, dim3((unsigned)max_rows), dim3(256), 0, stream, y, I, sched_for_rows,
                        (long long)max_rows, q, scale);
     return hipGetLastError();
 }

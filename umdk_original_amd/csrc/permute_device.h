@@ -7,6 +7,8 @@
 //           src/cam/comm_operator/ascend_kernels/fused_deep_moe/op_kernel/fused_deep_moe/gemm/kernel/
 //           grouped_matmul_slice_m_per_token_dequant_swiglu_quant_multistage_workspace.h:780-818 (no epsilon)
 //   rows    moe_dispatch_normal.h:486-535 (int8 or 16-bit row, fp32 scale and (srcRank, token, k) per row)
+// QUANT 3 has no counterpart in the reference: OCP FP8 E4M3 values with one power-of-two (E8M0) scale per row
+// and 128 columns, as include/cam_fp8_spec.h defines them.
 #ifndef CAM_PERMUTE_DEVICE_H_
 #define CAM_PERMUTE_DEVICE_H_
 
@@ -39,7 +41,35 @@ struct TokenRow {
     v4u raw[kDispMaxChunks];
     v2u q[kDispMaxChunks];
     float scale_out;
+    uint32_t scale8[kDispMaxChunks];  // QUANT 3: E8M0 scale of the 128-column block chunk j of this lane lies in
 };
+
+// Exponent x of the smallest power of two 2^x with amax / 2^x <= 448 (amax = m * 2^e: e - 8, one more when
+// m > 1.75), 0 for amax == 0, clamped to [-127, 127].
+__device__ __forceinline__ int fp8_block_scale_exp(float amax)
+{
+    const uint32_t a = __float_as_uint(amax);
+    if (a == 0u) {
+        return 0;
+    }
+    int e;
+    uint32_t frac;
+    if ((a >> 23) == 0u) {
+        const int lead = __clz(a) - 9;  // shifts that bring the leading one to bit 22
+        e = -127 - lead;
+        frac = (a << (lead + 1)) & 0x7fffffu;
+    } else {
+        e = (int)(a >> 23) - 127;
+        frac = a & 0x7fffffu;
+    }
+    const int x = e - 8 + (frac > 0x600000u ? 1 : 0);
+    return min(max(x, -127), 127);
+}
+
+__device__ __forceinline__ float exp2_int(int x)
+{
+    return x >= -126 ? __uint_as_float((uint32_t)(x + 127) << 23) : __uint_as_float(0x00400000u);
+}
 
 __device__ __forceinline__ void load_token_row(const uint16_t *x, int t, int H, int lane, TokenRow &r)
 {
@@ -55,10 +85,51 @@ __device__ __forceinline__ void load_token_row(const uint16_t *x, int t, int H, 
     }
 }
 
+// FP8 with one scale per 128 columns.  Chunk c = 64 j + lane holds columns 8c .. 8c+7, so a block of 128
+// columns is the 16 chunks of lanes 16 q .. 16 q + 15 at one j: its largest magnitude is a maximum over a
+// quarter of the wave.  The scaled values lie within +-448, where the hardware conversion (round to nearest
+// even) needs no saturation.
+template <int ACT>
+__device__ __forceinline__ void quant_token_row_fp8(TokenRow &r)
+{
+#pragma unroll
+    for (int j = 0; j < kDispMaxChunks; ++j) {
+        float x[8];
+        float m = 0.0f;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            x[2 * i] = act_bits_to_f32<ACT>(r.raw[j][i] & 0xffffu);
+            x[2 * i + 1] = act_bits_to_f32<ACT>(r.raw[j][i] >> 16);
+            m = fmaxf(m, fmaxf(fabsf(x[2 * i]), fabsf(x[2 * i + 1])));
+        }
+#pragma unroll
+        for (int off = 1; off < 16; off <<= 1) {
+            m = fmaxf(m, __shfl_xor(m, off, kWave));
+        }
+        const int e = fp8_block_scale_exp(m);
+        r.scale8[j] = (uint32_t)(e + 127);
+        const float f1 = exp2_int(-(e / 2)), f2 = exp2_int(-(e - e / 2));
+        int lo = 0, hi = 0;
+        lo = __builtin_amdgcn_cvt_pk_fp8_f32(__fmul_rn(__fmul_rn(x[0], f1), f2), __fmul_rn(__fmul_rn(x[1], f1), f2), lo,
+                                             false);
+        lo = __builtin_amdgcn_cvt_pk_fp8_f32(__fmul_rn(__fmul_rn(x[2], f1), f2), __fmul_rn(__fmul_rn(x[3], f1), f2), lo,
+                                             true);
+        hi = __builtin_amdgcn_cvt_pk_fp8_f32(__fmul_rn(__fmul_rn(x[4], f1), f2), __fmul_rn(__fmul_rn(x[5], f1), f2), hi,
+                                             false);
+        hi = __builtin_amdgcn_cvt_pk_fp8_f32(__fmul_rn(__fmul_rn(x[6], f1), f2), __fmul_rn(__fmul_rn(x[7], f1), f2), hi,
+                                             true);
+        r.q[j] = v2u{(uint32_t)lo, (uint32_t)hi};
+    }
+}
+
 // QUANT 1: scale = 127 / (max|x| + 1e-12); QUANT 2: scale = 127 / max|x|, an all-zero row giving zeros and scale 0.
 template <int QUANT, int ACT>
 __device__ __forceinline__ void quant_token_row(TokenRow &r)
 {
+    if (QUANT == 3) {
+        quant_token_row_fp8<ACT>(r);
+        return;
+    }
     float m = 0.0f;
 #pragma unroll
     for (int j = 0; j < kDispMaxChunks; ++j) {
@@ -115,8 +186,21 @@ __device__ __forceinline__ void store_token_row(const TokenRow &r, void *out, fl
             }
         }
     }
+    if (QUANT == 3) {
+        // one E8M0 byte per 128 columns, written by the first lane of each quarter of the wave
+        uint8_t *sc = (uint8_t *)scales + row * (H >> 7);
+        if ((lane & 15) == 0) {
+#pragma unroll
+            for (int j = 0; j < kDispMaxChunks; ++j) {
+                const int c = j * kWave + lane;
+                if (c < nch) {
+                    sc[c >> 4] = (uint8_t)r.scale8[j];
+                }
+            }
+        }
+    }
     if (lane == 0) {
-        if (QUANT != 0) {
+        if (QUANT == 1 || QUANT == 2) {
             scales[row] = r.scale_out;
         }
         if (src_info != nullptr) {

@@ -112,9 +112,15 @@ def moe_dispatch_fused(x, topk_idx, num_experts, quant_mode=0, num_rows=None, ra
     A = max(int(T * K if num_rows is None else num_rows), 1)
     dev = x.device
     i32 = dict(dtype=torch.int32, device=dev)
+    if quant_mode == 4:   # block-scaled FP8: E4M3 rows, one E8M0 scale per row and 128 columns
+        rx = torch.empty((A, H), dtype=torch.float8_e4m3fn, device=dev)
+        rs = torch.empty((A, H // 128), dtype=torch.uint8, device=dev)
+    else:
+        rx = torch.empty((A, H), dtype=torch.int8 if quant_mode != 0 else x.dtype, device=dev)
+        rs = torch.empty(A, dtype=torch.float32, device=dev)
     out = dict(
-        recv_x=torch.empty((A, H), dtype=torch.int8 if quant_mode != 0 else x.dtype, device=dev),
-        recv_x_scales=torch.empty(A, dtype=torch.float32, device=dev),
+        recv_x=rx,
+        recv_x_scales=rs,
         expand_idx=torch.empty(3 * A, **i32),
         send_token_idx=torch.empty((T, K), **i32),
         slot_row=torch.empty((T, K), **i32),
@@ -297,6 +303,46 @@ def grouped_matmul_int32(x, weight, group_list, group_list_type=0):
     out = torch.zeros((x.size(0), weight[0].size(-1)), dtype=torch.int32, device=x.device)
     _lib.call("GroupedMatmulInt32", [x, weight, 1 if gate_up else 0, group_list, group_list_type, out])
     return out
+
+
+# --------------------------------------------------------------------------------------------------
+# Block-scaled FP8 (a definition of this library: include/cam_fp8_spec.h; the reference is W8A8 only)
+def grouped_matmul_fp8(x, x_scale, weight, weight_scale, group_list, group_list_type=0, out_dtype=torch.float32):
+    """x E4M3 [A,K], x_scale uint8 [A,K/128], weight E4M3 [G,K,N] prepacked, weight_scale uint8 [G,K/128,N/128].
+    Prepacked with gate_up=True: -> fp32 [A,N/2] = silu(gate) * up; else -> out_dtype [A,N] (fp32 sums or bf16)."""
+    _tag_list([weight])
+    gate_up = bool(getattr(weight, "_cam_gate_up", False))
+    n = weight.size(-1)
+    if gate_up:
+        out = torch.empty((x.size(0), n // 2), dtype=torch.float32, device=x.device)
+    else:
+        out = torch.empty((x.size(0), n), dtype=out_dtype, device=x.device)
+    _lib.call("GroupedMatmulFp8", [x, x_scale, weight, weight_scale, 1 if gate_up else 0, group_list,
+                                   group_list_type, out])
+    return out
+
+
+def quant_rows_fp8(x):
+    """fp32 [A,I] -> (E4M3 [A,I], uint8 E8M0 scales [A,I/128])."""
+    _require_gpu(x, "x")
+    q = torch.empty(x.shape, dtype=torch.float8_e4m3fn, device=x.device)
+    sc = torch.empty((x.size(0), x.size(1) // 128), dtype=torch.uint8, device=x.device)
+    _lib.call("QuantRowsFp8", [x, q, sc])
+    return q, sc
+
+
+def fused_deep_moe_fp8(x, expert_ids, gmm1_weight, gmm1_weight_scale, gmm2_weight, gmm2_weight_scale, expert_scales,
+                       x_active_mask=None, moe_expert_num=0):
+    """-> [output bf16 [bs,H], expertTokenNums int64 [experts]]."""
+    _require_gpu(x, "x")
+    _tag_list([gmm1_weight, gmm2_weight])
+    bs, h = x.shape
+    e = moe_expert_num or gmm1_weight.size(0)
+    output = torch.empty((bs, h), dtype=torch.bfloat16, device=x.device)
+    etn = torch.empty(e, dtype=torch.int64, device=x.device)
+    _lib.call("FusedDeepMoeFp8", [x, expert_ids, gmm1_weight, gmm1_weight_scale, gmm2_weight, gmm2_weight_scale,
+                                  expert_scales, x_active_mask, e, output, etn])
+    return [output, etn]
 
 
 def fused_deep_moe(x, expertIds, gmm1PermutedWeight, gmm1PermutedWeightScale, gmm2Weight, gmm2WeightScale,
