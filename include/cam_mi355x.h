@@ -204,7 +204,9 @@ CAM_API camStatus camMoeDispatchNormal(void *workspace, uint64_t workspaceSize, 
  * exchanged counts, two device-to-host copies and the aclnnMoeDispatchNormal call) as ONE kernel launch for
  * one rank: MoeDispatchPlan and MoeDispatchNormal fused, with the plan running underneath the first row
  * loads.  x bf16/fp16 [T,H]; topkIdx int64/int32 [T,K] -> recvX [A,H] (int8 when quantMode is 2 or 3, else
- * x's dtype), recvXScalesOptional fp32 [A] (required when quantising), expandIdx int32 [3A] = (srcRank,
+ * x's dtype), recvXScalesOptional fp32 [A] (required when quantising); quantMode 4, which the reference does
+ * not have, gives block-scaled FP8 rows instead (recvX E4M3 [A,H], recvXScales uint8 [A,H/128], cam_fp8_spec.h);
+ * expandIdx int32 [3A] = (srcRank,
  * token, k) per row, sendTokenIdx int32 [T,K]; optional slotRow int32 [T,K], numTokensPerExpert int32 [E],
  * sendOffset int32 [E], recvCount int32 [E], numRecvTokensPerExpert int64 [E], totalRecvTokens int64 [1],
  * all exactly as MoeDispatchPlan / MoeDispatchNormal produce them.  Rows outside [0,A) are dropped, so A
@@ -224,8 +226,9 @@ CAM_API camStatus camMoeDispatchPrefill(void *workspace, uint64_t workspaceSize,
 
 /* ------------------------------------------------------------------------------------------------
  * MoeCombineNormal -- replaces aclnnMoeCombineNormal (AUTOGEN/aclnn_moe_combine_normal.h:37-65).
- * recvX bf16 [A,H]; tokenSrcInfo int32 [3A]; epRecvCounts int32 [E]; recvTopkWeights fp32 [T,K]
- * -> out bf16 [T,H].  out[t] = bf16(sum over k ascending of float(recvX[row(t,k)]) * w[t,k]), multiply
+ * recvX bf16 or fp16 [A,H]; tokenSrcInfo int32 [3A]; epRecvCounts int32 [E]; recvTopkWeights fp32 [T,K]
+ * -> out [T,H] of recvX's type (op_host/moe_combine_normal.cpp:18,49 lists both 16-bit types).
+ * out[t] = round(sum over k ascending of float(recvX[row(t,k)]) * w[t,k]), multiply
  * and add rounded separately (AK/moe_combine_normal/op_kernel/moe_combine_normal.h:303-338); row(t,k) is
  * the row whose triple names (t,k) (:232-238).  Slots no row names contribute nothing.  Only the first
  * epRecvCounts[E-1] rows are looked at (:206-207): rows past the receive total were never written.
@@ -301,7 +304,7 @@ CAM_API camStatus camGroupedMatmulSwigluQuant(void *workspace, uint64_t workspac
  * FDM/gemm/kernel/grouped_matmul_slice_m_per_token_dequant_multistage_workspace.h:24-378; epilogue
  * FDM/epilogue/block/block_epilogue_per_token_dequant.hpp:572-703).
  * x int8 [A,I]; xScale fp32 [A]; weight list [G,I,H] / G x [I,H], CAM_FORMAT_MFMA_B with gateUp=0;
- * weightScale fp32 [G,H] -> out bf16 [A,H] = bf16((float(acc) * weightScale[g][h]) * xScale[m]).
+ * weightScale fp32 [G,H] -> out bf16 (or fp16) [A,H] = round((float(acc) * weightScale[g][h]) * xScale[m]).
  * out int8 [A, H + H/4] selects wire rows instead: every bf16 row above is quantised in blocks of 8 columns as
  * AK/moe_combine_shmem/op_kernel/moe_combine_shmem.h:567-592 does before a row leaves the rank:
  *   m = max |x| over the block; s = m * (1/127); q = int8(half(x / s)) (both casts round to nearest even);
@@ -328,13 +331,14 @@ CAM_API camStatus camGroupedMatmulInt32(void *workspace, uint64_t workspaceSize,
 
 /* ------------------------------------------------------------------------------------------------
  * FusedDeepMoe -- replaces aclnnFusedDeepMoe (AUTOGEN/aclnn_fused_deep_moe.h:19-46).
- * x bf16 [bs,H]; expertIds int32 [bs,K]; gmm1PermutedWeight int8 [Epr,H,2I] (or Epr x [H,2I]),
+ * x bf16 or fp16 [bs,H]; expertIds int32 [bs,K]; gmm1PermutedWeight int8 [Epr,H,2I] (or Epr x [H,2I]),
  * CAM_FORMAT_MFMA_B gateUp=1; gmm1PermutedWeightScale fp32 [Epr,2I]; gmm2Weight int8 [Epr,I,H],
  * CAM_FORMAT_MFMA_B gateUp=0; gmm2WeightScale fp32 [Epr,H]; expertScales fp32 [bs,K];
  * expertSmoothScalesOptional must be NULL (the reference stores and never uses it,
  * AK/fused_deep_moe/op_kernel/fused_deep_moe.h:307); xActiveMaskOptional bool [bs], prefix semantics
- * (…swiglu_quant_multistage_workspace.h:647-678) -> output bf16 [bs,H], expertTokenNums int64 [Epr].
- * quantMode is accepted and ignored, as in the reference (fused_deep_moe.h:148,326).
+ * (…swiglu_quant_multistage_workspace.h:647-678) -> output [bs,H] of x's type (the expert rows GMM2 writes
+ * and the combined rows take it too), expertTokenNums int64 [Epr].
+ * quantMode in [0, 3] is accepted and has no effect, as in the reference (fused_deep_moe.h:148,326).
  * epRankSize must be 1 and sharedExpertRankNum 0.  Output rows of masked tokens are zero.
  * Limits kept (AK/fused_deep_moe/op_host/fused_deep_moe_tiling.cpp:49-61): 512 <= H <= 7168,
  * 1024 <= 2I <= 6144, K <= 12, moeExpertNum <= 512; H and I multiples of 128. */

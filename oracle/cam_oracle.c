@@ -382,6 +382,28 @@ ORACLE_API void cam_oracle_swiglu_quant(const float *d, int64_t M, int64_t I, in
 /* ---------------------------------------------------------------- A.9 GMM2 epilogue
  * FDM/epilogue/block/block_epilogue_per_token_dequant.hpp:665-684:
  *   out = bf16_rne((float(C2) * w2_scale[g][h]) * y_scale[m]). */
+static inline uint16_t f32_to_fp16(float f);
+static inline uint16_t f32_to_act(float f, int act) { return act ? f32_to_fp16(f) : f32_to_bf16(f); }
+
+/* act: 0 = bf16 rows, 1 = fp16 rows (the output takes the activation type of the layer's input,
+ * FDM/epilogue/block/block_epilogue_per_token_dequant.hpp:665-684 with ElementD = the token type). */
+ORACLE_API void cam_oracle_gmm2_epilogue_act(const int32_t *c, const float *w_scale, const float *y_scale,
+                                             const int64_t *group_list, int64_t G, int64_t H, int act,
+                                             uint16_t *out)
+{
+    for (int64_t g = 0; g < G; ++g) {
+        int64_t m0 = g == 0 ? 0 : group_list[g - 1];
+        int64_t m1 = group_list[g];
+        const float *ws = w_scale + g * H;
+#pragma omp parallel for schedule(static)
+        for (int64_t m = m0; m < m1; ++m) {
+            for (int64_t h = 0; h < H; ++h) {
+                out[m * H + h] = f32_to_act(((float)c[m * H + h] * ws[h]) * y_scale[m], act);
+            }
+        }
+    }
+}
+
 ORACLE_API void cam_oracle_gmm2_epilogue(const int32_t *c, const float *w_scale, const float *y_scale,
                                          const int64_t *group_list, int64_t G, int64_t H,
                                          uint16_t *out)
@@ -521,6 +543,32 @@ ORACLE_API void cam_oracle_comm_dequant_rows(const uint8_t *packed, int64_t A, i
         for (int64_t h = 0; h < H; ++h) {
             out[r * H + h] = f32_to_bf16((float)q[h] * bf16_to_f32(sc[h / CAM_COMMQ_BLOCK]));
         }
+    }
+}
+
+/* the same with rows and output in the activation type `act` (0 bf16, 1 fp16) */
+ORACLE_API void cam_oracle_combine_act(const uint16_t *y, const int32_t *row_of, const float *w, int64_t T,
+                                       int64_t K, int64_t H, int act, uint16_t *out)
+{
+#pragma omp parallel for schedule(static)
+    for (int64_t t = 0; t < T; ++t) {
+        float *acc = (float *)calloc((size_t)H, sizeof(float));
+        for (int64_t k = 0; k < K; ++k) {
+            int32_t row = row_of[t * K + k];
+            if (row < 0) {
+                continue;
+            }
+            float wk = w[t * K + k];
+            const uint16_t *yr = y + (int64_t)row * H;
+            for (int64_t h = 0; h < H; ++h) {
+                float p = act_to_f32(yr[h], act) * wk;
+                acc[h] = acc[h] + p;
+            }
+        }
+        for (int64_t h = 0; h < H; ++h) {
+            out[t * H + h] = f32_to_act(acc[h], act);
+        }
+        free(acc);
     }
 }
 

@@ -201,6 +201,47 @@ def gmm2_epilogue(c, w_scale, y_scale, group_list):
     return out
 
 
+def gmm2_epilogue_act(c, w_scale, y_scale, group_list, fp16):
+    c = _c(c, np.int32)
+    ws = _c(w_scale, np.float32)
+    ys = _c(y_scale, np.float32)
+    gl = _c(group_list, np.int64)
+    G, H = ws.shape
+    out = np.zeros((c.shape[0], H), np.uint16)
+    lib().cam_oracle_gmm2_epilogue_act(_p(c), _p(ws), _p(ys), _p(gl), _i64(G), _i64(H), ctypes.c_int(1 if fp16 else 0),
+                                       _p(out))
+    return out
+
+
+def combine_act(y_bits, row_of, w, fp16):
+    y_bits = _c(y_bits, np.uint16)
+    row_of = _c(row_of, np.int32)
+    w = _c(w, np.float32)
+    T, K = row_of.shape
+    H = y_bits.shape[1]
+    out = np.zeros((T, H), np.uint16)
+    lib().cam_oracle_combine_act(_p(y_bits), _p(row_of), _p(w), _i64(T), _i64(K), _i64(H),
+                                 ctypes.c_int(1 if fp16 else 0), _p(out))
+    return out
+
+
+def fused_layer_fp16(x_bits, idx, topk_w, w1, w1_scale, w2, w2_scale):
+    """The int8 layer with fp16 activations in and out, composed from the stage functions."""
+    idx = _c(idx, np.int64)
+    T, K = idx.shape
+    E = w1.shape[0]
+    _, cnt, _ = layout(idx, E, 1)
+    off, _ = offsets(cnt, T)
+    pos = send_token_idx(idx, E)
+    A = int(cnt.sum())
+    x1, x1s, _ = dispatch(x_bits, idx, off, pos, E, 2, max(A, 1), fp16=True)
+    gl = np.cumsum(cnt).astype(np.int64)
+    d = gmm1_epilogue(gmm_int32(x1, w1, gl), w1_scale, x1s, gl)
+    x2, x2s = swiglu_quant(d, rows=A)
+    y = gmm2_epilogue_act(gmm_int32(x2, w2, gl), w2_scale, x2s, gl, True)
+    return combine_act(y, rows_from_pos(idx, off, pos, E), topk_w, True), cnt
+
+
 def rows_from_pos(idx, off, pos, E):
     idx = _c(idx, np.int64)
     off = _c(off, np.int32)

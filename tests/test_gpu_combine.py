@@ -187,3 +187,18 @@ def test_prefill_with_worst_case_rows_then_combine(gpu, oracle):
     want_x, _, want_src = oracle.dispatch(synth.bf16_bits(x.cpu()), ids.numpy(), off, pos, E, 0, total)
     want = oracle.combine(want_x, oracle.rows_from_src_info(want_src, total, T, K), w.numpy())
     assert_bits_equal(to_np(comb), want, "combined x")
+
+
+def test_combine_fp16_rows_bit_exact(gpu, oracle):
+    """fp16 rows in, fp16 out (moe_combine_normal.cpp(op_host):18,49 lists bf16 and fp16)."""
+    announce("combine fp16 rows")
+    T, K, E, H = 45, 4, 16, 2048
+    ids, w = synth.sigmoid_zipf_routing(T, E, K, seed=61)
+    idx_np = ids.numpy()
+    cnt, off, pos, _ = plan_oracle(oracle, idx_np, E)
+    y = (torch.randn(T * K, H, generator=torch.Generator().manual_seed(62)) * 3).half()
+    row_of = oracle.rows_from_pos(idx_np, off, pos, E)
+    want = oracle.combine_act(y.view(torch.int16).numpy().view(np.uint16), row_of, w.numpy(), True)
+    got = cam.moe_combine_gather(y.to(gpu), None, torch.from_numpy(row_of.reshape(T, K)).to(gpu), w.to(gpu))
+    assert got.dtype == torch.float16
+    assert_bits_equal(got.cpu().view(torch.int16).numpy().view(np.uint16), want, "combined fp16 x")

@@ -95,3 +95,22 @@ def test_fused_negative_ids_and_skew(gpu, oracle):
     d = dict(x=synth.normal_bf16(T, H, seed=83), ids=ids, gates=gates, w1=w1, w1_scale=w1s, w2=w2, w2_scale=w2s)
     out, etn = _run(gpu, d)
     assert _check(oracle, d, out, etn) == 0
+
+
+def test_fused_layer_fp16_activations(gpu, oracle):
+    """fp16 tokens in, fp16 out (the reference lists both 16-bit types,
+    fused_deep_moe.cpp(op_host):22-24): quantisation reads fp16, GMM2 and the combine write fp16."""
+    announce("fused layer, fp16 activations")
+    T, H, E, K, I = 96, 1024, 8, 2, 512
+    ids, gates = synth.softmax_topk_routing(T, E, K, seed=51)
+    w1, w1s = synth.absmax_int8_weights(E, H, 2 * I, seed=511)
+    w2, w2s = synth.absmax_int8_weights(E, I, H, seed=512)
+    x = torch.randn(T, H, generator=torch.Generator().manual_seed(513)).half()
+    out, etn = cam.fused_deep_moe(x.to(gpu), ids.to(torch.int32).to(gpu), [cam.prepack_weight(w1.to(gpu), True)],
+                                  [w1s.to(gpu)], [cam.prepack_weight(w2.to(gpu), False)], [w2s.to(gpu)],
+                                  gates.to(gpu), None, None, "", 1, 0, E, 1, 0, 0, 0)
+    assert out.dtype == torch.float16
+    want, cnt = oracle.fused_layer_fp16(x.view(torch.int16).numpy().view(np.uint16), ids.numpy(), gates.numpy(),
+                                        w1.numpy(), w1s.numpy(), w2.numpy(), w2s.numpy())
+    assert_bits_equal(to_np(etn), cnt.astype(np.int64), "expert_token_nums")
+    assert_bits_equal(out.cpu().view(torch.int16).numpy().view(np.uint16), want, "fp16 layer output")

@@ -220,3 +220,18 @@ def test_many_tiles_per_expert_epilogues(gpu, oracle):
     c2 = oracle.gmm_int32(want_q, w2.numpy(), gl.numpy())
     want = oracle.gmm2_epilogue(c2, w2s.numpy(), want_s, gl.numpy())
     assert_bits_equal(to_np(out), want, "bf16 output")
+
+
+def test_gmm2_fp16_output_bit_exact(gpu, oracle):
+    """GroupedMatmulDequant writing IEEE fp16 (the layer's activation type when the tokens are fp16)."""
+    announce("gmm2 fp16 output")
+    sizes, I, H = [140, 0, 33], 512, 1024
+    a, w, gl, A = _inputs(sizes, I, H, seed=91, wrange=16)
+    ws = synth.channel_scales((len(sizes), H), seed=92)
+    xs = synth.channel_scales((A,), seed=93, lo=0.001, hi=0.01)
+    out = cam.grouped_matmul_dequant(a.to(gpu), xs.to(gpu), cam.prepack_weight(w.to(gpu), False), ws.to(gpu), gl.to(gpu),
+                                     out_dtype=torch.float16)
+    c = oracle.gmm_int32(a.numpy(), w.numpy(), gl.numpy())
+    want = oracle.gmm2_epilogue_act(c, ws.numpy(), xs.numpy(), gl.numpy(), True)
+    assert out.dtype == torch.float16
+    assert_bits_equal(out.cpu().view(torch.int16).numpy().view(np.uint16)[:A], want[:A], "fp16 output")

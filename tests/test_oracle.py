@@ -662,3 +662,28 @@ def test_fp8_gemm_against_float64_and_swiglu(oracle):
     c64 = c.astype(np.float32).astype(np.float64)
     ref = c64[:, :32] / (1 + np.exp(-c64[:, :32])) * c64[:, 32:]
     assert np.allclose(y, ref, rtol=3e-6, atol=1e-7)
+
+
+def test_fp16_activation_variants_of_gmm2_epilogue_and_combine(oracle):
+    """The fp16 forms differ from the bf16 ones only in the 16-bit conversions, which numpy's float16 pins."""
+    g = torch.Generator().manual_seed(31)
+    c = torch.randint(-200000, 200000, (6, 128), generator=g, dtype=torch.int32).numpy()
+    ws = (torch.rand(2, 128, generator=g) * 1e-3).numpy()
+    ys = (torch.rand(6, generator=g) * 1e-2).numpy()
+    gl = np.array([4, 6], np.int64)
+    got = oracle.gmm2_epilogue_act(c, ws, ys, gl, True)
+    grp = np.array([0, 0, 0, 0, 1, 1])
+    want = ((c.astype(np.float32) * ws[grp]) * ys[:, None]).astype(np.float16).view(np.uint16)
+    assert np.array_equal(got, want)
+    assert np.array_equal(oracle.gmm2_epilogue_act(c, ws, ys, gl, False), oracle.gmm2_epilogue(c, ws, ys, gl))
+    y = (torch.randn(8, 64, generator=g) * 2).half()
+    row_of = np.array([[0, 3], [5, -1], [7, 2]], np.int32)
+    w = np.array([[0.25, 0.5], [1.0, 9.0], [0.3, 0.7]], np.float32)
+    got = oracle.combine_act(y.view(torch.int16).numpy().view(np.uint16), row_of, w, True)
+    yf = y.float().numpy()
+    acc = np.zeros((3, 64), np.float32)
+    for t in range(3):
+        for k in range(2):
+            if row_of[t, k] >= 0:
+                acc[t] = acc[t] + (yf[row_of[t, k]] * w[t, k]).astype(np.float32)
+    assert np.array_equal(got, acc.astype(np.float16).view(np.uint16))

@@ -930,11 +930,12 @@ camStatus camMoeCombineNormalGetWorkspaceSize(const camTensor *recvX, const camT
     (void)epGroupName;
     (void)tpGroupNameOptional;
     (void)tpRankId;
-    CAM_TRY(check_tensor(recvX, "recvX", 2, CAM_DT_BF16));
+    // bf16 or fp16 rows (AK/moe_combine_normal/op_host/moe_combine_normal.cpp:18,49); out has the same type
+    CAM_TRY(check_tensor(recvX, "recvX", 2, CAM_DT_BF16, CAM_DT_FLOAT16));
     CAM_TRY(check_tensor(tokenSrcInfo, "tokenSrcInfo", 1, CAM_DT_INT32));
     CAM_TRY(check_tensor(epRecvCounts, "epRecvCounts", 1, CAM_DT_INT32));
     CAM_TRY(check_tensor(recvTopkWeights, "recvTopkWeights", 2, CAM_DT_FLOAT));
-    CAM_TRY(check_tensor(out, "out", 2, CAM_DT_BF16));
+    CAM_TRY(check_tensor(out, "out", 2, recvX->dtype));
     if (epWorldSize <= 0 || epWorldSize > cam::kMaxRanks) {
         return fail(CAM_ERR_RANGE, "epWorldSize %lld outside (0, %d]", (long long)epWorldSize, cam::kMaxRanks);
     }
@@ -991,6 +992,7 @@ camStatus camMoeCombineNormalGetWorkspaceSize(const camTensor *recvX, const camT
     g.K = (int)K;
     g.H = (int)H;
     g.A = A;
+    g.act_fp16 = recvX->dtype == CAM_DT_FLOAT16;
     // Rows at or past the receive total were never written (moe_combine_normal.h:206-207 bounds its loop the same way).
     g.row_limit = (const int32_t *)epRecvCounts->data + (moeExpertNum - 1);
     g.out = (uint16_t *)out->data;
@@ -1045,11 +1047,11 @@ camStatus camMoeCombineGatherGetWorkspaceSize(const camTensor *recvX, const camT
 {
     // recvX: bf16 rows [A,H], or rows quantised for the wire, int8 [A, H + H/4] (the int8 communication
     // quantisation of AK/moe_combine_shmem/op_kernel/moe_combine_shmem.h:564-592, dequantised as :755-773).
-    CAM_TRY(check_tensor(recvX, "recvX", 2, CAM_DT_BF16, CAM_DT_INT8));
+    CAM_TRY(check_tensor(recvX, "recvX", 2, CAM_DT_BF16, CAM_DT_FLOAT16, CAM_DT_INT8));
     CAM_TRY(check_tensor(slotRow, "slotRow", 2, CAM_DT_INT32));
     CAM_TRY(check_tensor(recvTopkWeights, "recvTopkWeights", 2, CAM_DT_FLOAT));
-    CAM_TRY(check_tensor(out, "out", 2, CAM_DT_BF16));
     const bool wire = recvX->dtype == CAM_DT_INT8;
+    CAM_TRY(check_tensor(out, "out", 2, wire ? CAM_DT_BF16 : recvX->dtype));
     const int64_t A = recvX->sizes[0], H = out->sizes[1];
     const int64_t T = recvTopkWeights->sizes[0], K = recvTopkWeights->sizes[1];
     if (recvX->sizes[1] != (wire ? H + H / 4 : H)) {
@@ -1100,6 +1102,7 @@ camStatus camMoeCombineGatherGetWorkspaceSize(const camTensor *recvX, const camT
     g.H = (int)H;
     g.A = A;
     g.wire_rows = wire ? 1 : 0;
+    g.act_fp16 = recvX->dtype == CAM_DT_FLOAT16;
     g.out = (uint16_t *)out->data;
     auto run = [g](void *, hipStream_t s) -> hipError_t { return cam::launch_combine(g, s); };
     return finish_phase1(kOpCombGather, 0, run, workspaceSize, executor);
@@ -1270,7 +1273,7 @@ camStatus camGroupedMatmulDequantGetWorkspaceSize(const camTensor *x, const camT
     CAM_TRY(check_gemm_inputs("GroupedMatmulDequant", x, xScale, true, groupList, groupListType, &gc));
     // out: bf16 [A,N], or int8 [A, N + N/4]: the bf16 rows quantised for the wire on their way out (blocks of 8
     // columns, AK/moe_combine_shmem/op_kernel/moe_combine_shmem.h:564-592), which MoeCombineGather reads back.
-    CAM_TRY(check_tensor(out, "out", 2, CAM_DT_BF16, CAM_DT_INT8));
+    CAM_TRY(check_tensor(out, "out", 2, CAM_DT_BF16, CAM_DT_FLOAT16, CAM_DT_INT8));
     const bool wire = out->dtype == CAM_DT_INT8;
     if (wire && out->sizes[1] % 10 != 0) {
         return fail(CAM_ERR_SHAPE, "int8 out must be [A, N + N/4] with N a multiple of 8");
@@ -1299,6 +1302,7 @@ camStatus camGroupedMatmulDequantGetWorkspaceSize(const camTensor *x, const camT
     g.gate_up = 0;
     g.epilogue = cam::kEpiDequantBf16;
     g.out = out->data;
+    g.out_fp16 = out->dtype == CAM_DT_FLOAT16;
     uint8_t *wire_out = (uint8_t *)out->data;
     auto run = [=](void *wsp, hipStream_t s) mutable -> hipError_t {
         sp.sched = (int32_t *)((char *)wsp + o_sched);
@@ -1420,9 +1424,6 @@ camStatus camFusedDeepMoeGetWorkspaceSize(const camTensor *x, const camTensor *e
         return fail(CAM_ERR_UNSUPPORTED, "FusedDeepMoe: epRankSize must be 1 and sharedExpertRankNum 0 "
                                          "(single-GPU library)");
     }
-    if (x->dtype != CAM_DT_BF16) {
-        return fail(CAM_ERR_UNSUPPORTED, "FusedDeepMoe: float16 activations are not built");
-    }
     if (expertSmoothScalesOptional != nullptr) {
         return fail(CAM_ERR_UNSUPPORTED, "expertSmoothScales is accepted by the reference but never used; pass NULL");
     }
@@ -1474,7 +1475,7 @@ camStatus camFusedDeepMoeGetWorkspaceSize(const camTensor *x, const camTensor *e
             return fail(CAM_ERR_SHAPE, "xActiveMask must be [bs]");
         }
     }
-    CAM_TRY(check_tensor(output, "output", 2, CAM_DT_BF16));
+    CAM_TRY(check_tensor(output, "output", 2, x->dtype));  // the layer's output has the type of its input
     if (output->sizes[0] != T || output->sizes[1] != H) {
         return fail(CAM_ERR_SHAPE, "output must be [bs, H]");
     }
@@ -1511,6 +1512,7 @@ camStatus camFusedDeepMoeGetWorkspaceSize(const camTensor *x, const camTensor *e
     const uint64_t o_x2s = c.take((uint64_t)A * 4);
 
     const uint16_t *xp = (const uint16_t *)x->data;
+    const int x_is_fp16 = x->dtype == CAM_DT_FLOAT16;
     const int32_t *ids = (const int32_t *)expertIds->data;
     const float *gates = (const float *)expertScales->data;
     const uint8_t *mask = xActiveMaskOptional ? (const uint8_t *)xActiveMaskOptional->data : nullptr;
@@ -1548,6 +1550,7 @@ camStatus camFusedDeepMoeGetWorkspaceSize(const camTensor *x, const camTensor *e
             cam::FusedDispatchArgs f{};
             f.p = p;
             f.x = xp;
+            f.x_is_fp16 = x_is_fp16;
             f.H = iH;
             f.A = A;
             f.quant = 2;
@@ -1561,6 +1564,7 @@ camStatus camFusedDeepMoeGetWorkspaceSize(const camTensor *x, const camTensor *e
             if (e != hipSuccess) return e;
             cam::DispatchArgs d{};
             d.x = xp;
+            d.x_is_fp16 = x_is_fp16;
             d.idx = ids;
             d.dst_row = row;
             d.T = iT;
@@ -1613,6 +1617,7 @@ camStatus camFusedDeepMoeGetWorkspaceSize(const camTensor *x, const camTensor *e
         g2.gate_up = 0;
         g2.epilogue = cam::kEpiDequantBf16;
         g2.out = y;
+        g2.out_fp16 = x_is_fp16;
         e = cam::launch_gemm(g2, s);
         if (e != hipSuccess) return e;
 
@@ -1625,6 +1630,7 @@ camStatus camFusedDeepMoeGetWorkspaceSize(const camTensor *x, const camTensor *e
         cb.H = iH;
         cb.A = A;
         cb.t_active = meta + 2;
+        cb.act_fp16 = x_is_fp16;
         cb.out = outp;
         return cam::launch_combine(cb, s);
     };

@@ -32,6 +32,17 @@ __device__ __forceinline__ uint32_t f32_to_bf16_bits(float f)
     return (u & 0x7fffffffu) > 0x7f800000u ? quiet : rounded;  // both sides computed: a select, no branch
 }
 
+// Round-to-nearest-even fp32 -> IEEE fp16 bit pattern (the hardware conversion; overflow gives infinity).
+__device__ __forceinline__ uint32_t f32_to_fp16_bits(float f)
+{
+    return (uint32_t)__builtin_bit_cast(unsigned short, (_Float16)f);
+}
+
+__device__ __forceinline__ float fp16_bits_to_f32(uint32_t bits16)
+{
+    return (float)__builtin_bit_cast(_Float16, (unsigned short)bits16);  // exact
+}
+
 __device__ __forceinline__ int lane_id()
 {
     return (int)__builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u));

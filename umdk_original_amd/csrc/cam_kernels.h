@@ -134,6 +134,7 @@ hipError_t launch_invert_src_info(const int32_t *src_info, int64_t A, const int3
 struct CombineArgs {
     const uint16_t *y;        // [A,H] bf16 bits, or wire rows [A, H + H/4] bytes (wire_rows != 0)
     int wire_rows;            // rows are H int8 values + H/8 bf16 block scales (launch_comm_quant's output)
+    int act_fp16;             // rows and output are IEEE fp16 instead of bf16 (not with wire_rows)
     const int32_t *slot_row;  // [T,K] row of slot (t,k) (<0: skip)
     const int32_t *src_info;  // optional: when set, slot_row entries are verified against the triples
     const float *w;           // [T,K]
@@ -175,6 +176,7 @@ struct GemmArgs {
     int gate_up;           // weight prepacked with gate/up pairing
     int epilogue;
     void *out;             // int32 [A,N] | fp32 [A,N/2] | bf16 bits [A,N]
+    int out_fp16;          // kEpiDequantBf16 writes IEEE fp16 instead of bf16
 };
 hipError_t launch_gemm(const GemmArgs &a, hipStream_t stream);
 

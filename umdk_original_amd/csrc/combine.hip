@@ -88,7 +88,14 @@ __global__ __launch_bounds__(256) void comm_quant_kernel(const uint16_t *__restr
     *(uint16_t *)(dst + H + b * 2) = sbits;
 }
 
-template <bool WIRE>
+// ACT: 0 = bf16 rows and output, 1 = IEEE fp16 (the layer's activation type).
+template <int ACT>
+__device__ __forceinline__ float comb_act_to_f32(uint32_t bits16)
+{
+    return ACT == 0 ? bf16_bits_to_f32(bits16) : fp16_bits_to_f32(bits16);
+}
+
+template <bool WIRE, int ACT>
 __global__ __launch_bounds__(kCombThreads) void combine_kernel(CombineArgs a, int segs)
 {
     const int t = blockIdx.x / segs;
@@ -150,8 +157,8 @@ __global__ __launch_bounds__(kCombThreads) void combine_kernel(CombineArgs a, in
                 } else if (ok[j]) {
 #pragma unroll
                     for (int c = 0; c < 4; ++c) {
-                        float x0 = bf16_bits_to_f32(v[j][c] & 0xffffu);
-                        float x1 = bf16_bits_to_f32(v[j][c] >> 16);
+                        float x0 = comb_act_to_f32<ACT>(v[j][c] & 0xffffu);
+                        float x1 = comb_act_to_f32<ACT>(v[j][c] >> 16);
                         acc[2 * c] = __fadd_rn(acc[2 * c], __fmul_rn(x0, w[j]));
                         acc[2 * c + 1] = __fadd_rn(acc[2 * c + 1], __fmul_rn(x1, w[j]));
                     }
@@ -162,7 +169,8 @@ __global__ __launch_bounds__(kCombThreads) void combine_kernel(CombineArgs a, in
     v4u o;
 #pragma unroll
     for (int c = 0; c < 4; ++c) {
-        o[c] = f32_to_bf16_bits(acc[2 * c]) | (f32_to_bf16_bits(acc[2 * c + 1]) << 16);
+        o[c] = ACT == 0 ? f32_to_bf16_bits(acc[2 * c]) | (f32_to_bf16_bits(acc[2 * c + 1]) << 16)
+                        : f32_to_fp16_bits(acc[2 * c]) | (f32_to_fp16_bits(acc[2 * c + 1]) << 16);
     }
     __builtin_nontemporal_store(o, (v4u *)(a.out + (long long)t * a.H + col));
 }
@@ -288,7 +296,7 @@ hipError_t launch_combine(const CombineArgs &a, hipStream_t stream)
     if (a.T <= 0) {
         return hipSuccess;
     }
-    if (a.H % 8 != 0) {
+    if (a.H % 8 != 0 || (a.wire_rows && a.act_fp16)) {
         return hipErrorInvalidValue;
     }
     const int segs = (a.H / 8 + kCombThreads - 1) / kCombThreads;
@@ -301,9 +309,11 @@ hipError_t launch_combine(const CombineArgs &a, hipStream_t stream)
         hipLaunchKernelGGL(combine_wire16_kernel, dim3((unsigned)(a.T * segs16)), dim3(kCombThreads), 0, stream, a,
                            segs16);
     } else if (a.wire_rows) {
-        hipLaunchKernelGGL(combine_kernel<true>, dim3((unsigned)blocks), dim3(kCombThreads), 0, stream, a, segs);
+        hipLaunchKernelGGL((combine_kernel<true, 0>), dim3((unsigned)blocks), dim3(kCombThreads), 0, stream, a, segs);
+    } else if (a.act_fp16) {
+        hipLaunchKernelGGL((combine_kernel<false, 1>), dim3((unsigned)blocks), dim3(kCombThreads), 0, stream, a, segs);
     } else {
-        hipLaunchKernelGGL(combine_kernel<false>, dim3((unsigned)blocks), dim3(kCombThreads), 0, stream, a, segs);
+        hipLaunchKernelGGL((combine_kernel<false, 0>), dim3((unsigned)blocks), dim3(kCombThreads), 0, stream, a, segs);
     }
     return hipGetLastError();
 }

@@ -411,12 +411,13 @@ __device__ __forceinline__ void run_item(const GemmArgs &a, const ItemCtx &t, in
                         uint32_t b[4];
 #pragma unroll
                         for (int e = 0; e < 4; ++e) {
+                            float v;
                             if constexpr (FP8) {
-                                b[e] = f32_to_bf16_bits(acc[mf][nf][4 * j + e]);
+                                v = acc[mf][nf][4 * j + e];
                             } else {
-                                b[e] = f32_to_bf16_bits(
-                                    __fmul_rn(__fmul_rn((float)acc[mf][nf][4 * j + e], ws[nf][j][e]), xs));
+                                v = __fmul_rn(__fmul_rn((float)acc[mf][nf][4 * j + e], ws[nf][j][e]), xs);
                             }
+                            b[e] = a.out_fp16 ? f32_to_fp16_bits(v) : f32_to_bf16_bits(v);
                         }
                         const v2u v = {b[0] | (b[1] << 16), b[2] | (b[3] << 16)};
                         *(v2u *)(slice + row_in * kEpiRowBytes + (nf * 32 + 8 * j + col_half) * 2) = v;

@@ -233,7 +233,8 @@ def moe_combine_gather(recv_x, token_src_info, slot_row, topk_weights, out=None,
     if out is None:
         # int8 rows are wire rows [A, H + H/4] (grouped_matmul_dequant(..., wire_rows=True))
         h = recv_x.size(1) // 5 * 4 if recv_x.dtype == torch.int8 else recv_x.size(1)
-        out = torch.empty((topk_weights.size(0), h), dtype=torch.bfloat16, device=recv_x.device)
+        out = torch.empty((topk_weights.size(0), h),
+                          dtype=torch.bfloat16 if recv_x.dtype == torch.int8 else recv_x.dtype, device=recv_x.device)
     _lib.call("MoeCombineGather", [recv_x, token_src_info, slot_row, ep_recv_counts, topk_weights, out])
     return out
 
@@ -282,7 +283,8 @@ def grouped_matmul_swiglu_quant(x, x_scale, weight, weight_scale, group_list, gr
     return y, ys
 
 
-def grouped_matmul_dequant(x, x_scale, weight, weight_scale, group_list, group_list_type=0, wire_rows=False):
+def grouped_matmul_dequant(x, x_scale, weight, weight_scale, group_list, group_list_type=0, wire_rows=False,
+                           out_dtype=torch.bfloat16):
     """GMM2 stage: int8 [A,I] -> bf16 [A,H]; wire_rows=True: -> int8 [A, H + H/4], the bf16 rows quantised for
     the wire (8-column blocks: int8 values, then bf16 block scales), which moe_combine_gather reads back."""
     weight = _tag_list(weight if isinstance(weight, (list, tuple)) else [weight])
@@ -291,7 +293,7 @@ def grouped_matmul_dequant(x, x_scale, weight, weight_scale, group_list, group_l
     if wire_rows:
         out = torch.empty((x.size(0), n + n // 4), dtype=torch.int8, device=x.device)
     else:
-        out = torch.empty((x.size(0), n), dtype=torch.bfloat16, device=x.device)
+        out = torch.empty((x.size(0), n), dtype=out_dtype, device=x.device)
     _lib.call("GroupedMatmulDequant", [x, x_scale, weight, weight_scale, group_list, group_list_type, out])
     return out
 
