@@ -1495,7 +1495,9 @@ camStatus camFusedDeepMoeGetWorkspaceSize(const camTensor *x, const camTensor *e
     const uint64_t o_meta = c.take(cam::kPlanMeta * 4);
     const uint64_t o_sched1 = c.take(cam::sched_bytes(A, (int)Epr, (int)(2 * I)));
     const uint64_t o_sched2 = c.take(cam::sched_bytes(A, (int)Epr, (int)H));
-    const bool fused_dispatch = cam::fused_dispatch_fits(T, K);
+    // one launch for plan + permute pays from about 16384 routed rows on; below that its hand-overs between
+    // workgroups take longer than the two extra launches of the plan (12.0 against 9.2 us at 128 tokens, top-2)
+    const bool fused_dispatch = cam::fused_dispatch_fits(T, K) && T * K >= 16384;
     const uint64_t o_hist = c.take(fused_dispatch ? cam::fused_dispatch_table_bytes(T, K, (int)Epr)
                                                   : cam::plan_workspace_bytes(T, K, (int)Epr));
     const uint64_t o_ctrl = c.take(cam::fused_dispatch_ctrl_bytes());
@@ -1849,7 +1851,9 @@ camStatus camFusedDeepMoeFp8GetWorkspaceSize(const camTensor *x, const camTensor
     const uint64_t o_meta = c.take(cam::kPlanMeta * 4);
     const uint64_t o_sched1 = c.take(cam::sched_bytes(A, (int)E, (int)(2 * I)));
     const uint64_t o_sched2 = c.take(cam::sched_bytes(A, (int)E, (int)H));
-    const bool fused_dispatch = cam::fused_dispatch_fits(T, K);
+    // one launch for plan + permute pays from about 16384 routed rows on; below that its hand-overs between
+    // workgroups take longer than the two extra launches of the plan (12.0 against 9.2 us at 128 tokens, top-2)
+    const bool fused_dispatch = cam::fused_dispatch_fits(T, K) && T * K >= 16384;
     const uint64_t o_hist = c.take(fused_dispatch ? cam::fused_dispatch_table_bytes(T, K, (int)E)
                                                   : cam::plan_workspace_bytes(T, K, (int)E));
     const uint64_t o_ctrl = c.take(cam::fused_dispatch_ctrl_bytes());
