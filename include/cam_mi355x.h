@@ -96,6 +96,17 @@ CAM_API const char *camGetRecentErrMsg(void);
 CAM_API camStatus camDestroyExecutor(camOpExecutor *executor);
 CAM_API const char *camGetVersion(void);
 
+/* How MoeDispatchPrefill and the fused layers launch the plan + permute of the dispatch (no counterpart in the
+ * reference; the results are identical in every mode).  CAM_DISPATCH_LAUNCH_AUTO (default): one launch where it
+ * is measured not to be slower than three -- 32768 <= T*K <= 524288 and T <= 4096 -- and MoeDispatchPlan's two
+ * launches followed by MoeDispatchNormal's otherwise.  CAM_DISPATCH_LAUNCH_SINGLE: one launch whenever
+ * T*K <= 524288.  CAM_DISPATCH_LAUNCH_SEPARATE: never one launch.  The setting is process-wide and read by
+ * phase 1 of those operators; returns CAM_ERR_RANGE for another value. */
+#define CAM_DISPATCH_LAUNCH_AUTO 0
+#define CAM_DISPATCH_LAUNCH_SINGLE 1
+#define CAM_DISPATCH_LAUNCH_SEPARATE 2
+CAM_API camStatus camSetDispatchLaunchMode(int32_t mode);
+
 /* ------------------------------------------------------------------------------------------------
  * DispatchLayout -- replaces aclnnDispatchLayout (AUTOGEN/aclnn_dispatch_layout.h:32-54).
  * topkIdx int64 [T,K] (int32 also accepted) -> numTokensPerRank int32 [R], numTokensPerExpert
@@ -212,8 +223,8 @@ CAM_API camStatus camMoeDispatchNormal(void *workspace, uint64_t workspaceSize, 
  * all exactly as MoeDispatchPlan / MoeDispatchNormal produce them.  Rows outside [0,A) are dropped, so A
  * may be a worst-case bound (T*K) and the true total read later from totalRecvTokens.
  * The workspace may hold anything on first use; a launch leaves it ready for the next one.  Launches
- * that share a workspace must not overlap.  Up to 524288 (token, k) entries take the single launch; above
- * that the operator falls back to the two launches of MoeDispatchPlan + MoeDispatchNormal. */
+ * that share a workspace must not overlap.  Whether the single launch or MoeDispatchPlan's and
+ * MoeDispatchNormal's launches run is decided by camSetDispatchLaunchMode (same results either way). */
 CAM_API camStatus camMoeDispatchPrefillGetWorkspaceSize(
     const camTensor *x, const camTensor *topkIdx, int64_t numExperts, int64_t numRanks, int64_t rankId,
     int64_t quantMode, const camTensor *recvX, const camTensor *recvXScalesOptional, const camTensor *expandIdx,

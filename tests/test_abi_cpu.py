@@ -341,3 +341,12 @@ def test_fp8_operator_validation():
     pre = _prefill_args()
     pre[5] = 4
     assert _lib.phase1("MoeDispatchPrefill", pre)[0] != CAM_OK          # int8 rows / fp32 scales do not fit
+
+
+def test_dispatch_launch_mode_setter_range():
+    from umdk_original_amd import _lib
+    h = _lib.lib()
+    for mode in (1, 2, 0):
+        assert h.camSetDispatchLaunchMode(mode) == 0
+    assert h.camSetDispatchLaunchMode(3) != 0 and "mode" in _lib.recent_error()
+    assert h.camSetDispatchLaunchMode(-1) != 0

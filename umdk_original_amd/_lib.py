@@ -115,7 +115,7 @@ DIRECT_SIGNATURES = {
     "MoeDispatchPlanNoAlloc": [_TP, _I64, _I64, _I64, _TP, _TP, _TP, _TP, _TP, _TP, _TP, _TP],
 }
 
-EXPORTS = ["camGetRecentErrMsg", "camDestroyExecutor", "camGetVersion"] + [
+EXPORTS = ["camGetRecentErrMsg", "camDestroyExecutor", "camGetVersion", "camSetDispatchLaunchMode"] + [
     "cam%s" % op for op in DIRECT_SIGNATURES] + [
     "cam%s%s" % (op, suffix) for op in SIGNATURES for suffix in ("GetWorkspaceSize", "")
 ]
@@ -135,6 +135,8 @@ def lib():
         handle.camGetRecentErrMsg.restype = ctypes.c_char_p
         handle.camGetVersion.restype = ctypes.c_char_p
         handle.camDestroyExecutor.argtypes = [ctypes.c_void_p]
+        handle.camSetDispatchLaunchMode.argtypes = [ctypes.c_int32]
+        handle.camSetDispatchLaunchMode.restype = ctypes.c_int32
         for op, argtypes in SIGNATURES.items():
             f1 = getattr(handle, "cam%sGetWorkspaceSize" % op)
             f1.argtypes = argtypes + _PHASE1_TAIL

@@ -9,6 +9,7 @@
 //   AK/fused_deep_moe/op_host/fused_deep_moe_tiling.cpp:49-61,83-348
 //   src/cam/comm_operator/pybind/moe_dispatch_prefill.cpp:44-70
 #include <algorithm>
+#include <atomic>
 #include <cstdarg>
 #include <cstdio>
 #include <cstring>
@@ -296,11 +297,42 @@ cam::SchedSpec sched_spec(int64_t rows, int64_t G, int64_t N)
     return sp;
 }
 
+std::atomic<int32_t> g_dispatch_launch_mode{CAM_DISPATCH_LAUNCH_AUTO};
+
+// One launch for plan + permute, or the plan's two launches and then the permute's.  Measured (int8 rows,
+// 256 experts, top-8, microseconds single / separate): 2048 x 7168: 40.1 / 34.1, 4096 x 4096: 40.0 / 41.2,
+// 4096 x 7168: 62.3 / 62.7, 8192 x 4096: 106.7 / 79.6, 8192 x 7168: 131.9 / 129.0; 128 tokens top-2: 12.0 / 9.2.
+// Below 32768 entries the hand-overs between workgroups cost more than two launches; above 4096 tokens the
+// workgroups beyond the first resident batch gain nothing from running under the plan.
+bool single_launch_dispatch(int64_t T, int64_t K)
+{
+    if (!cam::fused_dispatch_fits(T, K)) {
+        return false;
+    }
+    const int32_t mode = g_dispatch_launch_mode.load(std::memory_order_relaxed);
+    if (mode == CAM_DISPATCH_LAUNCH_SINGLE) {
+        return true;
+    }
+    if (mode == CAM_DISPATCH_LAUNCH_SEPARATE) {
+        return false;
+    }
+    return T * K >= 32768 && T <= 4096;
+}
+
 }  // namespace
 
 extern "C" {
 
 const char *camGetRecentErrMsg(void) { return g_err.c_str(); }
+
+camStatus camSetDispatchLaunchMode(int32_t mode)
+{
+    if (mode < CAM_DISPATCH_LAUNCH_AUTO || mode > CAM_DISPATCH_LAUNCH_SEPARATE) {
+        return fail(CAM_ERR_RANGE, "camSetDispatchLaunchMode: mode must be 0 (auto), 1 (single) or 2 (separate)");
+    }
+    g_dispatch_launch_mode.store(mode, std::memory_order_relaxed);
+    return CAM_OK;
+}
 
 const char *camGetVersion(void) { return "cam-mi355x 0.1 (gfx950)"; }
 
@@ -869,7 +901,7 @@ camStatus camMoeDispatchPrefillGetWorkspaceSize(const camTensor *x, const camTen
     f.src_info = (int32_t *)expandIdx->data;
     f.src_rank = (int)rankId;
     Carver c;
-    if (cam::fused_dispatch_fits(T, K)) {
+    if (single_launch_dispatch(T, K)) {
         const uint64_t o_ctrl = c.take(cam::fused_dispatch_ctrl_bytes());
         const uint64_t o_table = c.take(cam::fused_dispatch_table_bytes(T, K, (int)numExperts));
         auto run = [f, o_ctrl, o_table](void *ws, hipStream_t s) mutable -> hipError_t {
@@ -879,7 +911,7 @@ camStatus camMoeDispatchPrefillGetWorkspaceSize(const camTensor *x, const camTen
         };
         return finish_phase1(kOpPrefill, c.off, run, workspaceSize, executor);
     }
-    // More ids than the single launch is built for: the plan and the permute as separate launches.
+    // The plan and the permute as separate launches.
     const uint64_t o_hist = c.take(cam::plan_workspace_bytes(T, K, (int)numExperts));
     const uint64_t o_row = c.take((uint64_t)T * K * 4);
     auto run = [f, o_hist, o_row](void *ws, hipStream_t s) mutable -> hipError_t {
@@ -1495,9 +1527,7 @@ camStatus camFusedDeepMoeGetWorkspaceSize(const camTensor *x, const camTensor *e
     const uint64_t o_meta = c.take(cam::kPlanMeta * 4);
     const uint64_t o_sched1 = c.take(cam::sched_bytes(A, (int)Epr, (int)(2 * I)));
     const uint64_t o_sched2 = c.take(cam::sched_bytes(A, (int)Epr, (int)H));
-    // one launch for plan + permute pays from about 16384 routed rows on; below that its hand-overs between
-    // workgroups take longer than the two extra launches of the plan (12.0 against 9.2 us at 128 tokens, top-2)
-    const bool fused_dispatch = cam::fused_dispatch_fits(T, K) && T * K >= 16384;
+    const bool fused_dispatch = single_launch_dispatch(T, K);
     const uint64_t o_hist = c.take(fused_dispatch ? cam::fused_dispatch_table_bytes(T, K, (int)Epr)
                                                   : cam::plan_workspace_bytes(T, K, (int)Epr));
     const uint64_t o_ctrl = c.take(cam::fused_dispatch_ctrl_bytes());
@@ -1851,9 +1881,7 @@ camStatus camFusedDeepMoeFp8GetWorkspaceSize(const camTensor *x, const camTensor
     const uint64_t o_meta = c.take(cam::kPlanMeta * 4);
     const uint64_t o_sched1 = c.take(cam::sched_bytes(A, (int)E, (int)(2 * I)));
     const uint64_t o_sched2 = c.take(cam::sched_bytes(A, (int)E, (int)H));
-    // one launch for plan + permute pays from about 16384 routed rows on; below that its hand-overs between
-    // workgroups take longer than the two extra launches of the plan (12.0 against 9.2 us at 128 tokens, top-2)
-    const bool fused_dispatch = cam::fused_dispatch_fits(T, K) && T * K >= 16384;
+    const bool fused_dispatch = single_launch_dispatch(T, K);
     const uint64_t o_hist = c.take(fused_dispatch ? cam::fused_dispatch_table_bytes(T, K, (int)E)
                                                   : cam::plan_workspace_bytes(T, K, (int)E));
     const uint64_t o_ctrl = c.take(cam::fused_dispatch_ctrl_bytes());

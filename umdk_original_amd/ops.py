@@ -99,8 +99,19 @@ def moe_dispatch_plan(topk_idx, num_experts, num_ranks=1, rank=0):
     return out
 
 
+DISPATCH_LAUNCH_AUTO, DISPATCH_LAUNCH_SINGLE, DISPATCH_LAUNCH_SEPARATE = 0, 1, 2
+
+
+def set_dispatch_launch_mode(mode):
+    """Process-wide choice between the single-launch dispatch and the plan's and the permute's own launches
+    (camSetDispatchLaunchMode); the results do not depend on it."""
+    status = _lib.lib().camSetDispatchLaunchMode(int(mode))
+    if status != 0:
+        raise CamError("camSetDispatchLaunchMode failed (%d): %s" % (status, _lib.recent_error()))
+
+
 def moe_dispatch_fused(x, topk_idx, num_experts, quant_mode=0, num_rows=None, rank=0, num_ranks=1):
-    """Plan + permute (+ quantisation) in one launch (MoeDispatchPrefill of the C ABI).
+    """Plan + permute (+ quantisation) as one operator (MoeDispatchPrefill of the C ABI).
 
     Outputs are sized for `num_rows` rows (default: the worst case T*K); rows at or past total[0] are
     left unwritten.  -> dict(recv_x, recv_x_scales, expand_idx, send_token_idx, slot_row,
