@@ -195,7 +195,11 @@ __device__ __forceinline__ void run_item(const GemmArgs &a, const ItemCtx &t, in
     const int ngroups = t.N / 64;
     const int bgroup = FLAT ? TEAM * 4 + wn : wn;  // the column group of the stage this wave loads
     const int nw_load = min(nb * (FLAT ? 8 : 4) + bgroup, ngroups - 1);
-    const int8_t *b_base = t.wg + (long long)nw_load * t.Kd * 64;
+    // Packed weights: column groups in blocks of eight; inside a block the 4 KB of a K step of its groups lie
+    // side by side, so the loads of one step of a workgroup cover one contiguous stretch of memory.
+    const int b_block = nw_load >> 3;
+    const int b_step = min(8, ngroups - 8 * b_block) * 4096;
+    const int8_t *b_base = t.wg + (long long)b_block * 8 * t.Kd * 64 + (nw_load & 7) * 4096;
     const unsigned b_voff = (unsigned)(lane * 16);
     const unsigned b_dst = (unsigned)(t.stage_a + bgroup * 4096);
 
@@ -210,7 +214,7 @@ __device__ __forceinline__ void run_item(const GemmArgs &a, const ItemCtx &t, in
             }
         }
         if (NB > 0) {
-            const int8_t *bb = b_base + (long long)s * 4096;
+            const int8_t *bb = b_base + (long long)s * b_step;
 #pragma unroll
             for (int j = 0; j < NB; ++j) {
                 if (FLAT || CAM_TALL_WEIGHTS_STREAM) {  // a flat item is the only reader of its weight panel
@@ -979,9 +983,12 @@ __global__ __launch_bounds__(256) void requant_fp8_kernel(const float *__restric
     }
 }
 
-// Row-major [G,Kd,N] int8 -> MFMA operand order.  One thread writes one 16-byte piece:
-//   piece index = (((g*NW + nw)*KS + ks)*2 + nf)*64 + lane, holding K rows ks*32 + (lane/32)*16 + 0..15 of
-//   logical column  gate_up ? nf*(N/2) + nw*32 + lane%32 : nw*64 + nf*32 + lane%32.
+// Row-major [G,Kd,N] int8 -> MFMA operand order.  One thread writes one 16-byte piece: piece (nw, ks, nf, lane)
+// holds K rows ks*32 + (lane/32)*16 + 0..15 of logical column
+//   gate_up ? nf*(N/2) + nw*32 + lane%32 : nw*64 + nf*32 + lane%32.
+// The NW = N/64 column groups are stored in blocks of eight (the last block may hold fewer, gw of them); a block
+// starts at piece 8*(nw/8)*KS*128 of the expert and orders its pieces as [ks/2][nw%8][ks%2][nf][lane], i.e. the
+// gw * 4 KB that one 64-byte K step of the block's groups needs are contiguous.
 __global__ __launch_bounds__(256) void prepack_kernel(const int8_t *__restrict__ src, int8_t *__restrict__ dst,
                                                       int Kd, int N, int gate_up, long long pieces_per_expert)
 {
@@ -1010,7 +1017,12 @@ __global__ __launch_bounds__(256) void prepack_kernel(const int8_t *__restrict__
         w[j] = b0 | (b1 << 8) | (b2 << 16) | (b3 << 24);
     }
     v4u o = {w[0], w[1], w[2], w[3]};
-    *((v4u *)(dst + (long long)g * Kd * N) + p) = o;
+    const int NW = N / 64;
+    const int block = nw >> 3;
+    const int gw = min(8, NW - 8 * block);
+    const long long q = (long long)block * 8 * KS * 128 + (long long)(ks >> 1) * (gw * 256) + (nw & 7) * 256 +
+                        (ks & 1) * 128 + nf * 64 + lane;
+    *((v4u *)(dst + (long long)g * Kd * N) + q) = o;
 }
 
 int g_num_cus = 0;  // workgroups of the persistent kernel: one per CU of the current device
