@@ -376,7 +376,9 @@ CAM_API camStatus camFusedDeepMoe(void *workspace, uint64_t workspaceSize, camOp
  * GroupedMatmulFp8: x E4M3 [A,K]; xScale uint8 [A,K/128]; weight E4M3 [G,K,N], CAM_FORMAT_MFMA_B (PrepackWeight
  *   with the same gateUp); weightScale uint8 [G,K/128,N/128]; groupList int64 [G] as for the int8 operators.
  *   gateUp == 0: out fp32 [A,N] (the sums) or bf16 [A,N];  gateUp != 0: out fp32 [A,N/2] = silu(gate) * up with
- *   gate = columns [0,N/2) and up = [N/2,N) of the logical weight, as in the int8 layer.
+ *   gate = columns [0,N/2) and up = [N/2,N) of the logical weight, as in the int8 layer; or out E4M3 [A,N/2]
+ *   with outScaleOptional uint8 [A,N/256]: that product quantised in the GEMM's epilogue, bit-identical to
+ *   QuantRowsFp8 applied to the fp32 form (outScaleOptional is NULL for the other outputs).
  * QuantRowsFp8: x fp32 [A,I] -> q E4M3 [A,I], scale uint8 [A,I/128] (the re-quantisation between the two GEMMs).
  * FusedDeepMoeFp8: x bf16 [bs,H]; expertIds int32 [bs,K]; gmm1Weight E4M3 [E,H,2I] (MFMA_B, gateUp=1) with
  *   gmm1WeightScale uint8 [E,H/128,2I/128]; gmm2Weight E4M3 [E,I,H] (MFMA_B, gateUp=0) with gmm2WeightScale
@@ -387,6 +389,7 @@ CAM_API camStatus camGroupedMatmulFp8GetWorkspaceSize(const camTensor *x, const 
                                                       const camTensor *weight, const camTensor *weightScale,
                                                       int64_t gateUp, const camTensor *groupList,
                                                       int64_t groupListType, const camTensor *out,
+                                                      const camTensor *outScaleOptional,
                                                       uint64_t *workspaceSize, camOpExecutor **executor);
 CAM_API camStatus camGroupedMatmulFp8(void *workspace, uint64_t workspaceSize, camOpExecutor *executor,
                                       camStream_t stream);

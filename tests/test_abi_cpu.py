@@ -303,7 +303,7 @@ def test_fp8_operator_validation():
 
     gl = _t((2,), torch.int64)
     ok = [_t((10, 256), f8), _t((10, 2), u8), packed8((2, 256, 512)), _t((2, 2, 4), u8), 0, gl, 0,
-          _t((10, 512), torch.float32)]
+          _t((10, 512), torch.float32), None]
     assert _lib.phase1("GroupedMatmulFp8", ok)[0] == CAM_OK
     a = list(ok)
     a[7] = _t((10, 512), torch.bfloat16)
@@ -313,6 +313,16 @@ def test_fp8_operator_validation():
     assert _lib.phase1("GroupedMatmulFp8", a)[0] == CAM_OK
     a[7] = _t((10, 256), torch.bfloat16)
     assert _lib.phase1("GroupedMatmulFp8", a)[0] == CAM_ERR_DTYPE
+    a[7], a[8] = _t((10, 256), f8), _t((10, 2), u8)    # product quantised in the epilogue
+    assert _lib.phase1("GroupedMatmulFp8", a)[0] == CAM_OK
+    a[8] = None
+    assert _lib.phase1("GroupedMatmulFp8", a)[0] == CAM_ERR_NULL
+    a[8] = _t((10, 1), u8)
+    assert _lib.phase1("GroupedMatmulFp8", a)[0] == CAM_ERR_SHAPE
+    a[4], a[7], a[8] = 0, _t((10, 512), f8), _t((10, 4), u8)
+    assert _lib.phase1("GroupedMatmulFp8", a)[0] == CAM_ERR_DTYPE   # FP8 out needs the gate/up pairing
+    a[7] = _t((10, 512), torch.float32)
+    assert _lib.phase1("GroupedMatmulFp8", a)[0] == CAM_ERR_DTYPE   # outScale without an FP8 out
     a = list(ok)
     a[1] = _t((10, 3), u8)
     assert _lib.phase1("GroupedMatmulFp8", a)[0] == CAM_ERR_SHAPE

@@ -117,6 +117,43 @@ def test_grouped_matmul_fp8_bf16_output(gpu, oracle):
     assert (np.abs(got - want) <= tol).all()
 
 
+@pytest.mark.parametrize("sizes,K,N", [
+    ([33, 257, 0, 5], 1024, 512),      # flat and tall experts, an empty one, two product blocks
+    ([129, 3, 64], 4096, 768),         # three product blocks, K of the C5 layer
+    ([700, 130, 1], 256, 1280),        # 1280 = 2.5 flat column blocks: the last flat item has one live team
+    ([520], 512, 3072),                # three row tiles, N of the C5 layer
+])
+def test_grouped_matmul_fp8_quantised_product_bit_exact(gpu, oracle, sizes, K, N):
+    """The epilogue that quantises the SwiGLU product (E4M3 + E8M0 per 128 columns) against the two-step form on
+    the same device sums: fp32 product, then QuantRowsFp8.  Same arithmetic on the same values: bit for bit.
+    The fp32 product itself is pinned against the oracle by test_grouped_matmul_fp8_sums, QuantRowsFp8 by
+    test_quant_rows_fp8_bit_exact."""
+    announce("fp8 gemm quantised product sizes=%s K=%d N=%d" % (sizes, K, N))
+    G = len(sizes)
+    gl = torch.tensor(np.cumsum(sizes), dtype=torch.int64)
+    A = int(gl[-1])
+    a = _rand_fp8((A, K), K + N, 2.0)
+    sa = _rand_e8m0((A, K // 128), K + N + 1, -6, 2)
+    w = _rand_fp8((G, K, N), K + N + 2)
+    sw = _rand_e8m0((G, K // 128, N // 128), K + N + 3, -6, 2)
+    wp = cam.prepack_weight(w.to(gpu), True)
+    prod = cam.grouped_matmul_fp8(a.to(gpu), sa.to(gpu), wp, sw.to(gpu), gl.to(gpu))
+    want_q, want_s = cam.quant_rows_fp8(prod)
+    got_q, got_s = cam.grouped_matmul_fp8(a.to(gpu), sa.to(gpu), wp, sw.to(gpu), gl.to(gpu),
+                                          out_dtype=torch.float8_e4m3fn)
+    assert np.array_equal(got_s.cpu().numpy(), want_s.cpu().numpy())
+    assert np.array_equal(_u8(got_q), _u8(want_q))
+    # and against the oracle's quantisation of the oracle's product, where the device sums are within tolerance:
+    # scales may differ only where a block maximum sits on a power-of-two boundary, so compare dequantised values
+    c = oracle.fp8_gemm(_u8(a), sa.numpy(), _u8(w), sw.numpy(), gl.numpy())
+    oq, osc = oracle.fp8_quant_rows_f32(oracle.fp8_swiglu(c)[:A].astype(np.float32))
+    lut = oracle.e4m3_to_f32(np.arange(256, dtype=np.uint8)).astype(np.float64)
+    deq = lambda qq, ss: lut[qq] * np.repeat(np.exp2(ss.astype(np.float64) - 127), 128, axis=1)
+    dv, dw = deq(_u8(got_q), got_s.cpu().numpy()), deq(oq, osc)
+    blockmax = np.repeat(np.abs(dw).reshape(A, -1, 128).max(axis=2), 128, axis=1)
+    assert (np.abs(dv - dw) <= 0.13 * blockmax + 1e-30).all()
+
+
 def _layer_inputs(T, H, E, K, I, seed):
     ids, w = synth.sigmoid_zipf_routing(T, E, K, seed=seed)
     x = synth.normal_bf16(T, H, seed=seed + 1)

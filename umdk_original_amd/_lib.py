@@ -105,7 +105,7 @@ SIGNATURES = {
     "GroupedMatmulInt32": [_TP, _LP, _I64, _TP, _I64, _TP],
     "FusedDeepMoe": [_TP, _TP, _LP, _LP, _LP, _LP, _TP, _TP, _TP, _STR, _I64, _I64, _I64, _I64, _I64, _I64, _I64,
                      _TP, _TP],
-    "GroupedMatmulFp8": [_TP, _TP, _TP, _TP, _I64, _TP, _I64, _TP],
+    "GroupedMatmulFp8": [_TP, _TP, _TP, _TP, _I64, _TP, _I64, _TP, _TP],
     "QuantRowsFp8": [_TP, _TP, _TP],
     "FusedDeepMoeFp8": [_TP, _TP, _TP, _TP, _TP, _TP, _TP, _TP, _I64, _TP, _TP],
 }

@@ -1722,8 +1722,8 @@ camStatus check_fp8_dims(const char *op, int64_t Kd, int64_t N, bool gate_up)
 camStatus camGroupedMatmulFp8GetWorkspaceSize(const camTensor *x, const camTensor *xScale, const camTensor *weight,
                                               const camTensor *weightScale, int64_t gateUp,
                                               const camTensor *groupList, int64_t groupListType,
-                                              const camTensor *out, uint64_t *workspaceSize,
-                                              camOpExecutor **executor)
+                                              const camTensor *out, const camTensor *outScaleOptional,
+                                              uint64_t *workspaceSize, camOpExecutor **executor)
 {
     CAM_TRY(check_tensor(x, "x", 2, CAM_DT_FLOAT8_E4M3FN, CAM_DT_UINT8));
     CAM_TRY(check_aligned(x, "x", 16));
@@ -1742,13 +1742,31 @@ camStatus camGroupedMatmulFp8GetWorkspaceSize(const camTensor *x, const camTenso
     if (xScale->sizes[0] < A || xScale->sizes[1] != Kd / 128) {
         return fail(CAM_ERR_SHAPE, "xScale must be uint8 [rows, K/128] (E8M0)");
     }
-    CAM_TRY(check_tensor(out, "out", 2, CAM_DT_FLOAT, CAM_DT_BF16));
+    if (out == nullptr) {
+        return fail(CAM_ERR_NULL, "out is NULL");
+    }
+    const bool gate_up = gateUp != 0;
+    const bool quant_out = out->dtype == CAM_DT_FLOAT8_E4M3FN || out->dtype == CAM_DT_UINT8;
+    if (quant_out) {
+        CAM_TRY(check_tensor(out, "out", 2, CAM_DT_FLOAT8_E4M3FN, CAM_DT_UINT8));
+        if (!gate_up) {
+            return fail(CAM_ERR_DTYPE, "an FP8 out is the quantised SwiGLU product: it needs gateUp != 0");
+        }
+        CAM_TRY(check_tensor(outScaleOptional, "outScale", 2, CAM_DT_UINT8));
+        if (outScaleOptional->sizes[0] != A || outScaleOptional->sizes[1] * 128 != out->sizes[1]) {
+            return fail(CAM_ERR_SHAPE, "outScale must be uint8 [rows, I/128] (E8M0)");
+        }
+    } else {
+        CAM_TRY(check_tensor(out, "out", 2, CAM_DT_FLOAT, CAM_DT_BF16));
+        if (outScaleOptional != nullptr) {
+            return fail(CAM_ERR_DTYPE, "outScale goes with an FP8 out only");
+        }
+    }
     if (out->sizes[0] != A) {
         return fail(CAM_ERR_SHAPE, "out must have one row per row of x");
     }
-    const bool gate_up = gateUp != 0;
-    if (gate_up && out->dtype != CAM_DT_FLOAT) {
-        return fail(CAM_ERR_DTYPE, "the SwiGLU product (gateUp != 0) is written as float32");
+    if (gate_up && !quant_out && out->dtype != CAM_DT_FLOAT) {
+        return fail(CAM_ERR_DTYPE, "the SwiGLU product (gateUp != 0) is written as float32 or as FP8 with outScale");
     }
     const int64_t N = gate_up ? 2 * out->sizes[1] : out->sizes[1];
     CAM_TRY(check_fp8_dims("GroupedMatmulFp8", Kd, N, gate_up));
@@ -1767,8 +1785,11 @@ camStatus camGroupedMatmulFp8GetWorkspaceSize(const camTensor *x, const camTenso
     g.Kd = (int)Kd;
     g.N = (int)N;
     g.gate_up = gate_up;
-    g.epilogue = gate_up ? cam::kEpiSwiglu : (out->dtype == CAM_DT_BF16 ? cam::kEpiDequantBf16 : cam::kEpiInt32);
+    g.epilogue = quant_out ? cam::kEpiSwigluFp8
+                           : (gate_up ? cam::kEpiSwiglu
+                                      : (out->dtype == CAM_DT_BF16 ? cam::kEpiDequantBf16 : cam::kEpiInt32));
     g.out = out->data;
+    g.out_scale8 = quant_out ? (uint8_t *)outScaleOptional->data : nullptr;
     const int64_t *gl = (const int64_t *)groupList->data;
     const int cumulative = groupListType == 0;
     auto run = [=](void *wsp, hipStream_t s) mutable -> hipError_t {
@@ -1978,11 +1999,10 @@ camStatus camFusedDeepMoeFp8GetWorkspaceSize(const camTensor *x, const camTensor
         g1.Kd = iH;
         g1.N = 2 * iI;
         g1.gate_up = 1;
-        g1.epilogue = cam::kEpiSwiglu;
-        g1.out = prod;
+        g1.epilogue = cam::kEpiSwigluFp8;  // the SwiGLU product leaves GMM1 quantised for GMM2
+        g1.out = x2;
+        g1.out_scale8 = x2s;
         e = cam::launch_gemm(g1, s);
-        if (e != hipSuccess) return e;
-        e = cam::launch_requant_fp8(prod, A, iI, specs[0].sched, x2, x2s, s);
         if (e != hipSuccess) return e;
 
         cam::GemmArgs g2{};

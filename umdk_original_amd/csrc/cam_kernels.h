@@ -156,7 +156,7 @@ struct WeightPtrs {
     const int8_t *w[kMaxListExperts];   // used when per_expert != 0
     const float *s[kMaxListExperts];
 };
-enum GemmEpilogue { kEpiInt32 = 0, kEpiSwiglu = 1, kEpiDequantBf16 = 2 };
+enum GemmEpilogue { kEpiInt32 = 0, kEpiSwiglu = 1, kEpiDequantBf16 = 2, kEpiSwigluFp8 = 3 };
 struct GemmArgs {
     const int8_t *a;       // [A,Kd] int8
     const float *a_scale;  // [A]
@@ -168,7 +168,9 @@ struct GemmArgs {
     // Block-scaled FP8 (fp8 != 0; include/cam_fp8_spec.h): a and w hold E4M3 bytes, the fp32 scales above are
     // unused, and every 128 bytes of K carry a power-of-two scale (E8M0 byte) per activation row and per 128
     // weight columns.  Stacked weights only.  Epilogues: kEpiInt32 stores the fp32 sums, kEpiSwiglu stores
-    // silu(gate) * up as fp32, kEpiDequantBf16 stores bf16(sum).
+    // silu(gate) * up as fp32, kEpiDequantBf16 stores bf16(sum), kEpiSwigluFp8 (FP8 only) stores that product
+    // already quantised for the next GEMM: E4M3 bytes in out [A,N/2] and one E8M0 byte per row and 128 columns
+    // in out_scale8 [A,N/256], bit-identical to kEpiSwiglu followed by launch_requant_fp8.
     int fp8;
     const uint8_t *a_scale8;  // [A, Kd/128]
     const uint8_t *w_scale8;  // [G, Kd/128, N/128]
@@ -177,6 +179,7 @@ struct GemmArgs {
     int epilogue;
     void *out;             // int32 [A,N] | fp32 [A,N/2] | bf16 bits [A,N]
     int out_fp16;          // kEpiDequantBf16 writes IEEE fp16 instead of bf16
+    uint8_t *out_scale8;   // kEpiSwigluFp8: [A, N/256]
 };
 hipError_t launch_gemm(const GemmArgs &a, hipStream_t stream);
 

@@ -451,7 +451,74 @@ __device__ __forceinline__ void run_item(const GemmArgs &a, const ItemCtx &t, in
     }
     };
 
-    epilogue();
+    // ---- FP8 gate/up GEMM whose output feeds the next FP8 GEMM: quantise the SwiGLU product here.  A block of
+    // 128 product columns is exactly what the four waves of a team hold for their rows (32 columns each), so the
+    // block maximum needs one exchange through LDS; every wave of the workgroup takes part in its barrier.
+    auto epilogue_quant = [&]() {
+        const bool work = MF > 0 && t.wave_live;
+        const int wave = tid >> 6;
+        const int row_in = lane & 31;
+        const int col_half = (lane >> 5) * 4;
+        float *rowmax = (float *)(lds + 8 * kEpiSlice);  // [wave][tile row of the wave's fragments]
+        if constexpr (FP8) {
+            if (work) {
+#pragma unroll
+                for (int mf = 0; mf < MF; ++mf) {
+                    float m = 0.0f;
+#pragma unroll
+                    for (int i = 0; i < 16; ++i) {
+                        const float y = __fmul_rn(cam_silu_spec(acc[mf][0][i]), acc[mf][1][i]);
+                        acc[mf][0][i] = y;
+                        m = fmaxf(m, fabsf(y));
+                    }
+                    m = fmaxf(m, __shfl_xor(m, 32, kWave));
+                    if (lane < 32) {
+                        rowmax[wave * 128 + mf * 32 + lane] = m;
+                    }
+                }
+            }
+            wait_lds_reads();
+            barrier_no_fence();
+            if (work) {
+                const int I = t.N / 2;
+                int8_t *slice = lds + wave * kEpiSlice;
+                uint8_t *q = (uint8_t *)a.out;
+#pragma unroll
+                for (int mf = 0; mf < MF; ++mf) {
+                    const float *pm = rowmax + (wave & 4) * 128 + mf * 32 + row_in;  // the team's four waves
+                    const float m = fmaxf(fmaxf(pm[0], pm[128]), fmaxf(pm[256], pm[384]));
+                    const int ex = fp8_block_scale_exp(m);
+                    const float f1 = exp2_int(-(ex / 2)), f2 = exp2_int(-(ex - ex / 2));
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) {
+                        int w = 0;
+                        w = __builtin_amdgcn_cvt_pk_fp8_f32(__fmul_rn(__fmul_rn(acc[mf][0][4 * j], f1), f2),
+                                                            __fmul_rn(__fmul_rn(acc[mf][0][4 * j + 1], f1), f2), w, false);
+                        w = __builtin_amdgcn_cvt_pk_fp8_f32(__fmul_rn(__fmul_rn(acc[mf][0][4 * j + 2], f1), f2),
+                                                            __fmul_rn(__fmul_rn(acc[mf][0][4 * j + 3], f1), f2), w, true);
+                        *(int *)(slice + row_in * 48 + 8 * j + col_half) = w;
+                    }
+                    // 32 rows x 32 bytes staged (48-byte pitch): two lanes per row write its two 16-byte halves
+                    const int row = lane >> 1, piece = lane & 1;
+                    const v4u v = *(const v4u *)(slice + row * 48 + piece * 16);
+                    if (mf * 32 + row < t.my_rows) {
+                        const long long grow = t.m0 + t.a_row0 + mf * 32 + row;
+                        *(v4u *)(q + grow * I + t.nw * 32 + piece * 16) = v;
+                    }
+                    if ((wave & 3) == 0 && lane < 32 && mf * 32 + lane < t.my_rows) {
+                        const long long grow = t.m0 + t.a_row0 + mf * 32 + lane;
+                        a.out_scale8[grow * (I >> 7) + (t.nw >> 2)] = (uint8_t)(ex + 127);
+                    }
+                }
+            }
+        }
+    };
+
+    if (FP8 && a.epilogue == kEpiSwigluFp8) {
+        epilogue_quant();
+    } else {
+        epilogue();
+    }
     barrier_no_fence();  // the staging slices are free again before the next item's loads land
 }
 
@@ -609,7 +676,9 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_kernel(GemmArgs a)
     }
 }
 
-// Builds the schedules of up to two GEMMs over the same group list (single workgroup of 1024 threads).
+// Builds the schedules of up to two GEMMs over the same group list.  Grid (P, schedules): every workgroup derives
+// the per-expert tables for its schedule and then writes every P-th batch of 256 items; the item arithmetic
+// (divisions, a binary search) is what takes the time, so it is what is spread over workgroups.
 // Expert g with r rows: r == 0 owns nothing; r <= 128 is "flat": one tile and ceil(N/512) column blocks;
 // otherwise "tall": ceil(r/256) tiles of (nearly) equal height, a multiple of 32, and ceil(N/256) column
 // blocks.  Experts are ranked by rows, largest first.
@@ -659,7 +728,7 @@ __device__ __forceinline__ int queue_of_group(long long before, int units, long 
 }
 
 __global__ __launch_bounds__(1024) void build_sched_kernel(const int64_t *group_list, int cumulative, int G,
-                                                          long long max_rows, int nspec, SchedSpec s0, SchedSpec s1)
+                                                          long long max_rows, SchedSpec s0, SchedSpec s1)
 {
     __shared__ int rows_s[kMaxExperts], off_s[kMaxExperts], order_s[kMaxExperts];
     __shared__ int first_item_s[kMaxExperts + 1];      // by rank: items of the experts ranked before
@@ -718,8 +787,8 @@ __global__ __launch_bounds__(1024) void build_sched_kernel(const int64_t *group_
     __syncthreads();
     const int total_rows = total_rows_s;
 
-    for (int sp = 0; sp < nspec; ++sp) {
-        const SchedSpec spec = sp == 0 ? s0 : s1;
+    {
+        const SchedSpec spec = blockIdx.y == 0 ? s0 : s1;
         int32_t *sched = spec.sched;
         SchedItem *items = (SchedItem *)(sched + kSchedHeader);
         const int nb_tall = (spec.N + 255) / 256;
@@ -785,7 +854,7 @@ __global__ __launch_bounds__(1024) void build_sched_kernel(const int64_t *group_
             }
         }
         __syncthreads();
-        if (tid == 0) {
+        if (tid == 0 && blockIdx.x == 0) {
             int run = 0;
             for (int x = 0; x < kNumXcd; ++x) {
                 sched[kSchedQueueStart + x] = run;
@@ -798,8 +867,9 @@ __global__ __launch_bounds__(1024) void build_sched_kernel(const int64_t *group_
             sched[2] = 0;
             sched[3] = 0;
         }
-        // one thread per item, in rank-major order
-        for (int i = tid; i < n_items; i += 1024) {
+        // one thread per item, in rank-major order; the workgroups of a schedule share the items
+        // (256 items per workgroup and pass: four waves, one per SIMD, so that the arithmetic is not queued four deep)
+        for (int i = blockIdx.x * 256 + tid; tid < 256 && i < n_items; i += gridDim.x * 256) {
             int lo = 0, hi = G;  // largest rank with first_item <= i
             while (hi - lo > 1) {
                 const int mid = (lo + hi) >> 1;
@@ -865,7 +935,6 @@ __global__ __launch_bounds__(1024) void build_sched_kernel(const int64_t *group_
             it.pad1 = 0;
             items[pos] = it;
         }
-        __syncthreads();
     }
 }
 
@@ -1049,8 +1118,14 @@ hipError_t launch_build_sched(const int64_t *group_list, int cumulative, int G, 
     }
     const SchedSpec s0 = specs[0];
     const SchedSpec s1 = nspec > 1 ? specs[1] : specs[0];
-    hipLaunchKernelGGL(build_sched_kernel, dim3(1), dim3(1024), 0, stream, group_list, cumulative, G,
-                       (long long)max_rows, nspec, s0, s1);
+    int most = s0.max_items;
+    if (nspec > 1 && s1.max_items > most) {
+        most = s1.max_items;
+    }
+    int share = (most + 255) / 256;
+    share = share < 1 ? 1 : (share > 64 ? 64 : share);
+    hipLaunchKernelGGL(build_sched_kernel, dim3((unsigned)share, (unsigned)nspec), dim3(1024), 0, stream, group_list,
+                       cumulative, G, (long long)max_rows, s0, s1);
     return hipGetLastError();
 }
 
@@ -1078,8 +1153,14 @@ hipError_t launch_gemm(const GemmArgs &a, hipStream_t stream)
             a.per_expert || a.a_scale8 == nullptr || a.w_scale8 == nullptr) {
             return hipErrorInvalidValue;
         }
+        if (a.epilogue == kEpiSwigluFp8 && (!a.gate_up || a.out_scale8 == nullptr)) {
+            return hipErrorInvalidValue;
+        }
         hipLaunchKernelGGL(gemm_kernel<true>, dim3((unsigned)g_num_cus), dim3(kThreads), 0, stream, a);
     } else {
+        if (a.epilogue == kEpiSwigluFp8) {
+            return hipErrorInvalidValue;
+        }
         hipLaunchKernelGGL(gemm_kernel<false>, dim3((unsigned)g_num_cus), dim3(kThreads), 0, stream, a);
     }
     return hipGetLastError();

@@ -322,17 +322,23 @@ def grouped_matmul_int32(x, weight, group_list, group_list_type=0):
 # Block-scaled FP8 (a definition of this library: include/cam_fp8_spec.h; the reference is W8A8 only)
 def grouped_matmul_fp8(x, x_scale, weight, weight_scale, group_list, group_list_type=0, out_dtype=torch.float32):
     """x E4M3 [A,K], x_scale uint8 [A,K/128], weight E4M3 [G,K,N] prepacked, weight_scale uint8 [G,K/128,N/128].
-    Prepacked with gate_up=True: -> fp32 [A,N/2] = silu(gate) * up; else -> out_dtype [A,N] (fp32 sums or bf16)."""
+    Prepacked with gate_up=True: -> fp32 [A,N/2] = silu(gate) * up, or, with out_dtype=torch.float8_e4m3fn, that
+    product quantised in the epilogue -> (E4M3 [A,N/2], uint8 E8M0 scales [A,N/256]);
+    else -> out_dtype [A,N] (fp32 sums or bf16)."""
     _tag_list([weight])
     gate_up = bool(getattr(weight, "_cam_gate_up", False))
     n = weight.size(-1)
-    if gate_up:
+    out_scale = None
+    if gate_up and out_dtype == torch.float8_e4m3fn:
+        out = torch.empty((x.size(0), n // 2), dtype=torch.float8_e4m3fn, device=x.device)
+        out_scale = torch.empty((x.size(0), n // 256), dtype=torch.uint8, device=x.device)
+    elif gate_up:
         out = torch.empty((x.size(0), n // 2), dtype=torch.float32, device=x.device)
     else:
         out = torch.empty((x.size(0), n), dtype=out_dtype, device=x.device)
     _lib.call("GroupedMatmulFp8", [x, x_scale, weight, weight_scale, 1 if gate_up else 0, group_list,
-                                   group_list_type, out])
-    return out
+                                   group_list_type, out, out_scale])
+    return out if out_scale is None else (out, out_scale)
 
 
 def quant_rows_fp8(x):
