@@ -1578,6 +1578,9 @@ camStatus camFusedDeepMoeGetWorkspaceSize(const camTensor *x, const camTensor *e
         p.meta = meta;
         p.hist_ws = (int32_t *)(w + o_hist);
         hipError_t e;
+        cam::SchedSpec specs[2] = {sp1, sp2};  // both GEMM schedules come from the per-expert counts of the plan
+        specs[0].sched = (int32_t *)(w + o_sched1);
+        specs[1].sched = (int32_t *)(w + o_sched2);
         if (fused_dispatch) {
             cam::FusedDispatchArgs f{};
             f.p = p;
@@ -1607,16 +1610,21 @@ camStatus camFusedDeepMoeGetWorkspaceSize(const camTensor *x, const camTensor *e
             d.quant = 2;
             d.out = x1;
             d.scales = x1s;
+            // the plan has written the per-expert counts: spare workgroups of the permute build both schedules
+            d.sched.group_list = etn;
+            d.sched.cumulative = 0;
+            d.sched.G = iE;
+            d.sched.nspec = 2;
+            d.sched.max_rows = A;
+            d.sched.spec[0] = specs[0];
+            d.sched.spec[1] = specs[1];
             e = cam::launch_dispatch(d, s);
             if (e != hipSuccess) return e;
         }
-
-        // both GEMM schedules from the per-expert counts the plan has just written
-        cam::SchedSpec specs[2] = {sp1, sp2};
-        specs[0].sched = (int32_t *)(w + o_sched1);
-        specs[1].sched = (int32_t *)(w + o_sched2);
-        e = cam::launch_build_sched(etn, 0, iE, A, 2, specs, s);
-        if (e != hipSuccess) return e;
+        if (fused_dispatch) {  // the counts exist only once the single launch is over
+            e = cam::launch_build_sched(etn, 0, iE, A, 2, specs, s);
+            if (e != hipSuccess) return e;
+        }
 
         cam::GemmArgs g1{};
         g1.a = x1;
@@ -1951,6 +1959,9 @@ camStatus camFusedDeepMoeFp8GetWorkspaceSize(const camTensor *x, const camTensor
         p.meta = meta;
         p.hist_ws = (int32_t *)(w + o_hist);
         hipError_t e;
+        cam::SchedSpec specs[2] = {sp1, sp2};
+        specs[0].sched = (int32_t *)(w + o_sched1);
+        specs[1].sched = (int32_t *)(w + o_sched2);
         if (fused_dispatch) {
             cam::FusedDispatchArgs f{};
             f.p = p;
@@ -1980,14 +1991,20 @@ camStatus camFusedDeepMoeFp8GetWorkspaceSize(const camTensor *x, const camTensor
             d.quant = 3;
             d.out = x1;
             d.scales = (float *)x1s;
+            d.sched.group_list = etn;  // spare workgroups of the permute build both schedules
+            d.sched.cumulative = 0;
+            d.sched.G = iE;
+            d.sched.nspec = 2;
+            d.sched.max_rows = A;
+            d.sched.spec[0] = specs[0];
+            d.sched.spec[1] = specs[1];
             e = cam::launch_dispatch(d, s);
             if (e != hipSuccess) return e;
         }
-        cam::SchedSpec specs[2] = {sp1, sp2};
-        specs[0].sched = (int32_t *)(w + o_sched1);
-        specs[1].sched = (int32_t *)(w + o_sched2);
-        e = cam::launch_build_sched(etn, 0, iE, A, 2, specs, s);
-        if (e != hipSuccess) return e;
+        if (fused_dispatch) {  // the counts exist only once the single launch is over
+            e = cam::launch_build_sched(etn, 0, iE, A, 2, specs, s);
+            if (e != hipSuccess) return e;
+        }
 
         cam::GemmArgs g1{};
         g1.a = (const int8_t *)x1;

@@ -17,6 +17,7 @@ constexpr int kMaxListExperts = 64;  // per-expert weight tensors that fit in th
 //   [kSchedQueueStart .. +8]  first item of each of the 8 queues, and the end of the last
 //   [kSchedQueueCount + 32 x] items already taken from queue x (zeroed by the builder, advanced by the GEMM);
 //                             one counter per 128-byte line, so that the queues do not share a line
+constexpr int kNumXcd = 8;  // queues of a schedule: workgroup i of a launch runs on XCD i % 8
 constexpr int kSchedHeader = 32 + 8 * 32;
 constexpr int kSchedQueueStart = 4;
 constexpr int kSchedQueueCount = 32;
@@ -82,6 +83,15 @@ int sched_max_items(int64_t max_rows, int G, int N);
 uint64_t sched_bytes(int64_t max_rows, int G, int N);
 hipError_t launch_build_sched(const int64_t *group_list, int cumulative, int G, int64_t max_rows, int nspec,
                               const SchedSpec *specs, hipStream_t stream);
+// The same job as kernel arguments: nspec == 0 means "nothing to build".
+struct SchedBuild {
+    const int64_t *group_list;
+    int cumulative, G, nspec;
+    long long max_rows;
+    SchedSpec spec[2];
+};
+// Workgroups that share the building of one schedule of sb (each writes every parts-th batch of 256 items).
+int sched_build_parts(const SchedBuild &sb);
 
 // ---------------------------------------------------------------------------------------------
 // Permute (+ per-token int8 quantisation).
@@ -99,6 +109,11 @@ struct DispatchArgs {
     float *scales;       // [A]   (quant only)
     int32_t *src_info;   // [3A]  optional
     int src_rank;
+    // GEMM schedules to build in the same launch (sched.nspec > 0): sched.nspec * sched_parts extra workgroups
+    // do what launch_build_sched would, beside the ones that move rows.  The group list must be complete before
+    // the launch (it is when it comes from launch_plan on the same stream).  sched_parts is set by the launcher.
+    SchedBuild sched;
+    int sched_parts;
 };
 hipError_t launch_dispatch(const DispatchArgs &a, hipStream_t stream);
 

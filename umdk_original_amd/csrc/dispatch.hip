@@ -17,6 +17,7 @@
 #include "cam_device.h"
 #include "cam_kernels.h"
 #include "permute_device.h"
+#include "sched_device.h"
 
 namespace cam {
 
@@ -41,7 +42,16 @@ __device__ __forceinline__ long long dispatch_row(const DispatchArgs &a, int t, 
 template <int QUANT, int ACT>
 __global__ __launch_bounds__(kDispWaves * kWave) void dispatch_kernel(DispatchArgs a)
 {
-    const int t = blockIdx.x * kDispWaves + (threadIdx.x >> 6);
+    // The first workgroups of the launch build the GEMM schedules (they start first and finish under the row
+    // traffic of the others); they depend on nothing this launch writes.
+    __shared__ SchedShared sched_s;
+    const int builders = a.sched.nspec * a.sched_parts;
+    if ((int)blockIdx.x < builders) {
+        build_sched_part<kDispWaves * kWave>(sched_s, a.sched, (int)blockIdx.x / a.sched_parts,
+                                             (int)blockIdx.x % a.sched_parts, a.sched_parts);
+        return;
+    }
+    const int t = ((int)blockIdx.x - builders) * kDispWaves + (threadIdx.x >> 6);
     const int lane = threadIdx.x & (kWave - 1);
     if (t >= a.T) {
         return;
@@ -62,15 +72,29 @@ __global__ __launch_bounds__(kDispWaves * kWave) void dispatch_kernel(DispatchAr
 
 }  // namespace
 
-hipError_t launch_dispatch(const DispatchArgs &a, hipStream_t stream)
+hipError_t launch_dispatch(const DispatchArgs &a_in, hipStream_t stream)
 {
-    if (a.T <= 0) {
+    if (a_in.T <= 0) {
+        if (a_in.sched.nspec > 0) {  // no rows to move, but the schedules are still owed
+            return launch_build_sched(a_in.sched.group_list, a_in.sched.cumulative, a_in.sched.G, a_in.sched.max_rows,
+                                      a_in.sched.nspec, a_in.sched.spec, stream);
+        }
         return hipSuccess;
     }
-    if (a.H % 8 != 0 || a.H / 8 > kDispMaxChunks * kWave || (a.quant == 3 && a.H % 128 != 0)) {
+    const DispatchArgs &a0 = a_in;
+    if (a0.H % 8 != 0 || a0.H / 8 > kDispMaxChunks * kWave || (a0.quant == 3 && a0.H % 128 != 0)) {
         return hipErrorInvalidValue;
     }
-    dim3 grid((a.T + kDispWaves - 1) / kDispWaves), block(kDispWaves * kWave);
+    DispatchArgs a = a_in;
+    a.sched_parts = 0;
+    if (a.sched.nspec != 0) {
+        if (a.sched.nspec < 0 || a.sched.nspec > 2 || a.sched.G <= 0 || a.sched.G > kMaxExperts ||
+            a.sched.group_list == nullptr) {
+            return hipErrorInvalidValue;
+        }
+        a.sched_parts = sched_build_parts(a.sched);
+    }
+    dim3 grid((a.T + kDispWaves - 1) / kDispWaves + a.sched.nspec * a.sched_parts), block(kDispWaves * kWave);
     if (a.quant == 0) {
         hipLaunchKernelGGL((dispatch_kernel<0, 0>), grid, block, 0, stream, a);  // a copy does not look at the format
     } else if (a.quant == 1) {

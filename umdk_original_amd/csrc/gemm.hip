@@ -49,6 +49,7 @@
 #include "cam_kernels.h"
 #include "rank_device.h"
 #include "permute_device.h"
+#include "sched_device.h"
 #include "../../include/cam_expf_spec.h"
 
 namespace cam {
@@ -57,7 +58,6 @@ namespace {
 
 constexpr int kBK = 64;                         // K bytes per sub-step
 constexpr int kThreads = 512;                   // two teams of four waves
-constexpr int kNumXcd = 8;
 constexpr int kMaxStages = 4;
 constexpr int kStageTall = 256 * kBK + 256 * kBK;   // 16 KB of activations + 16 KB of weights
 constexpr int kStageFlat = 128 * kBK + 512 * kBK;   //  8 KB of activations + 32 KB of weights
@@ -571,12 +571,22 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_kernel(GemmArgs a)
             }
             own_empty = true;
         }
+        // Look at all the other queues at once: a look is a round trip to the memory side (1-2 us), and a
+        // workgroup that finds nothing does this before it leaves, so seven looks in a row would be the tail of
+        // every launch.
+        int seen[kNumXcd - 1], len[kNumXcd - 1];
+#pragma unroll
         for (int k = 1; k < kNumXcd; ++k) {
             const int qq = (q + k) % kNumXcd;
-            const int len = qstart[qq + 1] - qstart[qq];
-            if (__hip_atomic_load(&qcount[qq * kSchedQueueStride], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) < len) {
+            seen[k - 1] = __hip_atomic_load(&qcount[qq * kSchedQueueStride], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            len[k - 1] = qstart[qq + 1] - qstart[qq];
+        }
+#pragma unroll
+        for (int k = 1; k < kNumXcd; ++k) {
+            const int qq = (q + k) % kNumXcd;
+            if (seen[k - 1] < len[k - 1]) {
                 const int i = atomicAdd(&qcount[qq * kSchedQueueStride], 1);
-                if (i < len) {
+                if (i < len[k - 1]) {
                     return qstart[qq] + i;
                 }
             }
@@ -676,266 +686,10 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_kernel(GemmArgs a)
     }
 }
 
-// Builds the schedules of up to two GEMMs over the same group list.  Grid (P, schedules): every workgroup derives
-// the per-expert tables for its schedule and then writes every P-th batch of 256 items; the item arithmetic
-// (divisions, a binary search) is what takes the time, so it is what is spread over workgroups.
-// Expert g with r rows: r == 0 owns nothing; r <= 128 is "flat": one tile and ceil(N/512) column blocks;
-// otherwise "tall": ceil(r/256) tiles of (nearly) equal height, a multiple of 32, and ceil(N/256) column
-// blocks.  Experts are ranked by rows, largest first.
-//   * Tall experts: the (expert, column block) groups, in rank order, are cut into eight consecutive runs of
-//     equal work (rows x column blocks), one per queue.  A queue therefore holds few experts, each with
-//     neighbouring column blocks: the CUs of an XCD that work side by side share the weight panels (row tiles
-//     of one group) and the activation tiles (column blocks of one expert) through their L2, and an expert's
-//     activations are fetched by as few XCDs as its size requires.
-//   * Flat experts are dealt to the queues whole, in rank order, so that the column blocks of one expert,
-//     which all read the same few activation rows, run on one XCD.
-// A queue lists its tall items big experts first, with its flat items spread evenly among them except for the
-// last kTallTail places.  A flat item streams its weights at the pace one CU can pull them from memory and takes
-// longer than a tall one although it computes less: spread out, flat items run beside tall ones, which need
-// the matrix cores rather than the memory, and the queues end with items of even length.
-// The work is laid out so that it needs few workgroup barriers: every prefix sum over the experts is the job
-// of one wave, which walks the ranks 64 at a time.
-constexpr int kTallTail = 24;  // tall items a queue ends with (three quarters of a round of its 32 workgroups)
-
-struct ExpertShape {
-    int rows, tiles, blocks, units;
-    bool tall, flat;
-};
-
-__device__ __forceinline__ ExpertShape expert_shape(int rows, int nb_tall, int nb_flat)
+__global__ __launch_bounds__(1024) void build_sched_kernel(SchedBuild sb)
 {
-    ExpertShape e;
-    e.rows = rows;
-    e.tall = rows > 128;
-    e.flat = rows > 0 && !e.tall;
-    e.tiles = e.tall ? (rows + 255) / 256 : (e.flat ? 1 : 0);
-    e.blocks = e.tall ? nb_tall : (e.flat ? nb_flat : 0);
-    e.units = (rows + 31) / 32;
-    return e;
-}
-
-// Queue of the tall group whose work (in units) starts at `before` and is `units` long: the queue its middle
-// falls into when the total work is cut into eight equal runs.
-__device__ __forceinline__ int queue_of_group(long long before, int units, long long wtotal)
-{
-    const long long mid16 = (2 * before + units) * kNumXcd;  // 2 * middle * 8
-    int x = 0;
-#pragma unroll
-    for (int k = 1; k < kNumXcd; ++k) {
-        x += mid16 >= 2 * wtotal * k ? 1 : 0;
-    }
-    return x;
-}
-
-__global__ __launch_bounds__(1024) void build_sched_kernel(const int64_t *group_list, int cumulative, int G,
-                                                          long long max_rows, SchedSpec s0, SchedSpec s1)
-{
-    __shared__ int rows_s[kMaxExperts], off_s[kMaxExperts], order_s[kMaxExperts];
-    __shared__ int first_item_s[kMaxExperts + 1];      // by rank: items of the experts ranked before
-    __shared__ int work_before_s[kMaxExperts];         // by rank: work of the tall experts ranked before
-    __shared__ int flat_rank_s[kMaxExperts];           // by rank: flat experts ranked before
-    __shared__ short ngroups_s[kNumXcd][kMaxExperts];  // by rank: the expert's groups in queue x (tall)
-    __shared__ int qbase_s[kNumXcd][kMaxExperts];      // by rank: items of earlier experts of its kind in queue x
-    __shared__ int qtall_s[kNumXcd], qflat_s[kNumXcd];
-    __shared__ int wtotal_s, total_rows_s;
-    const int tid = threadIdx.x;
-    const int lane = tid & (kWave - 1);
-    const int wave = tid >> 6;
-
-    // rows and first row of every expert (wave 0)
-    if (wave == 0) {
-        long long run = 0;  // rows before this chunk (counts) / unused (cumulative)
-        for (int base = 0; base < G; base += kWave) {
-            const int g = base + lane;
-            long long m0 = 0, m1 = 0;
-            if (cumulative) {
-                if (g < G) {
-                    m0 = g == 0 ? 0 : group_list[g - 1];
-                    m1 = group_list[g];
-                }
-            } else {
-                const int c = g < G ? (int)min(max(group_list[g], (int64_t)0), (int64_t)max_rows) : 0;
-                const int inc = wave_inclusive_scan(c, lane);
-                m0 = run + inc - c;
-                m1 = m0 + c;
-                run += __shfl(inc, kWave - 1, kWave);
-            }
-            // Clamp to the rows that exist so that a corrupt group list cannot index past the tensors.
-            m0 = min(max(m0, 0ll), max_rows);
-            m1 = min(max(m1, m0), max_rows);
-            if (g < G) {
-                rows_s[g] = (int)(m1 - m0);
-                off_s[g] = (int)m0;
-            }
-            const int chunk_rows = wave_sum(g < G ? (int)(m1 - m0) : 0);
-            if (lane == 0) {
-                total_rows_s = (base == 0 ? 0 : total_rows_s) + chunk_rows;
-            }
-        }
-    }
-    __syncthreads();
-    // rank by rows, largest first (ties: lower index first)
-    if (tid < G) {
-        const int cnt = rows_s[tid];
-        int rank = 0;
-        for (int j = 0; j < G; ++j) {
-            const int rj = rows_s[j];
-            rank += (rj > cnt || (rj == cnt && j < tid)) ? 1 : 0;
-        }
-        order_s[rank] = tid;
-    }
-    __syncthreads();
-    const int total_rows = total_rows_s;
-
-    {
-        const SchedSpec spec = blockIdx.y == 0 ? s0 : s1;
-        int32_t *sched = spec.sched;
-        SchedItem *items = (SchedItem *)(sched + kSchedHeader);
-        const int nb_tall = (spec.N + 255) / 256;
-        const int nb_flat = (spec.N + 511) / 512;
-
-        // by rank: items, tall work and flat experts before (wave 0)
-        if (wave == 0) {
-            int items_run = 0, work_run = 0, flat_run = 0;
-            for (int base = 0; base < G; base += kWave) {
-                const int rank = base + lane;
-                const ExpertShape e = expert_shape(rank < G ? rows_s[order_s[rank]] : 0, nb_tall, nb_flat);
-                const int vi = e.blocks * e.tiles, vw = e.tall ? e.blocks * e.units : 0, vf = e.flat ? 1 : 0;
-                const int ii = wave_inclusive_scan(vi, lane);
-                const int iw = wave_inclusive_scan(vw, lane);
-                const int jf = wave_inclusive_scan(vf, lane);
-                if (rank < G) {
-                    first_item_s[rank] = items_run + ii - vi;
-                    work_before_s[rank] = work_run + iw - vw;
-                    flat_rank_s[rank] = flat_run + jf - vf;
-                }
-                items_run += __shfl(ii, kWave - 1, kWave);
-                work_run += __shfl(iw, kWave - 1, kWave);
-                flat_run += __shfl(jf, kWave - 1, kWave);
-            }
-            if (lane == 0) {
-                first_item_s[G] = items_run;
-                wtotal_s = max(work_run, 1);
-            }
-        }
-        __syncthreads();
-        const int n_items = first_item_s[G];
-        const long long wtotal = wtotal_s;
-
-        // by rank and queue: items of earlier experts.  Wave x (0..7) counts the tall items of queue x, wave 8 + x
-        // its flat items.
-        {
-            const int x = wave & (kNumXcd - 1);
-            const bool flat_wave = wave >= kNumXcd;
-            int run = 0;
-            for (int base = 0; base < G; base += kWave) {
-                const int rank = base + lane;
-                const ExpertShape e = expert_shape(rank < G ? rows_s[order_s[rank]] : 0, nb_tall, nb_flat);
-                int v = 0;
-                if (flat_wave) {
-                    v = (e.flat && flat_rank_s[rank] % kNumXcd == x) ? e.blocks : 0;
-                } else if (e.tall) {
-                    int mine = 0;
-                    const long long before = work_before_s[rank];
-                    for (int c = 0; c < e.blocks; ++c) {
-                        mine += queue_of_group(before + (long long)c * e.units, e.units, wtotal) == x ? 1 : 0;
-                    }
-                    ngroups_s[x][rank] = (short)mine;
-                    v = mine * e.tiles;
-                }
-                const int inc = wave_inclusive_scan(v, lane);
-                if (rank < G && (flat_wave ? e.flat : e.tall)) {
-                    qbase_s[x][rank] = run + inc - v;
-                }
-                run += __shfl(inc, kWave - 1, kWave);
-            }
-            if (lane == 0) {
-                (flat_wave ? qflat_s : qtall_s)[x] = run;
-            }
-        }
-        __syncthreads();
-        if (tid == 0 && blockIdx.x == 0) {
-            int run = 0;
-            for (int x = 0; x < kNumXcd; ++x) {
-                sched[kSchedQueueStart + x] = run;
-                sched[kSchedQueueCount + x * kSchedQueueStride] = 0;
-                run += qflat_s[x] + qtall_s[x];
-            }
-            sched[kSchedQueueStart + kNumXcd] = run;
-            sched[0] = min(n_items, spec.max_items);
-            sched[1] = total_rows;
-            sched[2] = 0;
-            sched[3] = 0;
-        }
-        // one thread per item, in rank-major order; the workgroups of a schedule share the items
-        // (256 items per workgroup and pass: four waves, one per SIMD, so that the arithmetic is not queued four deep)
-        for (int i = blockIdx.x * 256 + tid; tid < 256 && i < n_items; i += gridDim.x * 256) {
-            int lo = 0, hi = G;  // largest rank with first_item <= i
-            while (hi - lo > 1) {
-                const int mid = (lo + hi) >> 1;
-                if (first_item_s[mid] <= i) {
-                    lo = mid;
-                } else {
-                    hi = mid;
-                }
-            }
-            const int rank = lo;
-            const int eg = order_s[rank];
-            const ExpertShape e = expert_shape(rows_s[eg], nb_tall, nb_flat);
-            const int local = i - first_item_s[rank];
-            const int c = local / e.tiles;
-            const int j = local - c * e.tiles;
-            int x, qpos;
-            if (e.flat) {
-                x = flat_rank_s[rank] % kNumXcd;
-                qpos = qbase_s[x][rank] + c;
-            } else {
-                x = queue_of_group(work_before_s[rank] + (long long)c * e.units, e.units, wtotal);
-                int cfirst = 0;  // the expert's groups in earlier queues
-                for (int xx = 0; xx < x; ++xx) {
-                    cfirst += ngroups_s[xx][rank];
-                }
-                qpos = qbase_s[x][rank] + (c - cfirst) * e.tiles + j;
-            }
-            {
-                // Queue order: the flat items spread evenly among the tall ones (flat item j has key (2j+1)/(2F),
-                // tall item i key (2i+1)/(2T), smaller keys first, a tall item first on a tie), except that the
-                // last kTallTail tall items follow the last flat one.
-                const long long F = qflat_s[x];
-                const long long T = max(qtall_s[x] - kTallTail, 0);
-                if (e.flat) {
-                    const long long num = (2ll * qpos + 1) * T - F;
-                    qpos += (int)(num < 0 ? 0 : min(T, num / (2 * F) + 1));
-                } else if (qpos < T) {
-                    const long long num = (2ll * qpos + 1) * F - T;
-                    qpos += (int)(num <= 0 ? 0 : min(F, (num + 2 * T - 1) / (2 * T)));
-                } else {
-                    qpos += (int)F;
-                }
-            }
-            int pos = qpos;
-            for (int xx = 0; xx < x; ++xx) {
-                pos += qflat_s[xx] + qtall_s[xx];
-            }
-            if (pos >= spec.max_items) {
-                continue;  // cannot happen with a table sized by sched_bytes(); guards a corrupt list
-            }
-            // tile j of e.tiles: heights are multiples of 32 that differ by at most 32
-            const int base_u = e.units / e.tiles, extra = e.units % e.tiles;
-            const int u0 = j * base_u + min(j, extra);
-            const int uj = base_u + (j < extra ? 1 : 0);
-            SchedItem it;
-            it.g = eg;
-            it.m0 = off_s[eg] + u0 * 32;
-            it.rows = min(uj * 32, e.rows - u0 * 32);
-            it.split = e.flat ? 0 : 32 * ((it.rows + 63) / 64);
-            it.nb = c;
-            it.flat = e.flat ? 1 : 0;
-            it.pad0 = 0;
-            it.pad1 = 0;
-            items[pos] = it;
-        }
-    }
+    __shared__ SchedShared sh;
+    build_sched_part<1024>(sh, sb, (int)blockIdx.y, (int)blockIdx.x, (int)gridDim.x);
 }
 
 // SwiGLU product rows (fp32) -> int8 rows + per-row scale:
@@ -1110,22 +864,32 @@ uint64_t sched_bytes(int64_t max_rows, int G, int N)
     return (uint64_t)(kSchedHeader + (int64_t)sched_max_items(max_rows, G, N) * (int)(sizeof(SchedItem) / 4)) * 4;
 }
 
+int sched_build_parts(const SchedBuild &sb)
+{
+    int most = 0;
+    for (int i = 0; i < sb.nspec; ++i) {
+        most = sb.spec[i].max_items > most ? sb.spec[i].max_items : most;
+    }
+    const int parts = (most + 255) / 256;
+    return parts < 1 ? 1 : (parts > 64 ? 64 : parts);
+}
+
 hipError_t launch_build_sched(const int64_t *group_list, int cumulative, int G, int64_t max_rows, int nspec,
                               const SchedSpec *specs, hipStream_t stream)
 {
     if (G <= 0 || G > kMaxExperts || nspec < 1 || nspec > 2) {
         return hipErrorInvalidValue;
     }
-    const SchedSpec s0 = specs[0];
-    const SchedSpec s1 = nspec > 1 ? specs[1] : specs[0];
-    int most = s0.max_items;
-    if (nspec > 1 && s1.max_items > most) {
-        most = s1.max_items;
-    }
-    int share = (most + 255) / 256;
-    share = share < 1 ? 1 : (share > 64 ? 64 : share);
-    hipLaunchKernelGGL(build_sched_kernel, dim3((unsigned)share, (unsigned)nspec), dim3(1024), 0, stream, group_list,
-                       cumulative, G, (long long)max_rows, s0, s1);
+    SchedBuild sb{};
+    sb.group_list = group_list;
+    sb.cumulative = cumulative;
+    sb.G = G;
+    sb.nspec = nspec;
+    sb.max_rows = (long long)max_rows;
+    sb.spec[0] = specs[0];
+    sb.spec[1] = nspec > 1 ? specs[1] : specs[0];
+    hipLaunchKernelGGL(build_sched_kernel, dim3((unsigned)sched_build_parts(sb), (unsigned)nspec), dim3(1024), 0,
+                       stream, sb);
     return hipGetLastError();
 }
 

@@ -133,6 +133,71 @@ __global__ __launch_bounds__(kGlobalThreads) void plan_global_kernel(PlanArgs a,
     }
 }
 
+// Both phases in one workgroup, for id sequences that fit one chunk (at most 8 * 256 entries): the chunk's
+// histogram is the per-expert count and every base is zero, so nothing has to pass between workgroups and the
+// plan costs one launch instead of two.
+template <typename IdT, int IT>
+__global__ __launch_bounds__(kLocalThreads) void plan_single_kernel(PlanArgs a)
+{
+    __shared__ int hist[kLocalWaves * kMaxExperts];
+    __shared__ int cnt_s[kMaxExperts];
+    __shared__ int off_s[kMaxExperts];
+    __shared__ int scan_s[kLocalWaves];
+    __shared__ int total_s;
+    __shared__ int active_s;
+    const int tid = threadIdx.x;
+    const int E = a.E;
+    const IdT *__restrict__ idx = (const IdT *)a.idx;
+    const int t_active = count_active(a.mask, a.T, tid, kLocalThreads, &active_s);
+    const long long n = (long long)t_active * a.K;
+    const long long n_all = (long long)a.T * a.K;
+    rank_chunk<IdT, IT>(idx, 0, n, n_all, E, hist, a.pos, cnt_s);
+    __syncthreads();  // cnt_s complete; the ranks in a.pos are visible to the whole workgroup
+    // thread i owns experts 2i and 2i+1
+    int c2[2];
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+        c2[h] = 2 * tid + h < E ? cnt_s[2 * tid + h] : 0;
+    }
+    const int pair_off = block_exclusive_scan<kLocalWaves>(c2[0] + c2[1], tid, scan_s, &total_s);
+    const int total = total_s;
+    const int o2[2] = {pair_off, pair_off + c2[0]};
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+        const int e = 2 * tid + h;
+        if (e < E) {
+            off_s[e] = o2[h];
+            if (a.cnt) a.cnt[e] = c2[h];
+            if (a.off) a.off[e] = o2[h];
+            if (a.recv_off) a.recv_off[e] = o2[h];
+            if (a.recv_count) a.recv_count[e] = o2[h] + c2[h];
+            if (a.tokens_per_expert) a.tokens_per_expert[e] = c2[h];
+            if (a.group_list) a.group_list[e] = (int64_t)o2[h] + c2[h];
+        }
+    }
+    __syncthreads();
+    if (a.dst_row != nullptr) {
+        for (long long i = tid; i < n_all; i += kLocalThreads) {
+            const int e = i < n ? load_id(idx, i, E) : -1;
+            a.dst_row[i] = e >= 0 ? off_s[e] + a.pos[i] : -1;
+        }
+    }
+    if (tid == 0 && a.total) {
+        a.total[0] = total;
+    }
+    if (a.per_rank_zero != nullptr) {
+        for (int r = tid; r < a.R; r += kLocalThreads) {
+            a.per_rank_zero[r] = 0;
+        }
+    }
+    if (tid == 0 && a.meta != nullptr) {
+        a.meta[0] = 0;
+        a.meta[1] = total;
+        a.meta[2] = t_active;
+        a.meta[3] = 0;
+    }
+}
+
 // isTokenInRank[t,r] and numTokensPerRank[r] (dispatch_layout.h:106-123): a token counts once per rank.
 template <typename IdT, typename OutT>
 __global__ __launch_bounds__(256) void in_rank_kernel(InRankArgs a)
@@ -204,6 +269,15 @@ template <typename IdT>
 hipError_t launch_plan_t(const PlanArgs &a, int it, int nb, int32_t *hist, hipStream_t stream)
 {
     dim3 grid(nb), blk(kLocalThreads);
+    if (nb == 1) {
+        switch (it) {
+            case 1: hipLaunchKernelGGL((plan_single_kernel<IdT, 1>), grid, blk, 0, stream, a); break;
+            case 2: hipLaunchKernelGGL((plan_single_kernel<IdT, 2>), grid, blk, 0, stream, a); break;
+            case 4: hipLaunchKernelGGL((plan_single_kernel<IdT, 4>), grid, blk, 0, stream, a); break;
+            default: hipLaunchKernelGGL((plan_single_kernel<IdT, 8>), grid, blk, 0, stream, a); break;
+        }
+        return hipGetLastError();
+    }
     switch (it) {
         case 1: hipLaunchKernelGGL((plan_local_kernel<IdT, 1>), grid, blk, 0, stream, a, hist); break;
         case 2: hipLaunchKernelGGL((plan_local_kernel<IdT, 2>), grid, blk, 0, stream, a, hist); break;
@@ -224,8 +298,14 @@ hipError_t launch_plan_t(const PlanArgs &a, int it, int nb, int32_t *hist, hipSt
 void plan_geometry(long long n_all, int *it_out, int *nb_out)
 {
     int it = 1;
-    while (it < 8 && (n_all + (long long)it * kLocalThreads - 1) / ((long long)it * kLocalThreads) > 64) {
-        it *= 2;
+    if (n_all <= 8 * kLocalThreads) {  // one chunk: the single-workgroup plan
+        while ((long long)it * kLocalThreads < n_all) {
+            it *= 2;
+        }
+    } else {
+        while (it < 8 && (n_all + (long long)it * kLocalThreads - 1) / ((long long)it * kLocalThreads) > 64) {
+            it *= 2;
+        }
     }
     long long nb = (n_all + (long long)it * kLocalThreads - 1) / ((long long)it * kLocalThreads);
     *it_out = it;
