@@ -75,11 +75,18 @@ CAM_SPEC_FN float cam_expf_spec(float x)
     float r2 = CAM_FMUL(r, r);
     float y = CAM_FADD(CAM_FADD(CAM_FMUL(p, r2), r), 1.0f);
     int ni = (int)n; /* |n| <= 150, exact */
+#if defined(__HIP_DEVICE_COMPILE__)
+    /* One v_ldexp_f32 gives the bits of the two multiplies below: y * s1 is exact (y in [0.7, 1.5], |n1| <= 75, the
+     * product stays normal), so the second multiply is the only rounding, and it rounds y * 2^n to nearest even
+     * exactly as ldexp does, into the subnormals and up to infinity alike. */
+    return __builtin_ldexpf(y, ni);
+#else
     int n1 = ni / 2;
     int n2 = ni - n1;
     float s1 = CAM_BITS_TO_F((uint32_t)(n1 + 127) << 23);
     float s2 = CAM_BITS_TO_F((uint32_t)(n2 + 127) << 23);
     return CAM_FMUL(CAM_FMUL(y, s1), s2);
+#endif
 }
 
 /* SiLU exactly as the reference orders it: e = exp(-t); d = 1 + e; out = t / d (IEEE division). */

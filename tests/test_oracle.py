@@ -294,6 +294,24 @@ def test_expf_spec_accuracy_and_edges(oracle):
     assert (np.diff(mono) >= 0).all()
 
 
+def test_expf_scaling_by_two_multiplies_equals_ldexp():
+    """The exp specification scales y in [0.7, 1.5] by 2^n with two power-of-two multiplies; the device code uses one
+    ldexp instead.  Both round y * 2^n once, to nearest even: identical bits for every n the specification can
+    produce (-150 .. 128), subnormal results, zero and infinity included."""
+    rng = _rng(123)
+    y = np.concatenate([rng.uniform(0.70, 1.42, 200000), [0.70710677, 1.0, 1.4142135, 1.0000001, 1.5]]).astype(np.float32)
+    with np.errstate(over="ignore", under="ignore"):
+        for n in range(-150, 129):
+            n1 = int(n / 2)  # C division truncates toward zero
+            n2 = n - n1
+            s1 = np.float32(2.0) ** np.float32(n1)
+            s2 = np.float32(2.0) ** np.float32(n2)
+            two_step = (y * s1) * s2
+            one_step = np.ldexp(y, n).astype(np.float32)
+            assert two_step.dtype == np.float32
+            assert np.array_equal(two_step.view(np.uint32), one_step.view(np.uint32)), n
+
+
 def test_silu_against_float64(oracle):
     ts = _rng(11).normal(0, 4, 5000).astype(np.float32)
     got = np.array([oracle.silu(float(t)) for t in ts], np.float64)
