@@ -97,9 +97,10 @@ CAM_API camStatus camDestroyExecutor(camOpExecutor *executor);
 CAM_API const char *camGetVersion(void);
 
 /* How MoeDispatchPrefill and the fused layers launch the plan + permute of the dispatch (no counterpart in the
- * reference; the results are identical in every mode).  CAM_DISPATCH_LAUNCH_AUTO (default): one launch where it
- * is measured not to be slower than three -- 32768 <= T*K <= 524288 and T <= 4096 -- and MoeDispatchPlan's two
- * launches followed by MoeDispatchNormal's otherwise.  CAM_DISPATCH_LAUNCH_SINGLE: one launch whenever
+ * reference; the results are identical in every mode).  CAM_DISPATCH_LAUNCH_AUTO (default): MoeDispatchPrefill
+ * takes one launch where it is measured not to be slower than three -- 32768 <= T*K <= 524288 and T <= 4096 --
+ * and MoeDispatchPlan's launches followed by MoeDispatchNormal's otherwise; the fused layers always take the
+ * separate launches (their permute launch builds the GEMM schedules on the side).  CAM_DISPATCH_LAUNCH_SINGLE: one launch whenever
  * T*K <= 524288.  CAM_DISPATCH_LAUNCH_SEPARATE: never one launch.  The setting is process-wide and read by
  * phase 1 of those operators; returns CAM_ERR_RANGE for another value. */
 #define CAM_DISPATCH_LAUNCH_AUTO 0

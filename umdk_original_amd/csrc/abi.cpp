@@ -304,7 +304,10 @@ std::atomic<int32_t> g_dispatch_launch_mode{CAM_DISPATCH_LAUNCH_AUTO};
 // 4096 x 7168: 62.3 / 62.7, 8192 x 4096: 106.7 / 79.6, 8192 x 7168: 131.9 / 129.0; 128 tokens top-2: 12.0 / 9.2.
 // Below 32768 entries the hand-overs between workgroups cost more than two launches; above 4096 tokens the
 // workgroups beyond the first resident batch gain nothing from running under the plan.
-bool single_launch_dispatch(int64_t T, int64_t K)
+// In a fused layer the separate permute launch also builds the GEMM schedules in spare workgroups, which the
+// single launch cannot (the counts exist only when it ends) and which is worth 11-15 us: there the single launch
+// runs only when asked for.
+bool single_launch_dispatch(int64_t T, int64_t K, bool in_layer)
 {
     if (!cam::fused_dispatch_fits(T, K)) {
         return false;
@@ -313,7 +316,7 @@ bool single_launch_dispatch(int64_t T, int64_t K)
     if (mode == CAM_DISPATCH_LAUNCH_SINGLE) {
         return true;
     }
-    if (mode == CAM_DISPATCH_LAUNCH_SEPARATE) {
+    if (mode == CAM_DISPATCH_LAUNCH_SEPARATE || in_layer) {
         return false;
     }
     return T * K >= 32768 && T <= 4096;
@@ -901,7 +904,7 @@ camStatus camMoeDispatchPrefillGetWorkspaceSize(const camTensor *x, const camTen
     f.src_info = (int32_t *)expandIdx->data;
     f.src_rank = (int)rankId;
     Carver c;
-    if (single_launch_dispatch(T, K)) {
+    if (single_launch_dispatch(T, K, false)) {
         const uint64_t o_ctrl = c.take(cam::fused_dispatch_ctrl_bytes());
         const uint64_t o_table = c.take(cam::fused_dispatch_table_bytes(T, K, (int)numExperts));
         auto run = [f, o_ctrl, o_table](void *ws, hipStream_t s) mutable -> hipError_t {
@@ -1527,7 +1530,7 @@ camStatus camFusedDeepMoeGetWorkspaceSize(const camTensor *x, const camTensor *e
     const uint64_t o_meta = c.take(cam::kPlanMeta * 4);
     const uint64_t o_sched1 = c.take(cam::sched_bytes(A, (int)Epr, (int)(2 * I)));
     const uint64_t o_sched2 = c.take(cam::sched_bytes(A, (int)Epr, (int)H));
-    const bool fused_dispatch = single_launch_dispatch(T, K);
+    const bool fused_dispatch = single_launch_dispatch(T, K, true);
     const uint64_t o_hist = c.take(fused_dispatch ? cam::fused_dispatch_table_bytes(T, K, (int)Epr)
                                                   : cam::plan_workspace_bytes(T, K, (int)Epr));
     const uint64_t o_ctrl = c.take(cam::fused_dispatch_ctrl_bytes());
@@ -1910,7 +1913,7 @@ camStatus camFusedDeepMoeFp8GetWorkspaceSize(const camTensor *x, const camTensor
     const uint64_t o_meta = c.take(cam::kPlanMeta * 4);
     const uint64_t o_sched1 = c.take(cam::sched_bytes(A, (int)E, (int)(2 * I)));
     const uint64_t o_sched2 = c.take(cam::sched_bytes(A, (int)E, (int)H));
-    const bool fused_dispatch = single_launch_dispatch(T, K);
+    const bool fused_dispatch = single_launch_dispatch(T, K, true);
     const uint64_t o_hist = c.take(fused_dispatch ? cam::fused_dispatch_table_bytes(T, K, (int)E)
                                                   : cam::plan_workspace_bytes(T, K, (int)E));
     const uint64_t o_ctrl = c.take(cam::fused_dispatch_ctrl_bytes());
