@@ -97,12 +97,12 @@ CAM_API camStatus camDestroyExecutor(camOpExecutor *executor);
 CAM_API const char *camGetVersion(void);
 
 /* How MoeDispatchPrefill and the fused layers launch the plan + permute of the dispatch (no counterpart in the
- * reference; the results are identical in every mode).  CAM_DISPATCH_LAUNCH_AUTO (default): MoeDispatchPrefill
- * takes one launch where it is measured not to be slower than three -- 32768 <= T*K <= 524288 and T <= 4096 --
- * and MoeDispatchPlan's launches followed by MoeDispatchNormal's otherwise; the fused layers always take the
- * separate launches (their permute launch builds the GEMM schedules on the side).  CAM_DISPATCH_LAUNCH_SINGLE: one launch whenever
- * T*K <= 524288.  CAM_DISPATCH_LAUNCH_SEPARATE: never one launch.  The setting is process-wide and read by
- * phase 1 of those operators; returns CAM_ERR_RANGE for another value. */
+ * reference; the results are identical in every mode).  CAM_DISPATCH_LAUNCH_AUTO (default) and
+ * CAM_DISPATCH_LAUNCH_SEPARATE: MoeDispatchPlan's launches followed by MoeDispatchNormal's, the faster form at
+ * every measured size (in a fused layer the permute launch also builds the GEMM schedules).
+ * CAM_DISPATCH_LAUNCH_SINGLE: plan, permute and quantisation as ONE launch whenever T*K <= 524288 (one graph node,
+ * no intermediate launch boundaries; 3-30 % slower).  The setting is process-wide and read by phase 1 of those
+ * operators; returns CAM_ERR_RANGE for another value. */
 #define CAM_DISPATCH_LAUNCH_AUTO 0
 #define CAM_DISPATCH_LAUNCH_SINGLE 1
 #define CAM_DISPATCH_LAUNCH_SEPARATE 2
@@ -213,9 +213,10 @@ CAM_API camStatus camMoeDispatchNormal(void *workspace, uint64_t workspaceSize, 
 /* ------------------------------------------------------------------------------------------------
  * MoeDispatchPrefill -- the whole body of the reference's binding-level operator moe_dispatch_prefill
  * (src/cam/comm_operator/pybind/moe_dispatch_prefill.cpp:96-192: the CPU ranking loop, the CPU loop over the
- * exchanged counts, two device-to-host copies and the aclnnMoeDispatchNormal call) as ONE kernel launch for
- * one rank: MoeDispatchPlan and MoeDispatchNormal fused, with the plan running underneath the first row
- * loads.  x bf16/fp16 [T,H]; topkIdx int64/int32 [T,K] -> recvX [A,H] (int8 when quantMode is 2 or 3, else
+ * exchanged counts, two device-to-host copies and the aclnnMoeDispatchNormal call) as one operator with no host
+ * round trip for one rank: MoeDispatchPlan and MoeDispatchNormal back to back on the stream (or, on request, as
+ * ONE kernel launch with the plan running underneath the first row loads).
+ * x bf16/fp16 [T,H]; topkIdx int64/int32 [T,K] -> recvX [A,H] (int8 when quantMode is 2 or 3, else
  * x's dtype), recvXScalesOptional fp32 [A] (required when quantising); quantMode 4, which the reference does
  * not have, gives block-scaled FP8 rows instead (recvX E4M3 [A,H], recvXScales uint8 [A,H/128], cam_fp8_spec.h);
  * expandIdx int32 [3A] = (srcRank,

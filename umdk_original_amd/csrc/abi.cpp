@@ -299,27 +299,17 @@ cam::SchedSpec sched_spec(int64_t rows, int64_t G, int64_t N)
 
 std::atomic<int32_t> g_dispatch_launch_mode{CAM_DISPATCH_LAUNCH_AUTO};
 
-// One launch for plan + permute, or the plan's two launches and then the permute's.  Measured (int8 rows,
-// 256 experts, top-8, microseconds single / separate): 2048 x 7168: 40.1 / 34.1, 4096 x 4096: 40.0 / 41.2,
-// 4096 x 7168: 62.3 / 62.7, 8192 x 4096: 106.7 / 79.6, 8192 x 7168: 131.9 / 129.0; 128 tokens top-2: 12.0 / 9.2.
-// Below 32768 entries the hand-overs between workgroups cost more than two launches; above 4096 tokens the
-// workgroups beyond the first resident batch gain nothing from running under the plan.
-// In a fused layer the separate permute launch also builds the GEMM schedules in spare workgroups, which the
-// single launch cannot (the counts exist only when it ends) and which is worth 11-15 us: there the single launch
-// runs only when asked for.
-bool single_launch_dispatch(int64_t T, int64_t K, bool in_layer)
+// One launch for plan + permute (dispatch_fused.hip), or the plan's launches and then the permute's.  Measured
+// (int8 rows, top-8, microseconds single / separate): 1024 x 7168: 24.1 / 20.9, 2048 x 7168: 39.7 / 33.4,
+// 4096 x 4096: 40.2 / 38.3, 4096 x 7168: 61.0 / 59.4, 8192 x 4096: 105.7 / 77.4, 8192 x 7168: 132.6 / 126.8.  The
+// single launch saves two launch latencies but its token workgroups sit idle until the ranking is through and
+// read the hand-over tables past the L2; since the permute keeps four workgroups per CU resident the separate
+// form is ahead at every size, and in a fused layer its permute launch also builds the GEMM schedules.  The
+// single launch therefore runs only when it is asked for.
+bool single_launch_dispatch(int64_t T, int64_t K)
 {
-    if (!cam::fused_dispatch_fits(T, K)) {
-        return false;
-    }
-    const int32_t mode = g_dispatch_launch_mode.load(std::memory_order_relaxed);
-    if (mode == CAM_DISPATCH_LAUNCH_SINGLE) {
-        return true;
-    }
-    if (mode == CAM_DISPATCH_LAUNCH_SEPARATE || in_layer) {
-        return false;
-    }
-    return T * K >= 32768 && T <= 4096;
+    return g_dispatch_launch_mode.load(std::memory_order_relaxed) == CAM_DISPATCH_LAUNCH_SINGLE &&
+           cam::fused_dispatch_fits(T, K);
 }
 
 }  // namespace
@@ -904,7 +894,7 @@ camStatus camMoeDispatchPrefillGetWorkspaceSize(const camTensor *x, const camTen
     f.src_info = (int32_t *)expandIdx->data;
     f.src_rank = (int)rankId;
     Carver c;
-    if (single_launch_dispatch(T, K, false)) {
+    if (single_launch_dispatch(T, K)) {
         const uint64_t o_ctrl = c.take(cam::fused_dispatch_ctrl_bytes());
         const uint64_t o_table = c.take(cam::fused_dispatch_table_bytes(T, K, (int)numExperts));
         auto run = [f, o_ctrl, o_table](void *ws, hipStream_t s) mutable -> hipError_t {
@@ -1530,7 +1520,7 @@ camStatus camFusedDeepMoeGetWorkspaceSize(const camTensor *x, const camTensor *e
     const uint64_t o_meta = c.take(cam::kPlanMeta * 4);
     const uint64_t o_sched1 = c.take(cam::sched_bytes(A, (int)Epr, (int)(2 * I)));
     const uint64_t o_sched2 = c.take(cam::sched_bytes(A, (int)Epr, (int)H));
-    const bool fused_dispatch = single_launch_dispatch(T, K, true);
+    const bool fused_dispatch = single_launch_dispatch(T, K);
     const uint64_t o_hist = c.take(fused_dispatch ? cam::fused_dispatch_table_bytes(T, K, (int)Epr)
                                                   : cam::plan_workspace_bytes(T, K, (int)Epr));
     const uint64_t o_ctrl = c.take(cam::fused_dispatch_ctrl_bytes());
@@ -1913,7 +1903,7 @@ camStatus camFusedDeepMoeFp8GetWorkspaceSize(const camTensor *x, const camTensor
     const uint64_t o_meta = c.take(cam::kPlanMeta * 4);
     const uint64_t o_sched1 = c.take(cam::sched_bytes(A, (int)E, (int)(2 * I)));
     const uint64_t o_sched2 = c.take(cam::sched_bytes(A, (int)E, (int)H));
-    const bool fused_dispatch = single_launch_dispatch(T, K, true);
+    const bool fused_dispatch = single_launch_dispatch(T, K);
     const uint64_t o_hist = c.take(fused_dispatch ? cam::fused_dispatch_table_bytes(T, K, (int)E)
                                                   : cam::plan_workspace_bytes(T, K, (int)E));
     const uint64_t o_ctrl = c.take(cam::fused_dispatch_ctrl_bytes());

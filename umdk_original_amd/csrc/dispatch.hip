@@ -39,8 +39,10 @@ __device__ __forceinline__ long long dispatch_row(const DispatchArgs &a, int t, 
     return pre + (window_row - a.recv_offset[e]);
 }
 
+// Four workgroups per CU (128 registers a lane) keep all 1024 workgroups of a 4096-token batch resident at once;
+// the FP8 variant would spill at that size and stays at three.
 template <int QUANT, int ACT>
-__global__ __launch_bounds__(kDispWaves * kWave) void dispatch_kernel(DispatchArgs a)
+__global__ __launch_bounds__(kDispWaves * kWave, QUANT == 3 ? 3 : 4) void dispatch_kernel(DispatchArgs a)
 {
     // The first workgroups of the launch build the GEMM schedules (they start first and finish under the row
     // traffic of the others); they depend on nothing this launch writes.
