@@ -140,6 +140,16 @@ __device__ __forceinline__ void quant_token_row(TokenRow &r)
         }
     }
     m = wave_max(m);
+    // Keep the row as its 16-bit words across the two passes: left alone, the compiler holds the 112 converted
+    // floats of the maximum pass for the scaling pass (a shift each to redo) and the kernel needs a third more
+    // registers.
+#pragma unroll
+    for (int j = 0; j < kDispMaxChunks; ++j) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            asm volatile("" : "+v"(r.raw[j][i]));
+        }
+    }
     float s;
     bool zero_row = false;
     if (QUANT == 1) {
