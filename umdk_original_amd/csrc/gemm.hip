@@ -92,15 +92,6 @@ __device__ __forceinline__ void dma16_stream(const void *base, unsigned voff, un
                  : "memory", "m0");
 }
 
-// Four bytes per lane, straight to LDS: lane i's word lands at lds_addr + 4*i.
-__device__ __forceinline__ void dma4(const void *base, unsigned voff, unsigned lds_addr)
-{
-    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, %2"
-                 :
-                 : "s"(lds_addr), "v"(voff), "s"((unsigned long long)base)
-                 : "memory", "m0");
-}
-
 #ifndef CAM_TALL_WEIGHTS_STREAM
 #define CAM_TALL_WEIGHTS_STREAM 0
 #endif
@@ -132,32 +123,11 @@ struct ItemCtx {
     int m0, rows;           // first row and rows of the tile
     int a_row0, my_rows;    // first tile row of this wave's fragments, rows of them that exist
     int bslot;              // this wave's 64-column group inside the stage
+    int nw;                 // this wave's packed 64-column group of the weight (clamped to a valid one)
+    bool wave_live;         // the group exists (ragged last column block)
     int stage_a, stage_bytes;
     int Kd, N;
 };
-
-// Requests the per-channel weight scales of column block nbc of the item's expert into LDS (int8 items), one
-// word per thread of the first 64 * groups threads: entry 64 * slot + c for the plain column order, and
-// 32 * slot + c (gate) / 32 * groups + 32 * slot + c (up) for the paired order, slot = position of the 64-column
-// group in the block.  The epilogue then starts without a round trip to memory, and because the request is older
-// than the block's weight loads, the waits of the K loop cover it.
-__device__ __forceinline__ void issue_col_scales(const GemmArgs &a, const ItemCtx &t, int nbc, bool flat, float *dst_s)
-{
-    const int tid = threadIdx.x;
-    const int ngr = flat ? 8 : 4;
-    if (tid < ngr * 64) {
-        int col;
-        if (a.gate_up) {
-            const int half = tid >= ngr * 32 ? 1 : 0;
-            col = half * (a.N / 2) + min(nbc * ngr * 32 + (tid - half * ngr * 32), a.N / 2 - 1);
-        } else {
-            col = min(nbc * ngr * 64 + tid, a.N - 1);
-        }
-        const unsigned dst = (unsigned)(unsigned long long)(__attribute__((address_space(3))) float *)dst_s +
-                             (unsigned)__builtin_amdgcn_readfirstlane(tid & ~63) * 4u;
-        dma4(t.sg, (unsigned)col * 4u, dst);
-    }
-}
 
 // One wave's part of one item.  TEAM 0 multiplies in the first phase of every sub-step, TEAM 1 in the second.
 // FLAT selects the tile shape (it fixes the loads per wave and sub-step); MF is the wave's fragment count.
@@ -179,8 +149,8 @@ struct AccType<true> {
 // scales of the item wait in LDS (a_scale8_s[kb * 256 + tile row], w_scale8_s[column group * kScaleKb + kb]) and
 // are read with the fragments.
 template <int MF, int TEAM, bool FLAT, bool FP8>
-__device__ __forceinline__ void run_item(const GemmArgs &a, const ItemCtx &t, int nb, int nblk, int8_t *lds,
-                                         float *row_scale_s, const uint8_t *a_scale8_s,
+__device__ __forceinline__ void run_item(const GemmArgs &a, const ItemCtx &t, int nb, int8_t *lds,
+                                         const float *row_scale_s, const uint8_t *a_scale8_s,
                                          const uint8_t *w_scale8_s)
 {
     constexpr int NS = FLAT ? 3 : 4;                       // ring of stages
@@ -194,18 +164,16 @@ __device__ __forceinline__ void run_item(const GemmArgs &a, const ItemCtx &t, in
     const unsigned lds0 = (unsigned)(unsigned long long)(__attribute__((address_space(3))) int8_t *)lds;
 
     typename AccType<FP8>::type acc[MFR][2];
-    auto clear_acc = [&]() {
 #pragma unroll
-        for (int mf = 0; mf < MFR; ++mf) {
+    for (int mf = 0; mf < MFR; ++mf) {
 #pragma unroll
-            for (int nf = 0; nf < 2; ++nf) {
+        for (int nf = 0; nf < 2; ++nf) {
 #pragma unroll
-                for (int i = 0; i < 16; ++i) {
-                    acc[mf][nf][i] = 0;
-                }
+            for (int i = 0; i < 16; ++i) {
+                acc[mf][nf][i] = 0;
             }
         }
-    };
+    }
 
     // ---- loads.  Tall: team 0 brings the activations (wave wn: tile rows 64wn .. 64wn+63, four loads of 16
     // rows), team 1 the weights (wave wn: the 4 KB of column group wn).  Flat: team 0 brings the activations
@@ -226,24 +194,12 @@ __device__ __forceinline__ void run_item(const GemmArgs &a, const ItemCtx &t, in
     }
     const int ngroups = t.N / 64;
     const int bgroup = FLAT ? TEAM * 4 + wn : wn;  // the column group of the stage this wave loads
-    // What depends on the column block.  A flat item may cover several consecutive column blocks of its expert
-    // (nblk > 1): same activation rows, next weight panel.
-    int nw = 0;              // this wave's packed 64-column group of the weight (clamped to a valid one)
-    bool wave_live = false;  // the group exists (ragged last column block)
-    int b_step = 0;
-    const int8_t *b_base = nullptr;
-    auto set_block = [&](int nbc) {
-        const int group = nbc * (FLAT ? 8 : 4) + t.bslot;
-        wave_live = group < ngroups;
-        nw = min(group, ngroups - 1);
-        const int nw_load = min(nbc * (FLAT ? 8 : 4) + bgroup, ngroups - 1);
-        // Packed weights: column groups in blocks of eight; inside a block the 4 KB of a K step of its groups lie
-        // side by side, so the loads of one step of a workgroup cover one contiguous stretch of memory.
-        const int b_block = nw_load >> 3;
-        b_step = min(8, ngroups - 8 * b_block) * 4096;
-        b_base = t.wg + (long long)b_block * 8 * t.Kd * 64 + (nw_load & 7) * 4096;
-    };
-    set_block(nb);
+    const int nw_load = min(nb * (FLAT ? 8 : 4) + bgroup, ngroups - 1);
+    // Packed weights: column groups in blocks of eight; inside a block the 4 KB of a K step of its groups lie
+    // side by side, so the loads of one step of a workgroup cover one contiguous stretch of memory.
+    const int b_block = nw_load >> 3;
+    const int b_step = min(8, ngroups - 8 * b_block) * 4096;
+    const int8_t *b_base = t.wg + (long long)b_block * 8 * t.Kd * 64 + (nw_load & 7) * 4096;
     const unsigned b_voff = (unsigned)(lane * 16);
     const unsigned b_dst = (unsigned)(t.stage_a + bgroup * 4096);
 
@@ -344,18 +300,11 @@ __device__ __forceinline__ void run_item(const GemmArgs &a, const ItemCtx &t, in
     for (int p = 0; p < NS; ++p) {
         issue(p, p);
     }
-    // Stage s of a column block lies in slot (base + s) % NS.  The first block starts at slot 0; a following block
-    // has its first NS-1 stages fetched into slots 1 .. NS-1 while the previous block's epilogue stages its
-    // results through slot 0, and starts at slot 1.
-    int base = 0;
-    const int nblocks = FLAT ? nblk : 1;
-    for (int blk = 0; blk < nblocks; ++blk) {
-    clear_acc();
     wait_loads_outstanding<(NS - 1) * LPS>();
     barrier_no_fence();  // stage 0 has landed
-    int slot = base;     // slot of stage s
+    int slot = 0;        // slot of stage s
     if (TEAM == 0) {
-        read_frags(base, 0);
+        read_frags(0, 0);
         wait_lds_reads();
         for (int s = 0; s < KT; ++s) {
             const int next = slot + 1 == NS ? 0 : slot + 1;
@@ -390,19 +339,14 @@ __device__ __forceinline__ void run_item(const GemmArgs &a, const ItemCtx &t, in
     // per lane and fragment and the column scales fetched as 16-byte vectors.  To store whole 128-byte lines,
     // every wave passes one fragment at a time through its own slice of LDS: 128 staged bytes per row, then
     // 16 bytes per lane and 8 rows per store instruction.
-    // The rows an epilogue writes are the same for every column block of the item; an opaque copy of their first
-    // index keeps the compiler from computing all the store addresses once, ahead of the K loops, and holding them
-    // in registers it does not have.
-    int out_row0 = t.m0 + t.a_row0;
-    asm volatile("" : "+s"(out_row0));
-    auto epilogue = [&](int enw, bool elive, const float *wsc) {
-    if (MF > 0 && elive) {
+    auto epilogue = [&]() {
+    if (MF > 0 && t.wave_live) {
         const int wave = tid >> 6;
         const int row_in = lane & 31;
         const int col_half = (lane >> 5) * 4;
         int8_t *slice = lds + wave * kEpiSlice;
         const int N = t.N;
-        const int nw = enw;
+        const int nw = t.nw;
 
         // Copies rows [0, 32) of the slice (128 bytes each) to dst + (first + row) * row_pitch_bytes.
         auto flush_fragment = [&](int8_t *dst, long long row_pitch_bytes, int mf) {
@@ -414,7 +358,7 @@ __device__ __forceinline__ void run_item(const GemmArgs &a, const ItemCtx &t, in
                 const v4u v = *(const v4u *)(slice + row * kEpiRowBytes + piece * 16);
                 const int trow = mf * 32 + row;
                 if (trow < t.my_rows) {
-                    *(v4u *)(dst + (long long)(out_row0 + trow) * row_pitch_bytes + piece * 16) = v;
+                    *(v4u *)(dst + (long long)(t.m0 + t.a_row0 + trow) * row_pitch_bytes + piece * 16) = v;
                 }
             }
         };
@@ -442,8 +386,8 @@ __device__ __forceinline__ void run_item(const GemmArgs &a, const ItemCtx &t, in
             if (!FP8) {
 #pragma unroll
                 for (int j = 0; j < 4; ++j) {
-                    sg_gate[j] = *(const v4f *)(wsc + t.bslot * 32 + 8 * j + col_half);
-                    sg_up[j] = *(const v4f *)(wsc + (FLAT ? 8 : 4) * 32 + t.bslot * 32 + 8 * j + col_half);
+                    sg_gate[j] = *(const v4f *)(t.sg + nw * 32 + 8 * j + col_half);
+                    sg_up[j] = *(const v4f *)(t.sg + I + nw * 32 + 8 * j + col_half);
                 }
             }
 #pragma unroll
@@ -475,7 +419,7 @@ __device__ __forceinline__ void run_item(const GemmArgs &a, const ItemCtx &t, in
                 for (int nf = 0; nf < 2; ++nf) {
 #pragma unroll
                     for (int j = 0; j < 4; ++j) {
-                        ws[nf][j] = *(const v4f *)(wsc + t.bslot * 64 + nf * 32 + 8 * j + col_half);
+                        ws[nf][j] = *(const v4f *)(t.sg + nw * 64 + nf * 32 + 8 * j + col_half);
                     }
                 }
             }
@@ -511,7 +455,7 @@ __device__ __forceinline__ void run_item(const GemmArgs &a, const ItemCtx &t, in
     // 128 product columns is exactly what the four waves of a team hold for their rows (32 columns each), so the
     // block maximum needs one exchange through LDS; every wave of the workgroup takes part in its barrier.
     auto epilogue_quant = [&]() {
-        const bool work = MF > 0 && wave_live;
+        const bool work = MF > 0 && t.wave_live;
         const int wave = tid >> 6;
         const int row_in = lane & 31;
         const int col_half = (lane >> 5) * 4;
@@ -558,58 +502,37 @@ __device__ __forceinline__ void run_item(const GemmArgs &a, const ItemCtx &t, in
                     const int row = lane >> 1, piece = lane & 1;
                     const v4u v = *(const v4u *)(slice + row * 48 + piece * 16);
                     if (mf * 32 + row < t.my_rows) {
-                        const long long grow = out_row0 + mf * 32 + row;
-                        *(v4u *)(q + grow * I + nw * 32 + piece * 16) = v;
+                        const long long grow = t.m0 + t.a_row0 + mf * 32 + row;
+                        *(v4u *)(q + grow * I + t.nw * 32 + piece * 16) = v;
                     }
                     if ((wave & 3) == 0 && lane < 32 && mf * 32 + lane < t.my_rows) {
-                        const long long grow = out_row0 + mf * 32 + lane;
-                        a.out_scale8[grow * (I >> 7) + (nw >> 2)] = (uint8_t)(ex + 127);
+                        const long long grow = t.m0 + t.a_row0 + mf * 32 + lane;
+                        a.out_scale8[grow * (I >> 7) + (t.nw >> 2)] = (uint8_t)(ex + 127);
                     }
                 }
             }
         }
     };
 
-    // A following column block of the same item: request its first NS-1 stages now, into the slots the staging
-    // of the epilogue does not touch (it uses the first 40 KB: slot 0 of a flat ring), so that they travel
-    // while the epilogue runs.
-    const int epi_nw = nw;
-    const bool epi_live = wave_live;
-    const bool more = FLAT && blk + 1 < nblocks;
-    if (more) {
-        set_block(nb + blk + 1);
-        if (!FP8 && a.epilogue != kEpiInt32) {
-            issue_col_scales(a, t, nb + blk + 1, true, row_scale_s + 256 + ((blk + 1) & 1) * 512);
-        }
-#pragma unroll
-        for (int p = 0; p < NS - 1; ++p) {
-            issue(p, 1 + p);
-        }
-    }
     if (FP8 && a.epilogue == kEpiSwigluFp8) {
         epilogue_quant();
     } else {
-        epilogue(epi_nw, epi_live, row_scale_s + 256 + (blk & 1) * 512);
+        epilogue();
     }
-    barrier_no_fence();  // the staging slices are free again before the next loads into them land
-    if (more) {
-        issue(NS - 1, 0);
-        base = 1;
-    }
-    }  // column blocks of the item
+    barrier_no_fence();  // the staging slices are free again before the next item's loads land
 }
 
 template <int TEAM, bool FLAT, bool FP8>
-__device__ __forceinline__ void run_item_mf(int mf, const GemmArgs &a, const ItemCtx &t, int nb, int nblk, int8_t *lds,
-                                            float *row_scale_s, const uint8_t *a_scale8_s,
+__device__ __forceinline__ void run_item_mf(int mf, const GemmArgs &a, const ItemCtx &t, int nb, int8_t *lds,
+                                            const float *row_scale_s, const uint8_t *a_scale8_s,
                                             const uint8_t *w_scale8_s)
 {
     switch (mf) {
-        case 0: run_item<0, TEAM, FLAT, FP8>(a, t, nb, nblk, lds, row_scale_s, a_scale8_s, w_scale8_s); break;
-        case 1: run_item<1, TEAM, FLAT, FP8>(a, t, nb, nblk, lds, row_scale_s, a_scale8_s, w_scale8_s); break;
-        case 2: run_item<2, TEAM, FLAT, FP8>(a, t, nb, nblk, lds, row_scale_s, a_scale8_s, w_scale8_s); break;
-        case 3: run_item<3, TEAM, FLAT, FP8>(a, t, nb, nblk, lds, row_scale_s, a_scale8_s, w_scale8_s); break;
-        default: run_item<4, TEAM, FLAT, FP8>(a, t, nb, nblk, lds, row_scale_s, a_scale8_s, w_scale8_s); break;
+        case 0: run_item<0, TEAM, FLAT, FP8>(a, t, nb, lds, row_scale_s, a_scale8_s, w_scale8_s); break;
+        case 1: run_item<1, TEAM, FLAT, FP8>(a, t, nb, lds, row_scale_s, a_scale8_s, w_scale8_s); break;
+        case 2: run_item<2, TEAM, FLAT, FP8>(a, t, nb, lds, row_scale_s, a_scale8_s, w_scale8_s); break;
+        case 3: run_item<3, TEAM, FLAT, FP8>(a, t, nb, lds, row_scale_s, a_scale8_s, w_scale8_s); break;
+        default: run_item<4, TEAM, FLAT, FP8>(a, t, nb, lds, row_scale_s, a_scale8_s, w_scale8_s); break;
     }
 }
 
@@ -617,8 +540,7 @@ template <bool FP8>
 __global__ __launch_bounds__(kThreads, 1) void gemm_kernel(GemmArgs a)
 {
     __shared__ __attribute__((aligned(1024))) int8_t lds[kLdsBytes];
-    // activation row scales of the item, then two buffers of weight column scales (column blocks alternate)
-    __shared__ __attribute__((aligned(16))) float row_scale_s[256 + 2 * 512];
+    __shared__ float row_scale_s[256];
     __shared__ uint8_t a_scale8_s[FP8 ? kScaleKb * 256 : 4];
     __shared__ uint8_t w_scale8_s[FP8 ? 16 * kScaleKb : 4];
     __shared__ int item_s;
@@ -696,7 +618,6 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_kernel(GemmArgs a)
         const int split = __builtin_amdgcn_readfirstlane(it.split);
         const int nb = __builtin_amdgcn_readfirstlane(it.nb);
         const bool flat = __builtin_amdgcn_readfirstlane(it.flat) != 0;
-        const int nblk = flat && !FP8 ? max(1, __builtin_amdgcn_readfirstlane(it.pad0)) : 1;  // column blocks of the item
 
         ItemCtx t;
         t.Kd = a.Kd;
@@ -719,6 +640,9 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_kernel(GemmArgs a)
             t.stage_a = 256 * kBK;
             t.stage_bytes = kStageTall;
         }
+        const int group = nb * (flat ? 8 : 4) + t.bslot;
+        t.wave_live = group < a.N / 64;
+        t.nw = min(group, a.N / 64 - 1);
         if (FP8) {
             // the item's scales: activation rows x K blocks (transposed, so that the lanes of a fragment read
             // neighbouring bytes), and one row of K blocks per 64-column group of the item
@@ -737,26 +661,23 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_kernel(GemmArgs a)
                 const int col = a.gate_up ? nf * (a.N / 2) + grp * 32 : grp * 64 + nf * 32;
                 w_scale8_s[gf * kScaleKb + kb] = a.w_scale8[((long long)g * KB + kb) * nblk + (col >> 7)];
             }
-        } else if (a.epilogue != kEpiInt32) {
-            issue_col_scales(a, t, nb, flat, row_scale_s + 256);
-            if (tid < 256) {
-                row_scale_s[tid] = a.a_scale[m0 + min(tid, rows - 1)];
-            }
+        } else if (a.epilogue != kEpiInt32 && tid < 256) {
+            row_scale_s[tid] = a.a_scale[m0 + min(tid, rows - 1)];
         }
         __syncthreads();  // item_s may be rewritten and the row scales read from here on
 
         const int mf = t.my_rows <= 0 ? 0 : (t.my_rows + 31) >> 5;
         if (flat) {
             if (team == 0) {
-                run_item_mf<0, true, FP8>(mf, a, t, nb, nblk, lds, row_scale_s, a_scale8_s, w_scale8_s);
+                run_item_mf<0, true, FP8>(mf, a, t, nb, lds, row_scale_s, a_scale8_s, w_scale8_s);
             } else {
-                run_item_mf<1, true, FP8>(mf, a, t, nb, nblk, lds, row_scale_s, a_scale8_s, w_scale8_s);
+                run_item_mf<1, true, FP8>(mf, a, t, nb, lds, row_scale_s, a_scale8_s, w_scale8_s);
             }
         } else {
             if (team == 0) {
-                run_item_mf<0, false, FP8>(mf, a, t, nb, nblk, lds, row_scale_s, a_scale8_s, w_scale8_s);
+                run_item_mf<0, false, FP8>(mf, a, t, nb, lds, row_scale_s, a_scale8_s, w_scale8_s);
             } else {
-                run_item_mf<1, false, FP8>(mf, a, t, nb, nblk, lds, row_scale_s, a_scale8_s, w_scale8_s);
+                run_item_mf<1, false, FP8>(mf, a, t, nb, lds, row_scale_s, a_scale8_s, w_scale8_s);
             }
         }
         if (tid == 0) {
