@@ -693,47 +693,46 @@ __global__ __launch_bounds__(1024) void build_sched_kernel(SchedBuild sb)
 }
 
 // SwiGLU product rows (fp32) -> int8 rows + per-row scale:
-//   m = max|y|; y_scale = m * (1/127); q = rint((y * 127) * (1/m)).   One workgroup per row.
+//   m = max|y|; y_scale = m * (1/127); q = rint((y * 127) * (1/m)).   One wave per row (four rows per workgroup):
+// the row waits in registers between the maximum and the scaling, the maximum needs wave shuffles only, and no
+// wave waits for another.
 __global__ __launch_bounds__(256) void requant_kernel(const float *__restrict__ y, int I,
                                                       const int32_t *__restrict__ sched, long long max_rows,
                                                       int8_t *__restrict__ q, float *__restrict__ scale)
 {
-    __shared__ float wave_max_s[4];
-    const long long row = blockIdx.x;
+    const long long row = (long long)blockIdx.x * 4 + (threadIdx.x >> 6);
     const long long valid = sched != nullptr ? min((long long)sched[1], max_rows) : max_rows;
     if (row >= valid) {
         return;
     }
-    const int tid = threadIdx.x;
+    const int lane = threadIdx.x & (kWave - 1);
     const int n4 = I >> 2;
-    constexpr int kMaxPer = 4;  // I <= 4096
+    constexpr int kMaxPer = 16;  // I <= 4096
     v4f v[kMaxPer];
     float m = 0.0f;
     const v4f *src = (const v4f *)(y + row * I);
 #pragma unroll
     for (int j = 0; j < kMaxPer; ++j) {
-        const int c = tid + j * 256;
+        const int c = lane + j * kWave;
         v[j] = v4f{0.f, 0.f, 0.f, 0.f};
         if (c < n4) {
             v[j] = __builtin_nontemporal_load(src + c);
-            m = fmaxf(m, fmaxf(fmaxf(fabsf(v[j][0]), fabsf(v[j][1])), fmaxf(fabsf(v[j][2]), fabsf(v[j][3]))));
         }
     }
-    m = wave_max(m);
-    if ((tid & 63) == 0) {
-        wave_max_s[tid >> 6] = m;
+#pragma unroll
+    for (int j = 0; j < kMaxPer; ++j) {
+        m = fmaxf(m, fmaxf(fmaxf(fabsf(v[j][0]), fabsf(v[j][1])), fmaxf(fabsf(v[j][2]), fabsf(v[j][3]))));
     }
-    __syncthreads();
-    m = fmaxf(fmaxf(wave_max_s[0], wave_max_s[1]), fmaxf(wave_max_s[2], wave_max_s[3]));
+    m = wave_max(m);
     const bool zero_row = m == 0.0f;
     const float rcp = zero_row ? 0.0f : __fdiv_rn(1.0f, m);
-    if (tid == 0) {
+    if (lane == 0) {
         scale[row] = zero_row ? 0.0f : __fmul_rn(m, 1.0f / 127.0f);
     }
     uint32_t *dst = (uint32_t *)(q + row * I);
 #pragma unroll
     for (int j = 0; j < kMaxPer; ++j) {
-        const int c = tid + j * 256;
+        const int c = lane + j * kWave;
         if (c < n4) {
             int b[4];
 #pragma unroll
@@ -939,7 +938,7 @@ hipError_t launch_requant(const float *y, int64_t max_rows, int I, const int32_t
     if (I % 4 != 0 || I > 4096) {
         return hipErrorInvalidValue;
     }
-    hipLaunchKernelGGL(requant_kernel, dim3((unsigned)max_rows), dim3(256), 0, stream, y, I, sched_for_rows,
+    hipLaunchKernelGGL(requant_kernel, dim3((unsigned)((max_rows + 3) / 4)), dim3(256), 0, stream, y, I, sched_for_rows,
                        (long long)max_rows, q, scale);
     return hipGetLastError();
 }
