@@ -94,7 +94,9 @@ hipError_t launch_dispatch(const DispatchArgs &a_in, hipStream_t stream)
             a.sched.group_list == nullptr) {
             return hipErrorInvalidValue;
         }
+        // Few builders: every one repeats the per-expert tables, and the row traffic hides them anyway.
         a.sched_parts = sched_build_parts(a.sched);
+        a.sched_parts = a.sched_parts > 8 ? 8 : a.sched_parts;
     }
     dim3 grid((a.T + kDispWaves - 1) / kDispWaves + a.sched.nspec * a.sched_parts), block(kDispWaves * kWave);
     if (a.quant == 0) {
