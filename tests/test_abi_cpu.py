@@ -360,3 +360,16 @@ def test_dispatch_launch_mode_setter_range():
         assert h.camSetDispatchLaunchMode(mode) == 0
     assert h.camSetDispatchLaunchMode(3) != 0 and "mode" in _lib.recent_error()
     assert h.camSetDispatchLaunchMode(-1) != 0
+
+
+def test_torch_operator_library_is_built_and_registers_the_reference_schemas():
+    import os
+    from umdk_original_amd import ops
+    path = os.path.join(os.path.dirname(_lib.LIB_PATH), "libcam_torch_ops.so")
+    assert os.path.exists(path), "python -m umdk_original_amd.build builds it"
+    assert ops._torch_lib == "cpp"
+    for name in ("fused_deep_moe", "get_dispatch_layout", "moe_dispatch_prefill", "moe_combine_prefill",
+                 "prepack_weight"):
+        assert hasattr(torch.ops.umdk_cam_op_lib, name)
+    s = str(torch.ops.umdk_cam_op_lib.moe_combine_prefill.default._schema)
+    assert "Tensor send_head, str group_ep, int rank, int num_ranks" in s

@@ -114,3 +114,33 @@ def test_fused_layer_fp16_activations(gpu, oracle, dispatch_launch):
                                         w1.numpy(), w1s.numpy(), w2.numpy(), w2s.numpy())
     assert_bits_equal(to_np(etn), cnt.astype(np.int64), "expert_token_nums")
     assert_bits_equal(out.cpu().view(torch.int16).numpy().view(np.uint16), want, "fp16 layer output")
+
+
+def test_torch_ops_are_the_cpp_library_and_check_the_weight_mark(gpu, oracle):
+    """torch.ops.umdk_cam_op_lib.* come from the C++ operator library (csrc/torch_binding.cpp): a view of a packed
+    weight is accepted, a clone() of one (packed bytes without the mark) and a plain row-major weight are refused."""
+    from umdk_original_amd import ops
+    assert ops._torch_lib == "cpp"
+    announce("torch ops through the C++ library")
+    T, H, E, K, I = 64, 1024, 8, 2, 512
+    ids, gates = synth.softmax_topk_routing(T, E, K, seed=91)
+    w1, w1s = synth.absmax_int8_weights(E, H, 2 * I, seed=911)
+    w2, w2s = synth.absmax_int8_weights(E, I, H, seed=912)
+    x = synth.normal_bf16(T, H, seed=913)
+    w1p = torch.ops.umdk_cam_op_lib.prepack_weight(w1.to(gpu), True)
+    w2p = torch.ops.umdk_cam_op_lib.prepack_weight(w2.to(gpu), False)
+    args = lambda a, b: (x.to(gpu), ids.to(torch.int32).to(gpu), [a], [w1s.to(gpu)], [b], [w2s.to(gpu)],
+                         gates.to(gpu), None, None, "", 1, 0, E, 1, 0, 0, 0)
+    out, etn = torch.ops.umdk_cam_op_lib.fused_deep_moe(*args(w1p, w2p))
+    want, cnt = oracle.fused_layer(synth.bf16_bits(x), ids.numpy().astype(np.int64), gates.numpy(), w1.numpy(),
+                                   w1s.numpy(), w2.numpy(), w2s.numpy())
+    assert_bits_equal(to_np(etn), cnt, "expert_token_nums")
+    assert_bits_equal(to_np(out), want, "layer output through the C++ operator library")
+    out2, _ = torch.ops.umdk_cam_op_lib.fused_deep_moe(*args(w1p.view(E, H, 2 * I), w2p[:]))   # views keep the mark
+    assert torch.equal(out2, out)
+    with pytest.raises(RuntimeError, match="prepack_weight"):
+        torch.ops.umdk_cam_op_lib.fused_deep_moe(*args(w1p.clone(), w2p))
+    with pytest.raises(RuntimeError, match="prepack_weight"):
+        torch.ops.umdk_cam_op_lib.fused_deep_moe(*args(w1p, w2.to(gpu)))
+    with pytest.raises(RuntimeError, match="prepack_weight"):
+        torch.ops.umdk_cam_op_lib.fused_deep_moe(*args(w2p, w2p))   # packed for the other projection

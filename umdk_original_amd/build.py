@@ -1,4 +1,5 @@
-"""Builds libcam_mi355x.so (HIP kernels + C ABI) for gfx950 with hipcc, in-tree."""
+"""Builds libcam_mi355x.so (HIP kernels + C ABI) for gfx950 with hipcc, and libcam_torch_ops.so (the C++
+registration of torch.ops.umdk_cam_op_lib on top of that ABI) with the host compiler, both in-tree."""
 import os
 import subprocess
 import sys
@@ -44,7 +45,33 @@ def build(verbose=False):
     subprocess.check_call(cmd)
     for o in objs:
         os.remove(o)
+    build_torch_ops(verbose)
     return LIB_PATH
+
+
+TORCH_OPS_PATH = os.path.join(LIB_DIR, "libcam_torch_ops.so")
+
+
+def build_torch_ops(verbose=False):
+    """The torch operator library: host C++ only (no device code), linked against torch and libcam_mi355x.so."""
+    import torch
+    from torch.utils import cpp_extension
+    tdir = os.path.dirname(os.path.abspath(torch.__file__))
+    cxx = os.environ.get("CXX", "g++")
+    cmd = [cxx, "-O2", "-std=c++17", "-fPIC", "-shared", "-fvisibility=hidden",
+           "-D__HIP_PLATFORM_AMD__=1", "-DUSE_ROCM=1",
+           "-D_GLIBCXX_USE_CXX11_ABI=%d" % int(torch._C._GLIBCXX_USE_CXX11_ABI)]
+    for inc in cpp_extension.include_paths() + ["/opt/rocm/include"]:
+        cmd += ["-I", inc]
+    cmd += [os.path.join(_CSRC, "torch_binding.cpp"), "-o", TORCH_OPS_PATH,
+            "-L", os.path.join(tdir, "lib"), "-ltorch", "-ltorch_cpu", "-lc10", "-lc10_hip", "-ltorch_hip",
+            "-L", LIB_DIR, "-lcam_mi355x", "-Wl,-rpath,$ORIGIN", "-Wl,-rpath," + os.path.join(tdir, "lib")]
+    if verbose:
+        print(" ".join(cmd), flush=True)
+    p = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    if p.returncode != 0:
+        raise RuntimeError("building %s failed:\n%s" % (TORCH_OPS_PATH, p.stdout))
+    return TORCH_OPS_PATH
 
 
 if __name__ == "__main__":

@@ -17,6 +17,7 @@ prepacked with `prepack_weight` (the reference needs `npu_format_cast(..., FRACT
 place); `moe_dispatch_prefill` takes an optional `quant_mode` keyword (the reference binding
 hard-codes 0 although its kernel supports dynamic quantisation).
 """
+import os
 import weakref
 
 import torch
@@ -266,8 +267,12 @@ def prepack_weight(w, gate_up):
     """
     _require_gpu(w, "w")
     w = w.contiguous()
-    out = torch.empty_like(w)
-    _lib.call("PrepackWeight", [w, 1 if gate_up else 0, out])
+    if _torch_lib == "cpp":
+        # the C++ operator library remembers the storage of its packed results; fused_deep_moe checks it
+        out = torch.ops.umdk_cam_op_lib.prepack_weight(w, bool(gate_up))
+    else:
+        out = torch.empty_like(w)
+        _lib.call("PrepackWeight", [w, 1 if gate_up else 0, out])
     out._cam_format = CAM_FORMAT_MFMA_B
     out._cam_gate_up = bool(gate_up)
     _PACKED[out.data_ptr()] = (weakref.ref(out), bool(gate_up))
@@ -392,6 +397,14 @@ def register_torch_ops():
     """Define `umdk_cam_op_lib` and attach the ROCm implementations (idempotent)."""
     global _torch_lib
     if _torch_lib is not None:
+        return _torch_lib
+    # The C++ registration (csrc/torch_binding.cpp, built next to the kernel library) when it is there; the
+    # Python one below otherwise.  Both define the same schemas and call the same C ABI.
+    cpp = os.path.join(os.path.dirname(_lib.LIB_PATH), "libcam_torch_ops.so")
+    if os.path.exists(cpp) and os.environ.get("CAM_TORCH_OPS", "cpp") != "python":
+        _lib.lib()  # the kernel library first: the operator library links against it
+        torch.ops.load_library(cpp)
+        _torch_lib = "cpp"
         return _torch_lib
     lib = torch.library.Library("umdk_cam_op_lib", "DEF")
     lib.define("fused_deep_moe(Tensor x, Tensor expertIds, Tensor[] gmm1PermutedWeight, "
