@@ -148,10 +148,10 @@ struct AccType<true> {
 // column block and of its activation row for the current 128-byte K block, and accumulates in fp32.  The
 // scales of the item wait in LDS (a_scale8_s[kb * 256 + tile row], w_scale8_s[column group * kScaleKb + kb]) and
 // are read with the fragments.
-template <int MF, int TEAM, bool FLAT, bool FP8>
+template <int MF, int TEAM, bool FLAT, bool FP8, typename Hook>
 __device__ __forceinline__ void run_item(const GemmArgs &a, const ItemCtx &t, int nb, int8_t *lds,
                                          const float *row_scale_s, const uint8_t *a_scale8_s,
-                                         const uint8_t *w_scale8_s)
+                                         const uint8_t *w_scale8_s, Hook &between)
 {
     constexpr int NS = FLAT ? 3 : 4;                       // ring of stages
     constexpr int LPS = FLAT ? (TEAM == 0 ? 6 : 4) : 4;    // loads per wave and sub-step
@@ -339,8 +339,31 @@ __device__ __forceinline__ void run_item(const GemmArgs &a, const ItemCtx &t, in
     // per lane and fragment and the column scales fetched as 16-byte vectors.  To store whole 128-byte lines,
     // every wave passes one fragment at a time through its own slice of LDS: 128 staged bytes per row, then
     // 16 bytes per lane and 8 rows per store instruction.
+    // `between` is the workgroup's business between two items (taking the next one and asking for its first
+    // bytes, see gemm_kernel).  It runs after this wave has requested its column scales and before it uses them,
+    // so that its memory traffic travels under the arithmetic of the epilogue; it returns a value that depends on
+    // what it loaded, consumed at the very end so that nothing waits for those loads earlier.
+    int between_sink = 0;
     auto epilogue = [&]() {
-    if (MF > 0 && t.wave_live) {
+    const bool work = MF > 0 && t.wave_live;
+    v4f csc[2][4];  // column scales: [0] gate / [1] up of a paired group, or the two fragments of a plain one
+    if (FLAT && !FP8 && work && a.epilogue != kEpiInt32) {
+        const int col_half = (lane >> 5) * 4;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            if (a.epilogue == kEpiSwiglu) {
+                csc[0][j] = *(const v4f *)(t.sg + t.nw * 32 + 8 * j + col_half);
+                csc[1][j] = *(const v4f *)(t.sg + t.N / 2 + t.nw * 32 + 8 * j + col_half);
+            } else {
+                csc[0][j] = *(const v4f *)(t.sg + t.nw * 64 + 8 * j + col_half);
+                csc[1][j] = *(const v4f *)(t.sg + t.nw * 64 + 32 + 8 * j + col_half);
+            }
+        }
+    }
+    if (FLAT) {
+        between_sink = between();
+    }
+    if (work) {
         const int wave = tid >> 6;
         const int row_in = lane & 31;
         const int col_half = (lane >> 5) * 4;
@@ -386,8 +409,13 @@ __device__ __forceinline__ void run_item(const GemmArgs &a, const ItemCtx &t, in
             if (!FP8) {
 #pragma unroll
                 for (int j = 0; j < 4; ++j) {
-                    sg_gate[j] = *(const v4f *)(t.sg + nw * 32 + 8 * j + col_half);
-                    sg_up[j] = *(const v4f *)(t.sg + I + nw * 32 + 8 * j + col_half);
+                    if (FLAT) {
+                        sg_gate[j] = csc[0][j];
+                        sg_up[j] = csc[1][j];
+                    } else {
+                        sg_gate[j] = *(const v4f *)(t.sg + nw * 32 + 8 * j + col_half);
+                        sg_up[j] = *(const v4f *)(t.sg + I + nw * 32 + 8 * j + col_half);
+                    }
                 }
             }
 #pragma unroll
@@ -419,7 +447,7 @@ __device__ __forceinline__ void run_item(const GemmArgs &a, const ItemCtx &t, in
                 for (int nf = 0; nf < 2; ++nf) {
 #pragma unroll
                     for (int j = 0; j < 4; ++j) {
-                        ws[nf][j] = *(const v4f *)(t.sg + nw * 64 + nf * 32 + 8 * j + col_half);
+                        ws[nf][j] = FLAT ? csc[nf][j] : *(const v4f *)(t.sg + nw * 64 + nf * 32 + 8 * j + col_half);
                     }
                 }
             }
@@ -455,6 +483,9 @@ __device__ __forceinline__ void run_item(const GemmArgs &a, const ItemCtx &t, in
     // 128 product columns is exactly what the four waves of a team hold for their rows (32 columns each), so the
     // block maximum needs one exchange through LDS; every wave of the workgroup takes part in its barrier.
     auto epilogue_quant = [&]() {
+        if (FLAT) {
+            between_sink = between();
+        }
         const bool work = MF > 0 && t.wave_live;
         const int wave = tid >> 6;
         const int row_in = lane & 31;
@@ -520,19 +551,20 @@ __device__ __forceinline__ void run_item(const GemmArgs &a, const ItemCtx &t, in
         epilogue();
     }
     barrier_no_fence();  // the staging slices are free again before the next item's loads land
+    asm volatile("" ::"v"(between_sink));
 }
 
-template <int TEAM, bool FLAT, bool FP8>
+template <int TEAM, bool FLAT, bool FP8, typename Hook>
 __device__ __forceinline__ void run_item_mf(int mf, const GemmArgs &a, const ItemCtx &t, int nb, int8_t *lds,
                                             const float *row_scale_s, const uint8_t *a_scale8_s,
-                                            const uint8_t *w_scale8_s)
+                                            const uint8_t *w_scale8_s, Hook &between)
 {
     switch (mf) {
-        case 0: run_item<0, TEAM, FLAT, FP8>(a, t, nb, lds, row_scale_s, a_scale8_s, w_scale8_s); break;
-        case 1: run_item<1, TEAM, FLAT, FP8>(a, t, nb, lds, row_scale_s, a_scale8_s, w_scale8_s); break;
-        case 2: run_item<2, TEAM, FLAT, FP8>(a, t, nb, lds, row_scale_s, a_scale8_s, w_scale8_s); break;
-        case 3: run_item<3, TEAM, FLAT, FP8>(a, t, nb, lds, row_scale_s, a_scale8_s, w_scale8_s); break;
-        default: run_item<4, TEAM, FLAT, FP8>(a, t, nb, lds, row_scale_s, a_scale8_s, w_scale8_s); break;
+        case 0: run_item<0, TEAM, FLAT, FP8>(a, t, nb, lds, row_scale_s, a_scale8_s, w_scale8_s, between); break;
+        case 1: run_item<1, TEAM, FLAT, FP8>(a, t, nb, lds, row_scale_s, a_scale8_s, w_scale8_s, between); break;
+        case 2: run_item<2, TEAM, FLAT, FP8>(a, t, nb, lds, row_scale_s, a_scale8_s, w_scale8_s, between); break;
+        case 3: run_item<3, TEAM, FLAT, FP8>(a, t, nb, lds, row_scale_s, a_scale8_s, w_scale8_s, between); break;
+        default: run_item<4, TEAM, FLAT, FP8>(a, t, nb, lds, row_scale_s, a_scale8_s, w_scale8_s, between); break;
     }
 }
 
@@ -544,6 +576,7 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_kernel(GemmArgs a)
     __shared__ uint8_t a_scale8_s[FP8 ? kScaleKb * 256 : 4];
     __shared__ uint8_t w_scale8_s[FP8 ? 16 * kScaleKb : 4];
     __shared__ int item_s;
+    __shared__ int next_s;
 
     const int tid = threadIdx.x;
     const int team = __builtin_amdgcn_readfirstlane(tid >> 8);
@@ -666,21 +699,67 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_kernel(GemmArgs a)
         }
         __syncthreads();  // item_s may be rewritten and the row scales read from here on
 
+        // Between the K loop and the epilogue of this item: thread 0 learns which item comes next (its take has
+        // been in flight since this item began), and every wave asks for the first bytes that item will load --
+        // one word of every 128-byte line of its first stages -- so that they are on their way to this XCD's L2
+        // while the epilogue computes, and the next item's first direct-to-LDS loads find them there.
+        auto between = [&]() -> int {
+            if (tid == 0) {
+                next = take_end(taken);
+                next_s = next;
+            }
+            __syncthreads();
+            const int nidx = next_s;
+            int sink = 0;
+            if (nidx >= 0 && items[nidx].flat != 0) {  // tall items find their panels in L2 (sibling tiles)
+                const SchedItem nx = items[nidx];
+                const int ng = __builtin_amdgcn_readfirstlane(nx.g);
+                const int nm0 = __builtin_amdgcn_readfirstlane(nx.m0);
+                const int nrows = __builtin_amdgcn_readfirstlane(nx.rows);
+                const int nnb = __builtin_amdgcn_readfirstlane(nx.nb);
+                const bool nflat = __builtin_amdgcn_readfirstlane(nx.flat) != 0;
+                const int stages = nflat ? 3 : 4;
+                const int lane = tid & (kWave - 1);
+                if (nflat || team == 1) {  // the waves that load weights: 4 KB per stage and wave
+                    const int8_t *wgn = a.per_expert ? a.list.w[ng] : a.w + (long long)ng * a.Kd * a.N;
+                    const int ngroups = a.N / 64;
+                    const int grp = min(nnb * (nflat ? 8 : 4) + (nflat ? team * 4 + wn : wn), ngroups - 1);
+                    const int blk = grp >> 3;
+                    const long long step = (long long)min(8, ngroups - 8 * blk) * 4096;
+                    const int8_t *base = wgn + (long long)blk * 8 * a.Kd * 64 + (grp & 7) * 4096;
+                    const int steps = min(stages, a.Kd / kBK);
+                    for (int i = lane; i < steps * 32; i += kWave) {  // 32 lines per stage
+                        sink ^= *(const int *)(base + (long long)(i >> 5) * step + (i & 31) * 128);
+                    }
+                }
+                if (team == 0) {  // the waves that load activations: rows of 64 bytes per stage
+                    const int per_wave = nflat ? 32 : 64;
+                    const int span = min(stages * kBK, a.Kd);          // bytes of a row the first stages cover
+                    const int lines = (span + 127) / 128;
+                    for (int i = lane; i < per_wave * lines; i += kWave) {
+                        const int r = min(per_wave * wn + i / lines, nrows - 1);
+                        sink ^= *(const int *)(a.a + (long long)(nm0 + r) * a.Kd + (i % lines) * 128);
+                    }
+                }
+            }
+            return sink;
+        };
+
         const int mf = t.my_rows <= 0 ? 0 : (t.my_rows + 31) >> 5;
         if (flat) {
             if (team == 0) {
-                run_item_mf<0, true, FP8>(mf, a, t, nb, lds, row_scale_s, a_scale8_s, w_scale8_s);
+                run_item_mf<0, true, FP8>(mf, a, t, nb, lds, row_scale_s, a_scale8_s, w_scale8_s, between);
             } else {
-                run_item_mf<1, true, FP8>(mf, a, t, nb, lds, row_scale_s, a_scale8_s, w_scale8_s);
+                run_item_mf<1, true, FP8>(mf, a, t, nb, lds, row_scale_s, a_scale8_s, w_scale8_s, between);
             }
         } else {
             if (team == 0) {
-                run_item_mf<0, false, FP8>(mf, a, t, nb, lds, row_scale_s, a_scale8_s, w_scale8_s);
+                run_item_mf<0, false, FP8>(mf, a, t, nb, lds, row_scale_s, a_scale8_s, w_scale8_s, between);
             } else {
-                run_item_mf<1, false, FP8>(mf, a, t, nb, lds, row_scale_s, a_scale8_s, w_scale8_s);
+                run_item_mf<1, false, FP8>(mf, a, t, nb, lds, row_scale_s, a_scale8_s, w_scale8_s, between);
             }
         }
-        if (tid == 0) {
+        if (!flat && tid == 0) {  // a flat item has taken its successor between its K loop and its epilogue
             next = take_end(taken);
         }
     }
