@@ -288,30 +288,58 @@ __device__ __forceinline__ void run_item(const GemmArgs &a, const ItemCtx &t, in
         __builtin_amdgcn_sched_barrier(0);
     };
 
-    // ---- pipeline.  Loads retire in order and every sub-step issues exactly LPS loads per wave, so "at most
-    // n * LPS outstanding" says which sub-steps of this wave's loads have landed; the barrier after the wait
-    // makes that true for the whole workgroup.  Sub-step indices past the end are clamped (the last sub-step
-    // is fetched again into a stage nobody reads), so the loop body has no control flow.
+    // ---- pipeline.  Loads retire in order and every sub-step that requests a stage issues exactly LPS loads per
+    // wave, so "at most n * LPS outstanding" says which sub-steps of this wave's loads have landed; the barrier
+    // after the wait makes that true for the whole workgroup.  In the last NS sub-steps nothing is left to request
+    // and the wait is for what remains: with `rem` stages after the current one, stage s+1 has landed once at most
+    // rem - 1 stages are outstanding.
     //   barrier A(s): every load of stage s+1 has landed; team 1 is done reading stage s
     //   barrier B(s): team 0 is done reading stage s+1
     // Stage s is free once both teams have its fragments in registers, i.e. after barrier A(s): team 0 refills
     // it in the phase that follows, team 1 at the end of its own reading phase.
+    auto wait_stages = [&](int n) {  // at most n stages of this wave's loads outstanding (n wave-uniform)
+        if (n <= 0) {
+            wait_loads_outstanding<0>();
+        } else if (n == 1) {
+            wait_loads_outstanding<LPS>();
+        } else if (n == 2) {
+            wait_loads_outstanding<2 * LPS>();
+        } else {
+            wait_loads_outstanding<3 * LPS>();
+        }
+    };
+    // Tall tiles keep a loop body without control flow instead (their long bodies schedule worse with it: +2-4 %):
+    // sub-step indices past the end are clamped, i.e. the last sub-step is fetched again into a stage nobody
+    // reads, and every sub-step requests a stage.
 #pragma unroll
     for (int p = 0; p < NS; ++p) {
-        issue(p, p);
+        if (!FLAT || p <= last) {
+            issue(p, p);
+        }
     }
-    wait_loads_outstanding<(NS - 1) * LPS>();
+    if (FLAT) {
+        wait_stages(min(NS - 1, last));
+    } else {
+        wait_loads_outstanding<(NS - 1) * LPS>();
+    }
     barrier_no_fence();  // stage 0 has landed
     int slot = 0;        // slot of stage s
+    const int steady = FLAT ? KT - NS : KT;  // sub-steps that request the stage NS ahead
     if (TEAM == 0) {
         read_frags(0, 0);
         wait_lds_reads();
         for (int s = 0; s < KT; ++s) {
             const int next = slot + 1 == NS ? 0 : slot + 1;
             multiply();                                   // phase 1: stage s, from registers
-            wait_loads_outstanding<(NS - 2) * LPS>();     // my part of stage s+1 has landed
+            if (!FLAT || s < steady) {
+                wait_loads_outstanding<(NS - 2) * LPS>(); // my part of stage s+1 has landed
+            } else if (s < last) {
+                wait_stages(last - s - 1);
+            }
             barrier_no_fence();                           // A(s)
-            issue(s + NS, slot);                          // phase 2: refill stage s's slot ...
+            if (!FLAT || s < steady) {
+                issue(s + NS, slot);                      // phase 2: refill stage s's slot ...
+            }
             read_frags(next, s + 1);                      // ... and fetch the fragments of stage s+1
             wait_lds_reads();
             barrier_no_fence();                           // B(s)
@@ -322,15 +350,21 @@ __device__ __forceinline__ void run_item(const GemmArgs &a, const ItemCtx &t, in
             const int next = slot + 1 == NS ? 0 : slot + 1;
             read_frags(slot, s);                          // phase 1: fragments of stage s ...
             wait_lds_reads();
-            issue(s + NS, slot);                          // ... then refill its slot
-            wait_loads_outstanding<(NS - 1) * LPS>();     // my part of stage s+1 has landed
+            if (!FLAT || s < steady) {
+                issue(s + NS, slot);                      // ... then refill its slot
+                wait_loads_outstanding<(NS - 1) * LPS>(); // my part of stage s+1 has landed
+            } else if (s < last) {
+                wait_stages(last - s - 1);
+            }
             barrier_no_fence();                           // A(s)
             multiply();                                   // phase 2: stage s
             barrier_no_fence();                           // B(s)
             slot = next;
         }
     }
-    wait_loads_outstanding<0>();
+    if (!FLAT) {
+        wait_loads_outstanding<0>();
+    }
     barrier_no_fence();  // nobody reads or fills the stages any more: the epilogue may stage through them
 
     // ---- epilogue, accumulators in registers.
