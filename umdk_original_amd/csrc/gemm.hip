@@ -148,10 +148,10 @@ struct AccType<true> {
 // column block and of its activation row for the current 128-byte K block, and accumulates in fp32.  The
 // scales of the item wait in LDS (a_scale8_s[kb * 256 + tile row], w_scale8_s[column group * kScaleKb + kb]) and
 // are read with the fragments.
-template <int MF, int TEAM, bool FLAT, bool FP8, typename Hook>
+template <int MF, int TEAM, bool FLAT, bool FP8, typename Hook, typename Stage>
 __device__ __forceinline__ void run_item(const GemmArgs &a, const ItemCtx &t, int nb, int8_t *lds,
                                          const float *row_scale_s, const uint8_t *a_scale8_s,
-                                         const uint8_t *w_scale8_s, Hook &between)
+                                         const uint8_t *w_scale8_s, Hook &between, Stage &stage_scales)
 {
     constexpr int NS = FLAT ? 3 : 4;                       // ring of stages
     constexpr int LPS = FLAT ? (TEAM == 0 ? 6 : 4) : 4;    // loads per wave and sub-step
@@ -317,12 +317,17 @@ __device__ __forceinline__ void run_item(const GemmArgs &a, const ItemCtx &t, in
             issue(p, p);
         }
     }
+    // The item's scales go to LDS now, behind the requests for the first stages, so that their round trip to
+    // memory runs beside that of the weights instead of ahead of it.  (Their loads are younger than the stage
+    // loads and complete after them: the wait below is then met at once.)
+    stage_scales();
+    wait_lds_reads();
     if (FLAT) {
         wait_stages(min(NS - 1, last));
     } else {
         wait_loads_outstanding<(NS - 1) * LPS>();
     }
-    barrier_no_fence();  // stage 0 has landed
+    barrier_no_fence();  // stage 0 has landed and every wave's share of the scales is in LDS
     int slot = 0;        // slot of stage s
     const int steady = FLAT ? KT - NS : KT;  // sub-steps that request the stage NS ahead
     if (TEAM == 0) {
@@ -588,17 +593,17 @@ __device__ __forceinline__ void run_item(const GemmArgs &a, const ItemCtx &t, in
     asm volatile("" ::"v"(between_sink));
 }
 
-template <int TEAM, bool FLAT, bool FP8, typename Hook>
+template <int TEAM, bool FLAT, bool FP8, typename Hook, typename Stage>
 __device__ __forceinline__ void run_item_mf(int mf, const GemmArgs &a, const ItemCtx &t, int nb, int8_t *lds,
                                             const float *row_scale_s, const uint8_t *a_scale8_s,
-                                            const uint8_t *w_scale8_s, Hook &between)
+                                            const uint8_t *w_scale8_s, Hook &between, Stage &stage_scales)
 {
     switch (mf) {
-        case 0: run_item<0, TEAM, FLAT, FP8>(a, t, nb, lds, row_scale_s, a_scale8_s, w_scale8_s, between); break;
-        case 1: run_item<1, TEAM, FLAT, FP8>(a, t, nb, lds, row_scale_s, a_scale8_s, w_scale8_s, between); break;
-        case 2: run_item<2, TEAM, FLAT, FP8>(a, t, nb, lds, row_scale_s, a_scale8_s, w_scale8_s, between); break;
-        case 3: run_item<3, TEAM, FLAT, FP8>(a, t, nb, lds, row_scale_s, a_scale8_s, w_scale8_s, between); break;
-        default: run_item<4, TEAM, FLAT, FP8>(a, t, nb, lds, row_scale_s, a_scale8_s, w_scale8_s, between); break;
+        case 0: run_item<0, TEAM, FLAT, FP8>(a, t, nb, lds, row_scale_s, a_scale8_s, w_scale8_s, between, stage_scales); break;
+        case 1: run_item<1, TEAM, FLAT, FP8>(a, t, nb, lds, row_scale_s, a_scale8_s, w_scale8_s, between, stage_scales); break;
+        case 2: run_item<2, TEAM, FLAT, FP8>(a, t, nb, lds, row_scale_s, a_scale8_s, w_scale8_s, between, stage_scales); break;
+        case 3: run_item<3, TEAM, FLAT, FP8>(a, t, nb, lds, row_scale_s, a_scale8_s, w_scale8_s, between, stage_scales); break;
+        default: run_item<4, TEAM, FLAT, FP8>(a, t, nb, lds, row_scale_s, a_scale8_s, w_scale8_s, between, stage_scales); break;
     }
 }
 
@@ -710,28 +715,29 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_kernel(GemmArgs a)
         const int group = nb * (flat ? 8 : 4) + t.bslot;
         t.wave_live = group < a.N / 64;
         t.nw = min(group, a.N / 64 - 1);
-        if (FP8) {
-            // the item's scales: activation rows x K blocks (transposed, so that the lanes of a fragment read
-            // neighbouring bytes), and one row of K blocks per 64-column group of the item
-            const int KB = a.Kd >> 7;
-            for (int i = tid; i < 256 * KB; i += kThreads) {
-                const int r = i / KB, kb = i - r * KB;
-                a_scale8_s[kb * 256 + r] = a.a_scale8[(long long)(m0 + min(r, rows - 1)) * KB + kb];
+        auto stage_scales = [&]() {
+            if (FP8) {
+                // the item's scales: activation rows x K blocks (transposed, so that the lanes of a fragment read
+                // neighbouring bytes), and one row of K blocks per 64-column group of the item
+                const int KB = a.Kd >> 7;
+                for (int i = tid; i < 256 * KB; i += kThreads) {
+                    const int r = i / KB, kb = i - r * KB;
+                    a_scale8_s[kb * 256 + r] = a.a_scale8[(long long)(m0 + min(r, rows - 1)) * KB + kb];
+                }
+                const int ngr = flat ? 8 : 4;
+                const int nblk = a.N >> 7;
+                for (int i = tid; i < ngr * 2 * KB; i += kThreads) {
+                    const int gf = i / KB, kb = i - gf * KB;  // gf = column group of the item * 2 + fragment
+                    const int grp = min(nb * ngr + (gf >> 1), a.N / 64 - 1);  // packed 64-column group of the weight
+                    const int nf = gf & 1;
+                    // first logical column of the fragment (a paired group holds 32 gate and 32 up columns)
+                    const int col = a.gate_up ? nf * (a.N / 2) + grp * 32 : grp * 64 + nf * 32;
+                    w_scale8_s[gf * kScaleKb + kb] = a.w_scale8[((long long)g * KB + kb) * nblk + (col >> 7)];
+                }
+            } else if (a.epilogue != kEpiInt32 && tid < 256) {
+                row_scale_s[tid] = a.a_scale[m0 + min(tid, rows - 1)];
             }
-            const int ngr = flat ? 8 : 4;
-            const int nblk = a.N >> 7;
-            for (int i = tid; i < ngr * 2 * KB; i += kThreads) {
-                const int gf = i / KB, kb = i - gf * KB;  // gf = column group of the item * 2 + fragment
-                const int grp = min(nb * ngr + (gf >> 1), a.N / 64 - 1);  // packed 64-column group of the weight
-                const int nf = gf & 1;
-                // first logical column of the fragment (a paired group holds 32 gate and 32 up columns)
-                const int col = a.gate_up ? nf * (a.N / 2) + grp * 32 : grp * 64 + nf * 32;
-                w_scale8_s[gf * kScaleKb + kb] = a.w_scale8[((long long)g * KB + kb) * nblk + (col >> 7)];
-            }
-        } else if (a.epilogue != kEpiInt32 && tid < 256) {
-            row_scale_s[tid] = a.a_scale[m0 + min(tid, rows - 1)];
-        }
-        __syncthreads();  // item_s may be rewritten and the row scales read from here on
+        };
 
         // Between the K loop and the epilogue of this item: thread 0 learns which item comes next (its take has
         // been in flight since this item began), and every wave asks for the first bytes that item will load --
@@ -782,15 +788,15 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_kernel(GemmArgs a)
         const int mf = t.my_rows <= 0 ? 0 : (t.my_rows + 31) >> 5;
         if (flat) {
             if (team == 0) {
-                run_item_mf<0, true, FP8>(mf, a, t, nb, lds, row_scale_s, a_scale8_s, w_scale8_s, between);
+                run_item_mf<0, true, FP8>(mf, a, t, nb, lds, row_scale_s, a_scale8_s, w_scale8_s, between, stage_scales);
             } else {
-                run_item_mf<1, true, FP8>(mf, a, t, nb, lds, row_scale_s, a_scale8_s, w_scale8_s, between);
+                run_item_mf<1, true, FP8>(mf, a, t, nb, lds, row_scale_s, a_scale8_s, w_scale8_s, between, stage_scales);
             }
         } else {
             if (team == 0) {
-                run_item_mf<0, false, FP8>(mf, a, t, nb, lds, row_scale_s, a_scale8_s, w_scale8_s, between);
+                run_item_mf<0, false, FP8>(mf, a, t, nb, lds, row_scale_s, a_scale8_s, w_scale8_s, between, stage_scales);
             } else {
-                run_item_mf<1, false, FP8>(mf, a, t, nb, lds, row_scale_s, a_scale8_s, w_scale8_s, between);
+                run_item_mf<1, false, FP8>(mf, a, t, nb, lds, row_scale_s, a_scale8_s, w_scale8_s, between, stage_scales);
             }
         }
         if (!flat && tid == 0) {  // a flat item has taken its successor between its K loop and its epilogue
