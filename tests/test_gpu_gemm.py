@@ -235,3 +235,25 @@ def test_gmm2_fp16_output_bit_exact(gpu, oracle):
     want = oracle.gmm2_epilogue_act(c, ws.numpy(), xs.numpy(), gl.numpy(), True)
     assert out.dtype == torch.float16
     assert_bits_equal(out.cpu().view(torch.int16).numpy().view(np.uint16)[:A], want[:A], "fp16 output")
+
+
+@pytest.mark.parametrize("Kd,N,gate_up", [(256, 1024, False), (192 + 64, 1280, True), (128, 576, False)])
+def test_many_flat_items_per_workgroup_bit_exact(gpu, oracle, Kd, N, gate_up):
+    """A decode-like group list: 300 experts of 0-9 rows, i.e. 600-900 flat items on 256 workgroups, so that every
+    workgroup runs several flat items one after the other (the successor is taken and its first stages are
+    touched between the K loop and the epilogue; short K loops end without requesting stages), with ragged
+    column blocks and empty experts in between."""
+    announce("gemm many flat items Kd=%d N=%d gate_up=%s" % (Kd, N, gate_up))
+    rng = np.random.default_rng(Kd + N)
+    sizes = [int(v) for v in rng.integers(0, 10, size=300)]
+    a, w, gl, A = _inputs(sizes, Kd, N, seed=Kd * 3 + N)
+    wp = cam.prepack_weight(w.to(gpu), gate_up)
+    got = cam.grouped_matmul_int32(a.to(gpu), wp, gl.to(gpu))
+    want = oracle.gmm_int32(a.numpy(), w.numpy(), gl.numpy())
+    assert_bits_equal(to_np(got)[:A], want[:A], "int32 accumulators")
+    if not gate_up:
+        G = len(sizes)
+        ws = synth.channel_scales((G, N), seed=41)
+        xs = synth.channel_scales((max(A, 1),), seed=42, lo=0.001, hi=0.01)
+        out = cam.grouped_matmul_dequant(a.to(gpu), xs.to(gpu), wp, ws.to(gpu), gl.to(gpu))
+        assert_bits_equal(to_np(out)[:A], oracle.gmm2_epilogue(want, ws.numpy(), xs.numpy(), gl.numpy())[:A], "bf16 output")
