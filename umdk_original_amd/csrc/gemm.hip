@@ -45,6 +45,11 @@
 //     stored.  For GMM1 the prepack pairs gate column c with up column I+c inside one wave.
 //   * The K order inside a 32-deep MFMA step is whatever the two operands agree on (an integer dot
 //     product does not care), which is what lets both be loaded as plain 16-byte pieces.
+//   * Flat items are bound by the memory, and three things in this file exist for them alone: their weight
+//     panels are fetched with non-temporal loads (nobody else reads them); they stop requesting stages in
+//     their last sub-steps, where tall items keep a branch-free loop body and fetch the last sub-step again;
+//     and between the K loop and the epilogue of a flat item the workgroup takes its next item and, if that
+//     is flat too, touches the lines of its first stages so that they travel to L2 under the epilogue.
 #include "cam_device.h"
 #include "cam_kernels.h"
 #include "rank_device.h"
