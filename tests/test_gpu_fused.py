@@ -85,6 +85,18 @@ def test_fused_active_mask_and_tensor_lists(gpu, oracle, dispatch_launch):
     assert (out[23:] == 0).all()
 
 
+def test_fused_active_mask_over_several_ranking_chunks(gpu, oracle, dispatch_launch):
+    """2800 routing entries (two ranking chunks), the active prefix ends inside a workgroup's four tokens and
+    inside the first chunk's neighbour: the plan must stop counting at the prefix in every launch form."""
+    announce("fused mask, several ranking chunks (%s)" % dispatch_launch)
+    d = synth.ut_recipe(batch_size=700, hidden=1024, intermediate=512, num_experts=16, top_k=4, seed=9)
+    mask = torch.zeros(700, dtype=torch.bool)
+    mask[:601] = True
+    out, etn = _run(gpu, d, mask=mask, via_torch_ops=False)
+    assert _check(oracle, d, out, etn, n_active=601) == 0
+    assert (out[601:] == 0).all()
+
+
 def test_fused_negative_ids_and_skew(gpu, oracle, dispatch_launch):
     announce("fused skewed routing with dropped entries")
     T, H, E, K, I = 300, 1024, 32, 6, 512
