@@ -61,18 +61,43 @@ __global__ __launch_bounds__(kGlobalThreads) void plan_global_kernel(PlanArgs a,
     const int E = a.E;
     const IdT *__restrict__ idx = (const IdT *)a.idx;
 
+    // This thread's first entry of the chunk is requested before the histogram columns, so that its round trip
+    // to memory runs beside theirs instead of after the scan.
+    const long long n_all = (long long)a.T * a.K;
+    const long long lo = (long long)b * chunk;
+    const long long hi = min(n_all, lo + chunk);
+    const long long i0 = lo + tid;
+    long long raw0 = -1;
+    int pos0 = 0;
+    if (i0 < hi) {
+        raw0 = (long long)idx[i0];
+        pos0 = a.pos[i0];
+    }
+
     int cnt = 0, base = 0;
     if (tid < E) {
         const int32_t *col = hist_in + tid;
         int bb = 0;
-        for (; bb + 16 <= nb; bb += 16) {  // 16 independent loads in flight per thread
-            int v[16];
+        for (; bb + 64 <= nb; bb += 64) {  // 64 independent loads in flight per thread: one round trip at C2
+            int v[64];
 #pragma unroll
-            for (int j = 0; j < 16; ++j) {
+            for (int j = 0; j < 64; ++j) {
                 v[j] = col[(long long)(bb + j) * E];
             }
 #pragma unroll
-            for (int j = 0; j < 16; ++j) {
+            for (int j = 0; j < 64; ++j) {
+                cnt += v[j];
+                base += (bb + j) < b ? v[j] : 0;
+            }
+        }
+        for (; bb + 8 <= nb; bb += 8) {
+            int v[8];
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                v[j] = col[(long long)(bb + j) * E];
+            }
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
                 cnt += v[j];
                 base += (bb + j) < b ? v[j] : 0;
             }
@@ -91,14 +116,18 @@ __global__ __launch_bounds__(kGlobalThreads) void plan_global_kernel(PlanArgs a,
 
     const int t_active = hist_in[(long long)nb * E];
     const long long n = (long long)t_active * a.K;
-    const long long n_all = (long long)a.T * a.K;
-    const long long lo = (long long)b * chunk;
-    const long long hi = min(n_all, lo + chunk);
-    for (long long i = lo + tid; i < hi; i += kGlobalThreads) {
-        const int e = i < n ? load_id(idx, i, E) : -1;
+    for (long long i = i0; i < hi; i += kGlobalThreads) {
+        int e, p0;
+        if (i == i0) {
+            e = (i < n && raw0 >= 0 && raw0 < (long long)E) ? (int)raw0 : -1;
+            p0 = pos0;
+        } else {
+            e = i < n ? load_id(idx, i, E) : -1;
+            p0 = e >= 0 ? a.pos[i] : 0;
+        }
         int row = -1;
         if (e >= 0) {
-            const int p = a.pos[i] + base_s[e];
+            const int p = p0 + base_s[e];
             a.pos[i] = p;
             row = off_s[e] + p;
         }

@@ -87,24 +87,24 @@ __device__ __forceinline__ void rank_chunk(const IdT *__restrict__ idx, int b, l
     const int tid = threadIdx.x;
     const int lane = tid & (kWave - 1);
     const int w = tid >> 6;
-    for (int i = tid; i < kLocalWaves * kMaxExperts; i += kLocalThreads) {
-        hist[i] = 0;
-    }
-    __syncthreads();
+    // the ids are requested first: their trip to memory runs while the histograms are cleared
     const long long base = (long long)b * (IT * kLocalThreads) + (long long)w * (IT * kWave);
-    int nbits = 0;
-    while ((1 << nbits) < E) {
-        ++nbits;
-    }
-    int *my_hist = hist + w * kMaxExperts;
-    const unsigned long long lt_mask = (1ull << lane) - 1ull;
-
     int e[IT], r[IT];
 #pragma unroll
     for (int it = 0; it < IT; ++it) {
         const long long i = base + it * kWave + lane;
         e[it] = i < n ? load_id(idx, i, E) : -1;
     }
+    for (int i = tid; i < kLocalWaves * kMaxExperts; i += kLocalThreads) {
+        hist[i] = 0;
+    }
+    __syncthreads();
+    int nbits = 0;
+    while ((1 << nbits) < E) {
+        ++nbits;
+    }
+    int *my_hist = hist + w * kMaxExperts;
+    const unsigned long long lt_mask = (1ull << lane) - 1ull;
 #pragma unroll
     for (int it = 0; it < IT; ++it) {
         const bool act = e[it] >= 0;
