@@ -152,17 +152,6 @@ def main():
             torch.empty((T, K), dtype=torch.int32), torch.empty((T, K), dtype=torch.int32), None, None,
             torch.empty(E, dtype=torch.int32), None, torch.empty(1, dtype=torch.int64)])
         assert st == 0, msg
-        cam.set_dispatch_launch_mode(cam.DISPATCH_LAUNCH_SINGLE)  # the one-launch form needs its own workspace size
-        try:
-            st, ws_single, msg = _lib.phase1("MoeDispatchPrefill", [
-                xs[0], ids, E, 1, 0, 2, torch.empty((A, H), dtype=torch.int8), torch.empty(A),
-                torch.empty(3 * A, dtype=torch.int32), torch.empty((T, K), dtype=torch.int32),
-                torch.empty((T, K), dtype=torch.int32), None, None, torch.empty(E, dtype=torch.int32), None,
-                torch.empty(1, dtype=torch.int64)])
-        finally:
-            cam.set_dispatch_launch_mode(cam.DISPATCH_LAUNCH_AUTO)
-        assert st == 0, msg
-        ws_bytes = max(ws_bytes, ws_single)
         dsets = [dict(rx=torch.empty((A, H), dtype=torch.int8, device=dev),
                       sc=torch.empty(A, dtype=torch.float32, device=dev), info=torch.empty(3 * A, **i32),
                       pos=torch.empty((T, K), **i32), slot=torch.empty((T, K), **i32), cnt=torch.empty(E, **i32),
@@ -181,7 +170,7 @@ def main():
         def run_combine(i):
             d = dsets[i % NBUF]
             # the (token, k) -> row map the dispatch produced, handed straight to the gather
-            _lib.call("MoeCombineGather", [ys[i % NBUF], None, d["slot"], d["rcnt"], gw, couts[i % NBUF]])
+            _lib.call("MoeCombineGather", [ys[i % NBUF], None, d["slot"], d["rcnt"], gw, None, couts[i % NBUF]])
 
         for i in range(NBUF):
             run_dispatch(i)  # fills every set's map before any combine-only graph runs
@@ -249,18 +238,6 @@ def main():
                                                         note="MoeDispatchPlan + MoeDispatchNormal, three launches")
             log("dispatch as plan + normal operators: %.1f us" % (s_pair["mean"] * 1e6))
             del plan_bufs
-            # the same operator forced into ONE launch (plan under the first row loads)
-            cam.set_dispatch_launch_mode(cam.DISPATCH_LAUNCH_SINGLE)
-            try:
-                s_single = spread(graph_of(disp_rot), ROT, SPREAD_REPLAYS)
-            finally:
-                cam.set_dispatch_launch_mode(cam.DISPATCH_LAUNCH_AUTO)
-            kernels["dispatch_single_launch"] = dict(bound="hbm", us=us(s_single),
-                                                     achieved=disp_bytes / s_single["mean"] / 1e9, unit="GB/s",
-                                                     frac=disp_bytes / s_single["mean"] / HBM_PEAK,
-                                                     note="MoeDispatchPrefill forced into one launch "
-                                                          "(camSetDispatchLaunchMode)")
-            log("dispatch forced into one launch: %.1f us" % (s_single["mean"] * 1e6))
 
         if want("step") or want("combine"):
             s_comb = spread(graph_of(comb_rot), ROT, SPREAD_REPLAYS)
@@ -297,7 +274,7 @@ def main():
 
             def comb_decode():
                 for i in range(ROT):
-                    _lib.call("MoeCombineGather", [yd[i % NBUF], None, dd["slot_row"], dd["recv_count"], gwd,
+                    _lib.call("MoeCombineGather", [yd[i % NBUF], None, dd["slot_row"], dd["recv_count"], gwd, None,
                                                    od[i % NBUF]])
 
             s_cd = spread(graph_of(comb_decode), ROT, SPREAD_REPLAYS)
@@ -320,7 +297,7 @@ def main():
             def comb_wire():
                 for i in range(ROT):
                     d = dsets[i % NBUF]
-                    _lib.call("MoeCombineGather", [wire[i % NBUF], None, d["slot"], d["rcnt"], gw, couts[i % NBUF]])
+                    _lib.call("MoeCombineGather", [wire[i % NBUF], None, d["slot"], d["rcnt"], gw, None, couts[i % NBUF]])
 
             s_cw = spread(graph_of(comb_wire), ROT, SPREAD_REPLAYS)
             wire_bytes = A * (H + H // 4) + A * 4 + A * 4 + T * H * 2

@@ -96,18 +96,6 @@ CAM_API const char *camGetRecentErrMsg(void);
 CAM_API camStatus camDestroyExecutor(camOpExecutor *executor);
 CAM_API const char *camGetVersion(void);
 
-/* How MoeDispatchPrefill and the fused layers launch the plan + permute of the dispatch (no counterpart in the
- * reference; the results are identical in every mode).  CAM_DISPATCH_LAUNCH_AUTO (default) and
- * CAM_DISPATCH_LAUNCH_SEPARATE: MoeDispatchPlan's launches followed by MoeDispatchNormal's, the faster form at
- * every measured size (in a fused layer the permute launch also builds the GEMM schedules).
- * CAM_DISPATCH_LAUNCH_SINGLE: plan, permute and quantisation as ONE launch whenever T*K <= 524288 (one graph node,
- * no intermediate launch boundaries; 3-30 % slower).  The setting is process-wide and read by phase 1 of those
- * operators; returns CAM_ERR_RANGE for another value. */
-#define CAM_DISPATCH_LAUNCH_AUTO 0
-#define CAM_DISPATCH_LAUNCH_SINGLE 1
-#define CAM_DISPATCH_LAUNCH_SEPARATE 2
-CAM_API camStatus camSetDispatchLaunchMode(int32_t mode);
-
 /* ------------------------------------------------------------------------------------------------
  * DispatchLayout -- replaces aclnnDispatchLayout (AUTOGEN/aclnn_dispatch_layout.h:32-54).
  * topkIdx int64 [T,K] (int32 also accepted) -> numTokensPerRank int32 [R], numTokensPerExpert
@@ -214,8 +202,7 @@ CAM_API camStatus camMoeDispatchNormal(void *workspace, uint64_t workspaceSize, 
  * MoeDispatchPrefill -- the whole body of the reference's binding-level operator moe_dispatch_prefill
  * (src/cam/comm_operator/pybind/moe_dispatch_prefill.cpp:96-192: the CPU ranking loop, the CPU loop over the
  * exchanged counts, two device-to-host copies and the aclnnMoeDispatchNormal call) as one operator with no host
- * round trip for one rank: MoeDispatchPlan and MoeDispatchNormal back to back on the stream (or, on request, as
- * ONE kernel launch with the plan running underneath the first row loads).
+ * round trip for one rank: MoeDispatchPlan's launches and MoeDispatchNormal's back to back on the stream.
  * x bf16/fp16 [T,H]; topkIdx int64/int32 [T,K] -> recvX [A,H] (int8 when quantMode is 2 or 3, else
  * x's dtype), recvXScalesOptional fp32 [A] (required when quantising); quantMode 4, which the reference does
  * not have, gives block-scaled FP8 rows instead (recvX E4M3 [A,H], recvXScales uint8 [A,H/128], cam_fp8_spec.h);
@@ -224,9 +211,7 @@ CAM_API camStatus camMoeDispatchNormal(void *workspace, uint64_t workspaceSize, 
  * sendOffset int32 [E], recvCount int32 [E], numRecvTokensPerExpert int64 [E], totalRecvTokens int64 [1],
  * all exactly as MoeDispatchPlan / MoeDispatchNormal produce them.  Rows outside [0,A) are dropped, so A
  * may be a worst-case bound (T*K) and the true total read later from totalRecvTokens.
- * The workspace may hold anything on first use; a launch leaves it ready for the next one.  Launches
- * that share a workspace must not overlap.  Whether the single launch or MoeDispatchPlan's and
- * MoeDispatchNormal's launches run is decided by camSetDispatchLaunchMode (same results either way). */
+ * The workspace may hold anything on first use.  Launches that share a workspace must not overlap. */
 CAM_API camStatus camMoeDispatchPrefillGetWorkspaceSize(
     const camTensor *x, const camTensor *topkIdx, int64_t numExperts, int64_t numRanks, int64_t rankId,
     int64_t quantMode, const camTensor *recvX, const camTensor *recvXScalesOptional, const camTensor *expandIdx,
@@ -271,7 +256,11 @@ CAM_API camStatus camMoeCombineNormal(void *workspace, uint64_t workspaceSize, c
  *   then one bf16 scale per block of 8 columns -- the int8 communication quantisation of
  *   AK/moe_combine_shmem/op_kernel/moe_combine_shmem.h:564-592.  Each value is rebuilt as
  *   bf16(float(q) * float(scale)) (:755-773) before it is weighted and summed.  GroupedMatmulDequant writes
- *   such rows when its out tensor is int8. */
+ *   such rows when its out tensor is int8.
+ *   sharedXOptional [T,H] of out's type: the shared expert's output row of every token, added un-weighted to
+ *   the fp32 accumulator after the K routed rows and before the one rounding
+ *   (FDM/raw_distributed/cam_moe_distribute_combine.h:757-774; AK/moe_combine_shmem/op_kernel/
+ *   moe_combine_shmem.h:873-907).  Where that row lives on which rank is the caller's business here. */
 CAM_API camStatus camMoeCombineIndexGetWorkspaceSize(const camTensor *tokenSrcInfo, int64_t numRows,
                                                      const camTensor *slotRow, uint64_t *workspaceSize,
                                                      camOpExecutor **executor);
@@ -279,10 +268,64 @@ CAM_API camStatus camMoeCombineIndex(void *workspace, uint64_t workspaceSize, ca
                                      camStream_t stream);
 CAM_API camStatus camMoeCombineGatherGetWorkspaceSize(const camTensor *recvX, const camTensor *tokenSrcInfoOptional,
                                                       const camTensor *slotRow, const camTensor *epRecvCountsOptional,
-                                                      const camTensor *recvTopkWeights, const camTensor *out,
+                                                      const camTensor *recvTopkWeights,
+                                                      const camTensor *sharedXOptional, const camTensor *out,
                                                       uint64_t *workspaceSize, camOpExecutor **executor);
 CAM_API camStatus camMoeCombineGather(void *workspace, uint64_t workspaceSize, camOpExecutor *executor,
                                       camStream_t stream);
+
+/* ------------------------------------------------------------------------------------------------
+ * MoeDispatchShmem -- replaces aclnnMoeDispatchShmem (AUTOGEN/aclnn_moe_dispatch_shmem.h:46-53), one rank.
+ * x bf16/fp16 [bs,H]; expertIds int32 [bs,K]; scalesOptional fp32 [moeExpertNum,H] (per-expert smooth scales);
+ * xActiveMaskOptional must be NULL (reserved in the reference) -> expandXOut [A,H] (int8 when quantMode == 2, else
+ * x's dtype), dynamicScalesOut fp32 [A] (written when quantising), expandIdxOut int32 [bs*K] = the place of
+ * entry (t,k) among the entries of its expert (AK/moe_dispatch_shmem/op_kernel/moe_dispatch_shmem.h:541-548),
+ * expertTokenNumsOut int64 [moeExpertNum]: running totals when expertTokenNumsType == 0, per-expert counts when 1
+ * (:1022-1051), epRecvCountOut int32 [moeExpertNum]: inclusive running totals in (local expert, source rank)
+ * order (:853-856,:927-931); tpRecvCountOut is left untouched (tpWorldSize <= 1).
+ * Row of (t,k) with e = expertIds[t,k]: (e ? epRecvCountOut[e-1] : 0) + expandIdxOut[t*K+k]; rows outside [0,A)
+ * are dropped, so A may be the worst case bs*K.  Ids outside [0, moeExpertNum) name no expert (expandIdx -1).
+ * quantMode 2: every COPY is quantised on its own, xf = float(x) * scales[e][h] when scales are given, then
+ * s = 127 / max|xf| (no epsilon, :720), q = int8(rint(xf * s)), dynamicScalesOut = 1/s (:693-733); an all-zero row
+ * gives zeros and scale 0.  quantMode 0 copies (scales ignored); 1 (static) -> CAM_ERR_UNSUPPORTED.
+ * Limits lifted: the reference accepts only epWorldSize in {8,16,32,64,128,144,256,288} and H == 7168
+ * (AK/moe_dispatch_shmem/op_host/moe_dispatch_shmem_tiling.cpp:493-501,548); here epWorldSize must be 1
+ * (sharedExpertRankNum 0, tpWorldSize <= 1) and H is a multiple of 8 in [1024, 7168].  extInfo is ignored. */
+CAM_API camStatus camMoeDispatchShmemGetWorkspaceSize(
+    const camTensor *x, const camTensor *expertIds, const camTensor *scalesOptional,
+    const camTensor *xActiveMaskOptional, int64_t epWorldSize, int64_t epRankId, int64_t moeExpertNum,
+    int64_t tpWorldSize, int64_t tpRankId, int64_t expertShardType, int64_t sharedExpertNum,
+    int64_t sharedExpertRankNum, int64_t quantMode, int64_t globalBs, int64_t expertTokenNumsType, int64_t extInfo,
+    const camTensor *expandXOut, const camTensor *dynamicScalesOut, const camTensor *expandIdxOut,
+    const camTensor *expertTokenNumsOut, const camTensor *epRecvCountOut, const camTensor *tpRecvCountOut,
+    uint64_t *workspaceSize, camOpExecutor **executor);
+CAM_API camStatus camMoeDispatchShmem(void *workspace, uint64_t workspaceSize, camOpExecutor *executor,
+                                      camStream_t stream);
+
+/* ------------------------------------------------------------------------------------------------
+ * MoeCombineShmem -- replaces aclnnMoeCombineShmem (AUTOGEN/aclnn_moe_combine_shmem.h:49-56), one rank.
+ * expandX bf16/fp16 [A,H] (the expert outputs, in MoeDispatchShmem's row order); expertIds int32 [bs,K];
+ * expandIdx int32 [bs*K] and epSendCounts int32 [moeExpertNum] as MoeDispatchShmem wrote them; expertScales
+ * fp32 [bs,K]; the six optional tensors are reserved in the reference and must be NULL -> out [bs,H] of
+ * expandX's type: out[t] = round(sum over k ascending of float(row(t,k)) * expertScales[t,k]), multiply and add
+ * rounded separately (AK/moe_combine_shmem/op_kernel/moe_combine_shmem.h:819-912), row(t,k) located as above
+ * (:514-556,:833-837).  commQuantMode 2 (bf16 rows only): every row first takes the int8 wire format of :567-592
+ * (blocks of 8 columns, bf16 scales) and is rebuilt as :755-773 before it is weighted -- the rounding a row
+ * suffers when it crosses ranks; 0: rows are used as they are.  Ids outside [0, moeExpertNum) are skipped.
+ * epWorldSize must be 1 (sharedExpertRankNum 0, tpWorldSize <= 1); the shared expert's add-back, which needs a
+ * shared-expert rank there, is available as MoeCombineGather's sharedXOptional.
+ * Workspace: bs*K int32, plus the wire rows when commQuantMode is 2. */
+CAM_API camStatus camMoeCombineShmemGetWorkspaceSize(
+    const camTensor *expandX, const camTensor *expertIds, const camTensor *expandIdx, const camTensor *epSendCounts,
+    const camTensor *expertScales, const camTensor *tpSendCountsOptional, const camTensor *xActiveMaskOptional,
+    const camTensor *activationScaleOptional, const camTensor *weightScaleOptional,
+    const camTensor *groupListOptional, const camTensor *expandScalesOptional, int64_t epWorldSize,
+    int64_t epRankId, int64_t moeExpertNum, int64_t tpWorldSize, int64_t tpRankId, int64_t expertShardType,
+    int64_t sharedExpertNum, int64_t sharedExpertRankNum, int64_t globalBs, int64_t commQuantMode, int64_t extInfo,
+    int64_t outDtype, int64_t groupListType, const camTensor *out, uint64_t *workspaceSize,
+    camOpExecutor **executor);
+CAM_API camStatus camMoeCombineShmem(void *workspace, uint64_t workspaceSize, camOpExecutor *executor,
+                                     camStream_t stream);
 
 /* ------------------------------------------------------------------------------------------------
  * PrepackWeight -- one-time weight layout conversion, off the timed path; the counterpart of
@@ -352,6 +395,7 @@ CAM_API camStatus camGroupedMatmulInt32(void *workspace, uint64_t workspaceSize,
  * (…swiglu_quant_multistage_workspace.h:647-678) -> output [bs,H] of x's type (the expert rows GMM2 writes
  * and the combined rows take it too), expertTokenNums int64 [Epr].
  * quantMode in [0, 3] is accepted and has no effect, as in the reference (fused_deep_moe.h:148,326).
+ * sharedExpertNum must be 1 (AK/fused_deep_moe/op_host/fused_deep_moe_tiling.cpp:345).
  * epRankSize must be 1 and sharedExpertRankNum 0.  Output rows of masked tokens are zero.
  * Limits kept (AK/fused_deep_moe/op_host/fused_deep_moe_tiling.cpp:49-61): 512 <= H <= 7168,
  * 1024 <= 2I <= 6144, K <= 12, moeExpertNum <= 512; H and I multiples of 128. */

@@ -572,6 +572,155 @@ ORACLE_API void cam_oracle_combine_act(const uint16_t *y, const int32_t *row_of,
     }
 }
 
+/* The combine with the shared expert's row added back (FDM/raw_distributed/cam_moe_distribute_combine.h:757-774,
+ * AK/moe_combine_shmem/op_kernel/moe_combine_shmem.h:873-907): after the K routed rows, in the same fp32
+ * accumulator, acc = acc + float(shared[t]) -- un-weighted, one rounded add -- and only then the rounding to the
+ * activation type.  shared is [T,H] in the activation type, or NULL for the plain combine. */
+ORACLE_API void cam_oracle_combine_shared(const uint16_t *y, const int32_t *row_of, const float *w,
+                                          const uint16_t *shared, int64_t T, int64_t K, int64_t H, int act,
+                                          uint16_t *out)
+{
+#pragma omp parallel for schedule(static)
+    for (int64_t t = 0; t < T; ++t) {
+        float *acc = (float *)calloc((size_t)H, sizeof(float));
+        for (int64_t k = 0; k < K; ++k) {
+            int32_t row = row_of[t * K + k];
+            if (row < 0) {
+                continue;
+            }
+            float wk = w[t * K + k];
+            const uint16_t *yr = y + (int64_t)row * H;
+            for (int64_t h = 0; h < H; ++h) {
+                float p = act_to_f32(yr[h], act) * wk;
+                acc[h] = acc[h] + p;
+            }
+        }
+        if (shared) {
+            for (int64_t h = 0; h < H; ++h) {
+                acc[h] = acc[h] + act_to_f32(shared[t * H + h], act);
+            }
+        }
+        for (int64_t h = 0; h < H; ++h) {
+            out[t * H + h] = f32_to_act(acc[h], act);
+        }
+        free(acc);
+    }
+}
+
+/* ---------------------------------------------------------------- the SHMEM operator pair on one rank
+ * Dispatch: AK/moe_dispatch_shmem/op_kernel/moe_dispatch_shmem.h.
+ *   send side (:492-549): entry i = t*K + k goes to expert e = expertIds[i]; its place inside the expert is
+ *     expertCount(i), the number of earlier flat entries with the same id, which is also what expandIdx[i]
+ *     reports (:541-548); rows are quantised per COPY, not per token, because the optional smooth scale is the
+ *     destination expert's (:693-733): xf = float(x) * smooth[e][h] (one rounded multiply), m = max |xf|,
+ *     s = 127 / m (no epsilon, :720), q = int8(rint(xf * s)), stored scale = 1 / s.  An all-zero row is
+ *     defined as q = 0, scale 0 (0 * inf in the reference).
+ *   receive side (:840-933): rows in (local expert, source rank) order, epRecvCount = inclusive running
+ *     total in that order (:853-856,:927-931); with one rank that is the inclusive prefix sum of the counts.
+ *   expertTokenNums (:1022-1051): type 0 = running total through each local expert, type 1 = per expert.
+ * quant: 0 copies the 16-bit rows (smooth is ignored, as in the reference's non-quantising instantiation),
+ * 2 quantises.  act: 0 bf16, 1 fp16.  Ids outside [0,E) name no expert: no row, expandIdx -1.
+ * Returns the number of rows written. */
+ORACLE_API int64_t cam_oracle_dispatch_shmem(const uint16_t *x, const int32_t *ids, const float *smooth,
+                                             int64_t T, int64_t K, int64_t H, int64_t E, int quant, int act,
+                                             int token_nums_type, void *out, float *scales,
+                                             int32_t *expand_idx, int64_t *expert_token_nums,
+                                             int32_t *ep_recv_count)
+{
+    int32_t *cnt = (int32_t *)calloc((size_t)E, 4);
+    for (int64_t i = 0; i < T * K; ++i) {
+        int64_t e = ids[i];
+        if (e < 0 || e >= E) {
+            expand_idx[i] = -1;
+            continue;
+        }
+        expand_idx[i] = cnt[e];
+        cnt[e] += 1;
+    }
+    int64_t run = 0;
+    for (int64_t e = 0; e < E; ++e) {
+        run += cnt[e];
+        ep_recv_count[e] = (int32_t)run;
+        expert_token_nums[e] = token_nums_type == 0 ? run : (int64_t)cnt[e];
+    }
+#pragma omp parallel for schedule(static)
+    for (int64_t i = 0; i < T * K; ++i) {
+        int64_t e = ids[i];
+        if (e < 0 || e >= E) {
+            continue;
+        }
+        const uint16_t *xr = x + (i / K) * H;
+        int64_t row = (e == 0 ? 0 : ep_recv_count[e - 1]) + expand_idx[i];
+        if (quant == 0) {
+            memcpy((uint16_t *)out + row * H, xr, (size_t)H * 2);
+            continue;
+        }
+        int8_t *q = (int8_t *)out + row * H;
+        const float *sm = smooth ? smooth + e * H : NULL;
+        float m = 0.0f;
+        for (int64_t h = 0; h < H; ++h) {
+            float v = act_to_f32(xr[h], act);
+            if (sm) {
+                v = v * sm[h];
+            }
+            float a = fabsf(v);
+            m = a > m ? a : m;
+        }
+        if (m == 0.0f) {
+            memset(q, 0, (size_t)H);
+            scales[row] = 0.0f;
+            continue;
+        }
+        float s = 127.0f / m;
+        for (int64_t h = 0; h < H; ++h) {
+            float v = act_to_f32(xr[h], act);
+            if (sm) {
+                v = v * sm[h];
+            }
+            q[h] = (int8_t)(int32_t)nearbyintf(v * s);
+        }
+        scales[row] = 1.0f / s;
+    }
+    free(cnt);
+    return run;
+}
+
+/* Combine: AK/moe_combine_shmem/op_kernel/moe_combine_shmem.h:775-917 on one rank.  The row of slot (t,k) is
+ * found from the dispatch's outputs: rows of expert e start at epSendCounts[e-1] (:514-556 walks the same
+ * running totals) and the slot's place inside them is expandIdx[t*K+k] (:833-837).  comm_quant != 0 passes every
+ * row through the int8 wire format on its way (quantise :567-592, dequantise :755-773) before it is weighted;
+ * then acc = acc + float(row) * w[t,k] for k ascending, and one rounding to the activation type (:908-912).
+ * Ids outside [0,E) are skipped (the reference does not guard them).  bf16 only when comm_quant != 0. */
+ORACLE_API void cam_oracle_combine_shmem(const uint16_t *expand_x, const int32_t *ids, const int32_t *expand_idx,
+                                         const int32_t *ep_send_counts, const float *w, int64_t A, int64_t T,
+                                         int64_t K, int64_t H, int64_t E, int act, int comm_quant, uint16_t *out)
+{
+    int32_t *row_of = (int32_t *)malloc((size_t)(T * K > 0 ? T * K : 1) * 4);
+    for (int64_t i = 0; i < T * K; ++i) {
+        int64_t e = ids[i];
+        int64_t row = -1;
+        if (e >= 0 && e < E) {
+            row = (e == 0 ? 0 : ep_send_counts[e - 1]) + expand_idx[i];
+            if (row < 0 || row >= A) {
+                row = -1;
+            }
+        }
+        row_of[i] = (int32_t)row;
+    }
+    if (comm_quant) {
+        uint8_t *wire = (uint8_t *)malloc((size_t)(A > 0 ? A : 1) * (size_t)(H + H / 4));
+        uint16_t *rows = (uint16_t *)malloc((size_t)(A > 0 ? A : 1) * (size_t)H * 2);
+        cam_oracle_comm_quant_rows(expand_x, A, H, wire);
+        cam_oracle_comm_dequant_rows(wire, A, H, rows);
+        cam_oracle_combine_shared(rows, row_of, w, NULL, T, K, H, 0, out);
+        free(wire);
+        free(rows);
+    } else {
+        cam_oracle_combine_shared(expand_x, row_of, w, NULL, T, K, H, act, out);
+    }
+    free(row_of);
+}
+
 /* row_of for the fused op: off[e] + pos (cam_moe_distribute_combine.h:737-742), -1 where idx < 0. */
 ORACLE_API void cam_oracle_rows_from_pos(const int64_t *idx, const int32_t *off, const int32_t *pos,
                                          int64_t n, int64_t E, int32_t *row_of)

@@ -225,6 +225,54 @@ def combine_act(y_bits, row_of, w, fp16):
     return out
 
 
+def combine_shared(y_bits, row_of, w, shared_bits=None, fp16=False):
+    """The combine with the shared expert's [T,H] rows added back un-weighted after the routed rows."""
+    y_bits = _c(y_bits, np.uint16)
+    row_of = _c(row_of, np.int32)
+    w = _c(w, np.float32)
+    T, K = row_of.shape
+    H = y_bits.shape[1]
+    out = np.zeros((T, H), np.uint16)
+    sh = None if shared_bits is None else _c(shared_bits, np.uint16)
+    lib().cam_oracle_combine_shared(_p(y_bits), _p(row_of), _p(w), None if sh is None else _p(sh), _i64(T), _i64(K),
+                                    _i64(H), ctypes.c_int(1 if fp16 else 0), _p(out))
+    return out
+
+
+def dispatch_shmem(x_bits, ids, E, quant, smooth=None, fp16=False, token_nums_type=1, rows=None):
+    """One rank's moe_dispatch_shmem.  -> (expand_x, scales, expand_idx, expert_token_nums, ep_recv_count, total)."""
+    x_bits = _c(x_bits, np.uint16)
+    ids = _c(ids, np.int32)
+    T, K = ids.shape
+    H = x_bits.shape[1]
+    A = T * K if rows is None else rows
+    out = np.zeros((max(A, 1), H), np.int8 if quant else np.uint16)
+    scales = np.zeros(max(A, 1), np.float32)
+    expand_idx = np.zeros(T * K, np.int32)
+    etn = np.zeros(E, np.int64)
+    rc = np.zeros(E, np.int32)
+    sm = None if smooth is None else _c(smooth, np.float32)
+    f = lib().cam_oracle_dispatch_shmem
+    f.restype = ctypes.c_int64
+    total = f(_p(x_bits), _p(ids), None if sm is None else _p(sm), _i64(T), _i64(K), _i64(H), _i64(E),
+              ctypes.c_int(quant), ctypes.c_int(1 if fp16 else 0), ctypes.c_int(token_nums_type), _p(out), _p(scales),
+              _p(expand_idx), _p(etn), _p(rc))
+    return out, scales, expand_idx, etn, rc, int(total)
+
+
+def combine_shmem(expand_x_bits, ids, expand_idx, ep_send_counts, w, E, fp16=False, comm_quant=False):
+    """One rank's moe_combine_shmem: rows located from (epSendCounts, expandIdx), optional int8 wire round trip."""
+    xb = _c(expand_x_bits, np.uint16)
+    ids = _c(ids, np.int32)
+    T, K = ids.shape
+    A, H = xb.shape
+    out = np.zeros((T, H), np.uint16)
+    lib().cam_oracle_combine_shmem(_p(xb), _p(ids), _p(_c(expand_idx, np.int32)), _p(_c(ep_send_counts, np.int32)),
+                                   _p(_c(w, np.float32)), _i64(A), _i64(T), _i64(K), _i64(H), _i64(E),
+                                   ctypes.c_int(1 if fp16 else 0), ctypes.c_int(1 if comm_quant else 0), _p(out))
+    return out
+
+
 def fused_layer_fp16(x_bits, idx, topk_w, w1, w1_scale, w2, w2_scale):
     """The int8 layer with fp16 activations in and out, composed from the stage functions."""
     idx = _c(idx, np.int64)

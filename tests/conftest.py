@@ -27,14 +27,3 @@ def gpu():
     if not torch.cuda.is_available():
         pytest.skip("no GPU")
     return torch.device("cuda:0")
-
-
-@pytest.fixture(params=["single", "separate"])
-def dispatch_launch(request, gpu):
-    """Runs a test once with the single-launch dispatch forced and once with the plan's and the permute's own
-    launches forced (small test shapes would otherwise only see the latter); restores the default afterwards."""
-    import umdk_original_amd as cam
-    cam.set_dispatch_launch_mode(cam.DISPATCH_LAUNCH_SINGLE if request.param == "single"
-                                 else cam.DISPATCH_LAUNCH_SEPARATE)
-    yield request.param
-    cam.set_dispatch_launch_mode(cam.DISPATCH_LAUNCH_AUTO)

@@ -152,9 +152,17 @@ def test_moe_dispatch_prefill_validation():
 
 def test_combine_gather_validation():
     T, K, H, A, E = 4, 2, 1024, 8, 8
-    ok = [_t((A, H), torch.bfloat16), None, _t((T, K), torch.int32), None, _t((T, K), torch.float32),
+    ok = [_t((A, H), torch.bfloat16), None, _t((T, K), torch.int32), None, _t((T, K), torch.float32), None,
           _t((T, H), torch.bfloat16)]
     assert _lib.phase1("MoeCombineGather", ok)[0] == CAM_OK
+    # the shared expert's rows: [T,H] of the output's type
+    a = list(ok)
+    a[5] = _t((T, H), torch.bfloat16)
+    assert _lib.phase1("MoeCombineGather", a)[0] == CAM_OK
+    a[5] = _t((T + 1, H), torch.bfloat16)
+    assert _lib.phase1("MoeCombineGather", a)[0] == CAM_ERR_SHAPE
+    a[5] = _t((T, H), torch.float16)
+    assert _lib.phase1("MoeCombineGather", a)[0] == CAM_ERR_DTYPE
     a = list(ok)
     a[1], a[3] = _t((3 * A,), torch.int32), _t((E,), torch.int32)
     assert _lib.phase1("MoeCombineGather", a)[0] == CAM_OK
@@ -169,6 +177,78 @@ def test_combine_gather_validation():
     assert _lib.phase1("MoeCombineGather", a)[0] == CAM_OK
     a[0] = _t((A, H), torch.int8)
     assert _lib.phase1("MoeCombineGather", a)[0] == CAM_ERR_SHAPE
+
+
+def _dispatch_shmem_args(T=4, K=2, H=1024, E=8, quant=2, dtype=torch.bfloat16):
+    A = T * K
+    return [_t((T, H), dtype), _t((T, K), torch.int32), None, None, 1, 0, E, 1, 0, 0, 1, 0, quant, 0, 1, 0,
+            _t((A, H), torch.int8 if quant == 2 else dtype), _t((A,), torch.float32), _t((T * K,), torch.int32),
+            _t((E,), torch.int64), _t((E,), torch.int32), _t((1,), torch.int32)]
+
+
+def test_dispatch_shmem_validation():
+    """Attribute and shape checks of AK/moe_dispatch_shmem/op_host/moe_dispatch_shmem_tiling.cpp:365-535 that
+    have a meaning on one rank; the transport's limits (epWorldSize list, H == 7168) are lifted."""
+    assert _lib.phase1("MoeDispatchShmem", _dispatch_shmem_args())[0] == CAM_OK
+    assert _lib.phase1("MoeDispatchShmem", _dispatch_shmem_args(quant=0))[0] == CAM_OK
+    assert _lib.phase1("MoeDispatchShmem", _dispatch_shmem_args(dtype=torch.float16))[0] == CAM_OK
+    a = _dispatch_shmem_args()
+    a[2] = _t((8, 1024), torch.float32)            # smooth scales [moeExpertNum, H]
+    assert _lib.phase1("MoeDispatchShmem", a)[0] == CAM_OK
+    a[2] = _t((9, 1024), torch.float32)
+    assert _lib.phase1("MoeDispatchShmem", a)[0] == CAM_ERR_SHAPE
+    a = _dispatch_shmem_args()
+    a[3] = _t((4,), torch.bool)                    # xActiveMask is reserved
+    assert _lib.phase1("MoeDispatchShmem", a)[0] == CAM_ERR_UNSUPPORTED
+    for pos, bad, want in ((4, 8, CAM_ERR_UNSUPPORTED),     # more than one rank needs peers
+                           (4, 0, CAM_ERR_RANGE), (5, 1, CAM_ERR_RANGE), (9, 1, CAM_ERR_RANGE),
+                           (12, 1, CAM_ERR_UNSUPPORTED),    # static quantisation
+                           (12, 3, CAM_ERR_RANGE), (14, 2, CAM_ERR_RANGE), (7, 2, CAM_ERR_UNSUPPORTED),
+                           (13, 3, CAM_ERR_RANGE)):         # globalBs below bs * ranks
+        a = _dispatch_shmem_args()
+        a[pos] = bad
+        assert _lib.phase1("MoeDispatchShmem", a)[0] == want, (pos, bad, _lib.recent_error())
+    a = _dispatch_shmem_args()
+    a[18] = _t((7,), torch.int32)                  # expandIdx holds bs * K values
+    assert _lib.phase1("MoeDispatchShmem", a)[0] == CAM_ERR_SHAPE
+    a = _dispatch_shmem_args()
+    a[16] = _t((8, 1024), torch.bfloat16)          # int8 rows when quantising
+    assert _lib.phase1("MoeDispatchShmem", a)[0] == CAM_ERR_DTYPE
+    a = _dispatch_shmem_args()
+    a[19] = _t((7,), torch.int64)
+    assert _lib.phase1("MoeDispatchShmem", a)[0] == CAM_ERR_SHAPE
+
+
+def _combine_shmem_args(T=4, K=2, H=1024, E=8, A=8, comm=0, dtype=torch.bfloat16):
+    return [_t((A, H), dtype), _t((T, K), torch.int32), _t((T * K,), torch.int32), _t((E,), torch.int32),
+            _t((T, K), torch.float32), None, None, None, None, None, None, 1, 0, E, 1, 0, 0, 1, 0, 0, comm, 0, 0, 0,
+            _t((T, H), dtype)]
+
+
+def test_combine_shmem_validation():
+    """AK/moe_combine_shmem/op_host/moe_combine_shmem_tiling.cpp:120-200 on one rank."""
+    st, ws0, _ = _lib.phase1("MoeCombineShmem", _combine_shmem_args())
+    assert st == CAM_OK and ws0 >= 4 * 2 * 4
+    st, ws2, _ = _lib.phase1("MoeCombineShmem", _combine_shmem_args(comm=2))
+    assert st == CAM_OK and ws2 >= ws0 + 8 * (1024 + 256)  # the wire rows live in the workspace
+    assert _lib.phase1("MoeCombineShmem", _combine_shmem_args(dtype=torch.float16))[0] == CAM_OK
+    assert _lib.phase1("MoeCombineShmem", _combine_shmem_args(comm=2, dtype=torch.float16))[0] == CAM_ERR_UNSUPPORTED
+    assert _lib.phase1("MoeCombineShmem", _combine_shmem_args(comm=1))[0] == CAM_ERR_RANGE
+    for pos in (6, 7, 8, 9, 10):  # reserved inputs
+        a = _combine_shmem_args()
+        a[pos] = _t((4,), torch.float32)
+        assert _lib.phase1("MoeCombineShmem", a)[0] == CAM_ERR_UNSUPPORTED
+    for pos, bad, want in ((11, 8, CAM_ERR_UNSUPPORTED), (12, 1, CAM_ERR_RANGE), (16, 1, CAM_ERR_RANGE),
+                           (18, 1, CAM_ERR_RANGE), (14, 2, CAM_ERR_UNSUPPORTED)):
+        a = _combine_shmem_args()
+        a[pos] = bad
+        assert _lib.phase1("MoeCombineShmem", a)[0] == want, (pos, bad, _lib.recent_error())
+    a = _combine_shmem_args()
+    a[2] = _t((7,), torch.int32)
+    assert _lib.phase1("MoeCombineShmem", a)[0] == CAM_ERR_SHAPE
+    a = _combine_shmem_args()
+    a[24] = _t((4, 1024), torch.float16)
+    assert _lib.phase1("MoeCombineShmem", a)[0] == CAM_ERR_DTYPE
 
 
 def _packed(shape):
@@ -353,15 +433,6 @@ def test_fp8_operator_validation():
     assert _lib.phase1("MoeDispatchPrefill", pre)[0] != CAM_OK          # int8 rows / fp32 scales do not fit
 
 
-def test_dispatch_launch_mode_setter_range():
-    from umdk_original_amd import _lib
-    h = _lib.lib()
-    for mode in (1, 2, 0):
-        assert h.camSetDispatchLaunchMode(mode) == 0
-    assert h.camSetDispatchLaunchMode(3) != 0 and "mode" in _lib.recent_error()
-    assert h.camSetDispatchLaunchMode(-1) != 0
-
-
 def test_torch_operator_library_is_built_and_registers_the_reference_schemas():
     import os
     from umdk_original_amd import ops
@@ -369,7 +440,33 @@ def test_torch_operator_library_is_built_and_registers_the_reference_schemas():
     assert os.path.exists(path), "python -m umdk_original_amd.build builds it"
     assert ops._torch_lib == "cpp"
     for name in ("fused_deep_moe", "get_dispatch_layout", "moe_dispatch_prefill", "moe_combine_prefill",
-                 "prepack_weight"):
+                 "moe_dispatch_shmem", "moe_combine_shmem", "prepack_weight"):
         assert hasattr(torch.ops.umdk_cam_op_lib, name)
     s = str(torch.ops.umdk_cam_op_lib.moe_combine_prefill.default._schema)
     assert "Tensor send_head, str group_ep, int rank, int num_ranks" in s
+    s = str(torch.ops.umdk_cam_op_lib.moe_dispatch_shmem.default._schema)
+    assert "Tensor? scales, Tensor? xActiveMask, int epWorldSize, int epRankId, int moeExpertNum" in s
+    s = str(torch.ops.umdk_cam_op_lib.moe_combine_shmem.default._schema)
+    assert "int globalBS, int commQuantMode, int extInfo, int outDtype, int groupListType) -> Tensor" in s
+
+
+def test_torch_operators_have_autograd_and_meta_registrations():
+    """As in the reference: every operator sits on the autograd key too (backward returns no gradients,
+    src/cam/comm_operator/pybind/fused_deep_moe.cpp:152-229), and the operators whose shapes follow from their
+    arguments have Meta implementations (…/moe_dispatch_shmem.cpp:153-190, …/moe_combine_shmem.cpp:88-123)."""
+    for name in ("fused_deep_moe", "get_dispatch_layout", "moe_dispatch_prefill", "moe_combine_prefill",
+                 "moe_dispatch_shmem", "moe_combine_shmem"):
+        assert torch._C._dispatch_has_kernel_for_dispatch_key("umdk_cam_op_lib::" + name, "AutogradCUDA"), name
+        assert torch._C._dispatch_has_kernel_for_dispatch_key("umdk_cam_op_lib::" + name, "CUDA"), name
+    ops = torch.ops.umdk_cam_op_lib
+    x = torch.empty((6, 2048), dtype=torch.bfloat16, device="meta")
+    ids = torch.empty((6, 4), dtype=torch.int32, device="meta")
+    d = ops.moe_dispatch_shmem(x, ids, None, None, 1, 0, 16, 1, 0, 0, 1, 0, 2, 0, 1, 0)
+    assert [tuple(t.shape) for t in d] == [(24, 2048), (24,), (24,), (16,), (16,), (1,)]
+    assert d[0].dtype == torch.int8 and d[1].dtype == torch.float32 and d[3].dtype == torch.int64
+    d0 = ops.moe_dispatch_shmem(x, ids, None, None, 1, 0, 2, 1, 0, 0, 1, 0, 0, 0, 1, 0)
+    assert tuple(d0[0].shape) == (12, 2048) and d0[0].dtype == torch.bfloat16   # bs * min(K, experts) rows
+    w = torch.empty((6, 4), dtype=torch.float32, device="meta")
+    out = ops.moe_combine_shmem(torch.empty((24, 2048), dtype=torch.bfloat16, device="meta"), ids, d[2], d[4], w, None,
+                                None, None, None, None, None, 1, 0, 16, 1, 0, 0, 1, 0, 0, 0, 0, 0, 0)
+    assert tuple(out.shape) == (6, 2048) and out.dtype == torch.bfloat16

@@ -202,3 +202,38 @@ def test_combine_fp16_rows_bit_exact(gpu, oracle):
     got = cam.moe_combine_gather(y.to(gpu), None, torch.from_numpy(row_of.reshape(T, K)).to(gpu), w.to(gpu))
     assert got.dtype == torch.float16
     assert_bits_equal(got.cpu().view(torch.int16).numpy().view(np.uint16), want, "combined fp16 x")
+
+
+@pytest.mark.parametrize("T,K,E,H,wire,fp16", [(33, 8, 64, 7168, False, False), (21, 3, 8, 1032, False, False),
+                                                 (57, 16, 32, 4096, True, False), (19, 4, 8, 1032, True, False),
+                                                 (40, 8, 32, 2048, False, True)])
+def test_combine_with_shared_expert_rows(gpu, oracle, T, K, E, H, wire, fp16):
+    """The shared expert's row is added un-weighted after the routed rows, before the one rounding
+    (cam_moe_distribute_combine.h:757-774), for 16-bit rows of either type and for wire rows."""
+    announce("combine + shared rows T=%d K=%d E=%d H=%d wire=%d fp16=%d" % (T, K, E, H, wire, fp16))
+    ids, w = synth.sigmoid_zipf_routing(T, E, K, seed=T)
+    idx_np = ids.numpy()
+    idx_np[T // 2, 0] = -1  # an absent slot; and one token with no routed rows at all
+    idx_np[0, :] = -1
+    cnt, off, pos, _ = plan_oracle(oracle, idx_np, E)
+    A = T * K
+    row_of = oracle.rows_from_pos(idx_np, off, pos, E)
+    y = synth.normal_bf16(A, H, seed=T + 1)
+    sh = synth.normal_bf16(T, H, seed=T + 2)
+    if fp16:
+        y, sh = y.half(), sh.half()
+        yb, sb = y.view(torch.int16).numpy().view(np.uint16), sh.view(torch.int16).numpy().view(np.uint16)
+    else:
+        yb, sb = synth.bf16_bits(y), synth.bf16_bits(sh)
+    slot = torch.from_numpy(row_of.reshape(T, K)).to(gpu)
+    if wire:
+        packed = oracle.comm_quant_rows(yb)
+        want = oracle.combine_shared(oracle.comm_dequant_rows(packed, H), row_of, w.numpy(), sb)
+        got = cam.moe_combine_gather(torch.from_numpy(packed.view(np.int8)).to(gpu), None, slot, w.to(gpu),
+                                     shared_x=sh.to(gpu))
+    else:
+        want = oracle.combine_shared(yb, row_of, w.numpy(), sb, fp16=fp16)
+        got = cam.moe_combine_gather(y.to(gpu), None, slot, w.to(gpu), shared_x=sh.to(gpu))
+    gb = got.cpu().view(torch.int16).numpy().view(np.uint16)
+    assert_bits_equal(gb, want, "combined x with shared rows")
+    assert np.array_equal(gb[0], sb[0])  # no routed rows: the shared row alone, bit for bit

@@ -229,8 +229,8 @@ def _check_fused(oracle, d, x, idx_np, E, quant_mode, fp16=False):
     (300, 8, 256, 7168, torch.int64, 0.0),     # two chunks of 2048 ids
     (1500, 16, 512, 1032, torch.int64, 0.05),  # twelve chunks, odd row length
 ])
-def test_dispatch_prefill_operator(gpu, oracle, dispatch_launch, T, K, E, H, dtype, neg, quant_mode):
-    announce("dispatch prefill (%s) T=%d K=%d E=%d H=%d quant=%d" % (dispatch_launch, T, K, E, H, quant_mode))
+def test_dispatch_prefill_operator(gpu, oracle, T, K, E, H, dtype, neg, quant_mode):
+    announce("dispatch prefill T=%d K=%d E=%d H=%d quant=%d" % (T, K, E, H, quant_mode))
     ids = _random_ids(T, K, E, seed=T + K + E, neg_frac=neg, dtype=dtype)
     x = synth.normal_bf16(T, H, seed=T + 3)
     if T > 4:
@@ -239,9 +239,9 @@ def test_dispatch_prefill_operator(gpu, oracle, dispatch_launch, T, K, E, H, dty
     _check_fused(oracle, d, x, ids.numpy().astype(np.int64), E, quant_mode)
 
 
-def test_dispatch_prefill_workspace_reuse_and_garbage(gpu, oracle, dispatch_launch):
+def test_dispatch_prefill_workspace_reuse_and_garbage(gpu, oracle):
     """The same workspace, first filled with arbitrary bytes, serves several launches with different routings."""
-    announce("dispatch prefill workspace reuse (%s)" % dispatch_launch)
+    announce("dispatch prefill workspace reuse")
     from umdk_original_amd import _lib
     T, K, E, H = 513, 8, 64, 2048
     ws = torch.full((1 << 20,), 0xA5, dtype=torch.uint8, device=gpu)
@@ -266,8 +266,8 @@ def test_dispatch_prefill_workspace_reuse_and_garbage(gpu, oracle, dispatch_laun
         _check_fused(oracle, d, x, ids.numpy(), E, 2)
 
 
-def test_dispatch_prefill_full_size_config(gpu, oracle, dispatch_launch):
-    announce("dispatch prefill C2 full size (%s)" % dispatch_launch)
+def test_dispatch_prefill_full_size_config(gpu, oracle):
+    announce("dispatch prefill C2 full size")
     T, K, E, H = 4096, 8, 256, 7168
     ids, _ = synth.sigmoid_zipf_routing(T, E, K, seed=44)
     x = synth.normal_bf16(T, H, seed=44)
@@ -278,9 +278,9 @@ def test_dispatch_prefill_full_size_config(gpu, oracle, dispatch_launch):
 
 
 @pytest.mark.parametrize("quant_mode", [0, 2, 3])
-def test_dispatch_fp16_activations(gpu, oracle, dispatch_launch, quant_mode):
+def test_dispatch_fp16_activations(gpu, oracle, quant_mode):
     """fp16 activations (moe_dispatch_normal.cpp op_host :17-22 lists them beside bf16), both dispatch operators."""
-    announce("dispatch fp16 quant=%d (%s)" % (quant_mode, dispatch_launch))
+    announce("dispatch fp16 quant=%d (%s)" % (quant_mode))
     T, K, E, H = 70, 4, 16, 2048
     ids = _random_ids(T, K, E, seed=61, neg_frac=0.1)
     x = (torch.randn(T, H, generator=torch.Generator().manual_seed(62)) * 4).half()

@@ -30,7 +30,7 @@ def _u8(t):
     return t.view(torch.uint8).cpu().numpy()
 
 
-def test_dispatch_fp8_rows_and_scales_bit_exact(gpu, oracle, dispatch_launch):
+def test_dispatch_fp8_rows_and_scales_bit_exact(gpu, oracle):
     announce("fp8 dispatch T=77 H=4096")
     T, H, E, K = 77, 4096, 16, 4
     ids, _ = synth.sigmoid_zipf_routing(T, E, K, seed=3)
@@ -51,7 +51,7 @@ def test_dispatch_fp8_rows_and_scales_bit_exact(gpu, oracle, dispatch_launch):
             assert np.array_equal(rs[r], sc[t]), (t, k)
 
 
-def test_dispatch_fp8_from_fp16_activations(gpu, oracle, dispatch_launch):
+def test_dispatch_fp8_from_fp16_activations(gpu, oracle):
     announce("fp8 dispatch from fp16")
     T, H, E, K = 33, 1024, 8, 2
     ids, _ = synth.sigmoid_zipf_routing(T, E, K, seed=5)
@@ -177,7 +177,7 @@ def _check_layer(got, want_bits):
 
 
 @pytest.mark.parametrize("T,H,E,K,I", [(64, 1024, 8, 2, 512), (200, 2048, 16, 4, 768)])
-def test_fused_layer_fp8_against_oracle(gpu, oracle, dispatch_launch, T, H, E, K, I):
+def test_fused_layer_fp8_against_oracle(gpu, oracle, T, H, E, K, I):
     announce("fp8 fused layer T=%d H=%d E=%d K=%d I=%d" % (T, H, E, K, I))
     ids, w, x, w1, s1, w2, s2 = _layer_inputs(T, H, E, K, I, seed=T)
     out, etn = cam.fused_deep_moe_fp8(x.to(gpu), ids.to(torch.int32).to(gpu), cam.prepack_weight(w1.to(gpu), True),

@@ -51,7 +51,7 @@ def _check(oracle, d, out, etn, n_active=None):
     return mism
 
 
-def test_fused_cpu_golden_config(gpu, oracle, dispatch_launch):
+def test_fused_cpu_golden_config(gpu, oracle):
     """128 tokens, hidden 1024, 8 experts, softmax top-2, intermediate 512."""
     announce("fused C1")
     T, H, E, K, I = 128, 1024, 8, 2, 512
@@ -63,7 +63,7 @@ def test_fused_cpu_golden_config(gpu, oracle, dispatch_launch):
     assert _check(oracle, d, out, etn) == 0
 
 
-def test_fused_reference_unit_test_case(gpu, oracle, dispatch_launch):
+def test_fused_reference_unit_test_case(gpu, oracle):
     """The reference's CASE_4RANK shape collapsed onto one rank: E=16, K=8, bs=16, H=7168, I=2048."""
     announce("fused UT recipe")
     d = synth.ut_recipe(batch_size=16, hidden=7168, intermediate=2048, num_experts=16, top_k=8, seed=42)
@@ -75,7 +75,7 @@ def test_fused_reference_unit_test_case(gpu, oracle, dispatch_launch):
     torch.testing.assert_close(out.float().cpu(), synth.bits_to_bf16(want).float(), atol=2.0, rtol=0.02)
 
 
-def test_fused_active_mask_and_tensor_lists(gpu, oracle, dispatch_launch):
+def test_fused_active_mask_and_tensor_lists(gpu, oracle):
     announce("fused mask + per-expert weights")
     d = synth.ut_recipe(batch_size=40, hidden=1024, intermediate=512, num_experts=8, top_k=4, seed=7)
     mask = torch.zeros(40, dtype=torch.bool)
@@ -85,10 +85,10 @@ def test_fused_active_mask_and_tensor_lists(gpu, oracle, dispatch_launch):
     assert (out[23:] == 0).all()
 
 
-def test_fused_active_mask_over_several_ranking_chunks(gpu, oracle, dispatch_launch):
+def test_fused_active_mask_over_several_ranking_chunks(gpu, oracle):
     """2800 routing entries (two ranking chunks), the active prefix ends inside a workgroup's four tokens and
     inside the first chunk's neighbour: the plan must stop counting at the prefix in every launch form."""
-    announce("fused mask, several ranking chunks (%s)" % dispatch_launch)
+    announce("fused mask, several ranking chunks")
     d = synth.ut_recipe(batch_size=700, hidden=1024, intermediate=512, num_experts=16, top_k=4, seed=9)
     mask = torch.zeros(700, dtype=torch.bool)
     mask[:601] = True
@@ -97,7 +97,7 @@ def test_fused_active_mask_over_several_ranking_chunks(gpu, oracle, dispatch_lau
     assert (out[601:] == 0).all()
 
 
-def test_fused_negative_ids_and_skew(gpu, oracle, dispatch_launch):
+def test_fused_negative_ids_and_skew(gpu, oracle):
     announce("fused skewed routing with dropped entries")
     T, H, E, K, I = 300, 1024, 32, 6, 512
     ids, gates = synth.sigmoid_zipf_routing(T, E, K, seed=8, bias_scale=2.0)
@@ -109,7 +109,7 @@ def test_fused_negative_ids_and_skew(gpu, oracle, dispatch_launch):
     assert _check(oracle, d, out, etn) == 0
 
 
-def test_fused_layer_fp16_activations(gpu, oracle, dispatch_launch):
+def test_fused_layer_fp16_activations(gpu, oracle):
     """fp16 tokens in, fp16 out (the reference lists both 16-bit types,
     fused_deep_moe.cpp(op_host):22-24): quantisation reads fp16, GMM2 and the combine write fp16."""
     announce("fused layer, fp16 activations")

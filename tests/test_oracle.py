@@ -705,3 +705,139 @@ def test_fp16_activation_variants_of_gmm2_epilogue_and_combine(oracle):
             if row_of[t, k] >= 0:
                 acc[t] = acc[t] + (yf[row_of[t, k]] * w[t, k]).astype(np.float32)
     assert np.array_equal(got, acc.astype(np.float16).view(np.uint16))
+
+
+# ------------------------------------------------------------------ shared expert add-back
+def test_combine_shared_row_is_added_last_and_unweighted(oracle):
+    rng = _rng(91)
+    T, K, H, A = 5, 4, 32, 24
+    y = torch.from_numpy(rng.normal(0, 1, size=(A, H)).astype(np.float32)).bfloat16()
+    sh = torch.from_numpy(rng.normal(0, 1, size=(T, H)).astype(np.float32)).bfloat16()
+    row_of = rng.permutation(A)[: T * K].reshape(T, K).astype(np.int32)
+    row_of[1, 2] = -1
+    w = rng.uniform(0, 2, size=(T, K)).astype(np.float32)
+    out = oracle.combine_shared(synth.bf16_bits(y), row_of, w, synth.bf16_bits(sh))
+    # independent numpy float32 restatement: routed rows in k order, then the shared row, then ONE rounding
+    yf, acc = y.float().numpy(), np.zeros((T, H), np.float32)
+    for k in range(K):
+        ok = (row_of[:, k] >= 0)[:, None]
+        acc = np.where(ok, acc + yf[np.maximum(row_of[:, k], 0)] * w[:, k][:, None], acc)
+    acc = acc + sh.float().numpy()
+    assert np.array_equal(out, synth.bf16_bits(torch.from_numpy(acc).bfloat16()))
+    # no shared rows -> the plain combine
+    assert np.array_equal(oracle.combine_shared(synth.bf16_bits(y), row_of, w), oracle.combine(synth.bf16_bits(y), row_of, w))
+    # no routed rows at all -> the shared rows come back bit for bit (un-weighted: a weight would change them)
+    none = np.full((T, K), -1, np.int32)
+    assert np.array_equal(oracle.combine_shared(synth.bf16_bits(y), none, w, synth.bf16_bits(sh)), synth.bf16_bits(sh))
+
+
+def test_combine_shared_order_and_single_rounding_witnesses(oracle):
+    """(a + b) + s with s last differs from (s + a) + b here, and rounding the routed sum to bf16 before adding
+    the shared row differs from rounding once at the end."""
+    H = 8
+    big, small = 2.0 ** 24, 1.0
+    rows = synth.bf16_bits(torch.tensor([[big] * H, [small] * H]).bfloat16())
+    shared = synth.bf16_bits(torch.tensor([[-big] * H]).bfloat16())
+    w = np.ones((1, 2), np.float32)
+    out = oracle.bf16_bits_to_f32(oracle.combine_shared(rows, np.array([[0, 1]], np.int32), w, shared))
+    # routed first: 2^24 + 1 rounds to 2^24 in fp32, minus 2^24 -> 0; shared first would leave 1
+    assert (out == 0.0).all()
+    # single rounding: 1 + 2^-9 is not a bf16 value; with the shared row -1 the exact fp32 sum 2^-9 survives,
+    # while a bf16 rounding of the routed sum (-> 1.0) first would give 0
+    a = synth.bf16_bits(torch.tensor([[1.0] * H, [2.0 ** -9] * H]).bfloat16())
+    sh = synth.bf16_bits(torch.tensor([[-1.0] * H]).bfloat16())
+    out = oracle.bf16_bits_to_f32(oracle.combine_shared(a, np.array([[0, 1]], np.int32), w, sh))
+    assert (out == np.float32(2.0 ** -9)).all()
+
+
+# ------------------------------------------------------------------ the SHMEM operator pair on one rank
+@pytest.mark.parametrize("T,K,E,H", [(1, 1, 1, 16), (37, 4, 8, 64), (64, 8, 32, 128)])
+def test_dispatch_shmem_bookkeeping_closed_forms(oracle, T, K, E, H):
+    rng = _rng(7 * T + E)
+    ids = rng.integers(-1, E + 1, size=(T, K)).astype(np.int32)  # -1 and E name no expert
+    x = torch.from_numpy(rng.normal(0, 1, size=(T, H)).astype(np.float32)).bfloat16()
+    xb = synth.bf16_bits(x)
+    for ttype in (0, 1):
+        out, _, eidx, etn, rc, total = oracle.dispatch_shmem(xb, ids, E, 0, token_nums_type=ttype)
+        flat = ids.ravel()
+        ok = (flat >= 0) & (flat < E)
+        cnt = np.bincount(flat[ok], minlength=E)
+        assert total == ok.sum()
+        assert np.array_equal(rc, np.cumsum(cnt).astype(np.int32))           # inclusive running totals
+        assert np.array_equal(etn, np.cumsum(cnt) if ttype == 0 else cnt)    # type 0 cumulative, 1 per expert
+        # expandIdx: number of earlier flat entries with the same id (brute force)
+        want = np.array([-1 if not ok[i] else int((flat[:i] == flat[i]).sum()) for i in range(flat.size)], np.int32)
+        assert np.array_equal(eidx, want)
+        # rows: the stable sort of the valid entries by expert; row r holds the token of the r-th sorted entry
+        order = np.argsort(np.where(ok, flat, E), kind="stable")[: ok.sum()]
+        assert np.array_equal(out[:total], xb[order // K])
+        rows = np.where(ok, np.concatenate([[0], np.cumsum(cnt)])[np.clip(flat, 0, E - 1)] + eidx, -1)
+        assert np.array_equal(np.sort(rows[ok]), np.arange(total))
+
+
+def test_dispatch_shmem_quant_and_smooth_scales(oracle):
+    rng = _rng(5)
+    T, K, E, H = 20, 3, 6, 64
+    ids = np.stack([rng.permutation(E)[:K] for _ in range(T)]).astype(np.int32)
+    x = torch.from_numpy(rng.normal(0, 2, size=(T, H)).astype(np.float32)).bfloat16()
+    x[3] = 0  # an all-zero token: zeros and scale 0 by definition
+    xb = synth.bf16_bits(x)
+    # without smooth scales every copy equals the token's no-epsilon quantisation (variant 2)
+    q, sc, eidx, _, rc, total = oracle.dispatch_shmem(xb, ids, E, 2)
+    q2, s2 = oracle.quant_rows(xb, 2)
+    start = np.concatenate([[0], rc[:-1]])
+    rows = start[ids.ravel()] + eidx
+    assert np.array_equal(q[rows], np.repeat(q2, K, axis=0)) and np.array_equal(sc[rows], np.repeat(s2, K))
+    assert (q[rows[3 * K:4 * K]] == 0).all() and (sc[rows[3 * K:4 * K]] == 0).all()
+    # smooth scales of all ones change nothing; powers of two leave q alone and scale the stored scale exactly
+    ones = np.ones((E, H), np.float32)
+    q1, s1 = oracle.dispatch_shmem(xb, ids, E, 2, smooth=ones)[:2]
+    assert np.array_equal(q1, q) and np.array_equal(s1, sc)
+    pw = (2.0 ** rng.integers(-3, 4, size=E)).astype(np.float32)
+    qp, sp = oracle.dispatch_shmem(xb, ids, E, 2, smooth=np.repeat(pw[:, None], H, 1))[:2]
+    assert np.array_equal(qp, q)
+    assert np.array_equal(sp[rows], (sc[rows] * np.repeat(pw[None, :], T, 0)[np.arange(T)[:, None], ids].ravel()))
+    # general smooth scales: independent numpy float32 restatement, copy by copy
+    sm = rng.uniform(0.25, 4.0, size=(E, H)).astype(np.float32)
+    qs, ss = oracle.dispatch_shmem(xb, ids, E, 2, smooth=sm)[:2]
+    xf = x.float().numpy()
+    for t in range(T):
+        for k in range(K):
+            e = ids[t, k]
+            v = (xf[t] * sm[e]).astype(np.float32)                    # one rounded multiply
+            m = np.abs(v).max()
+            r = rows[t * K + k]
+            if m == 0:
+                assert (qs[r] == 0).all() and ss[r] == 0
+                continue
+            s = np.float32(127.0) / m
+            assert np.array_equal(qs[r], np.rint((v * s).astype(np.float32)).astype(np.int8))
+            assert ss[r] == np.float32(1.0) / s
+            assert np.abs(qs[r]).max() == 127
+    # the copies of one token now differ (the scale row is the destination expert's)
+    assert not np.array_equal(qs[rows[0]], qs[rows[1]])
+
+
+def test_combine_shmem_locates_rows_like_the_dispatch_and_applies_the_wire_rounding(oracle):
+    rng = _rng(6)
+    T, K, E, H = 24, 4, 8, 64
+    ids = np.stack([rng.permutation(E + 1)[:K] - 1 for _ in range(T)]).astype(np.int32)  # some -1
+    x = torch.from_numpy(rng.normal(0, 1, size=(T, H)).astype(np.float32)).bfloat16()
+    _, _, eidx, _, rc, total = oracle.dispatch_shmem(synth.bf16_bits(x), ids, E, 0)
+    y = torch.from_numpy(rng.normal(0, 1, size=(total, H)).astype(np.float32)).bfloat16()
+    yb = synth.bf16_bits(y)
+    w = rng.uniform(0, 1, size=(T, K)).astype(np.float32)
+    out = oracle.combine_shmem(yb, ids, eidx, rc, w, E)
+    # the same rows as the plan-based map (offset of the expert + place inside it), then the plain combine
+    cnt = np.bincount(ids[ids >= 0], minlength=E).astype(np.int32)
+    off, _ = oracle.offsets(cnt, T)
+    row_of = oracle.rows_from_pos(ids.astype(np.int64), off, eidx.reshape(T, K), E)
+    assert np.array_equal(out, oracle.combine(yb, row_of, w))
+    # K = 1, weight 1: combine(dispatch(x)) == x, the un-permute round trip
+    ids1 = rng.integers(0, E, size=(T, 1)).astype(np.int32)
+    rows1, _, e1, _, rc1, _ = oracle.dispatch_shmem(synth.bf16_bits(x), ids1, E, 0)
+    assert np.array_equal(oracle.combine_shmem(rows1, ids1, e1, rc1, np.ones((T, 1), np.float32), E), synth.bf16_bits(x))
+    # commQuantMode 2: every row first goes through the int8 wire format
+    wired = oracle.comm_dequant_rows(oracle.comm_quant_rows(yb), H)
+    assert np.array_equal(oracle.combine_shmem(yb, ids, eidx, rc, w, E, comm_quant=True), oracle.combine(wired, row_of, w))
+    assert not np.array_equal(wired, yb)

@@ -9,9 +9,8 @@ from .ops import (CamError, fused_deep_moe, fused_deep_moe_fp8, get_dispatch_lay
                   grouped_matmul_fp8, grouped_matmul_int32, quant_rows_fp8,
                   grouped_matmul_swiglu_quant, moe_combine_gather, moe_combine_index, moe_combine_normal,
                   moe_combine_prefill, moe_dispatch_fused, moe_dispatch_normal,
-                  moe_dispatch_plan, moe_dispatch_prefill, notify_dispatch, prepack_weight, register_torch_ops,
-                  set_dispatch_launch_mode, DISPATCH_LAUNCH_AUTO, DISPATCH_LAUNCH_SINGLE,
-                  DISPATCH_LAUNCH_SEPARATE)
+                  moe_dispatch_plan, moe_dispatch_prefill, moe_dispatch_shmem, moe_combine_shmem, notify_dispatch,
+                  prepack_weight, register_torch_ops)
 
 __version__ = "0.1.0"
 

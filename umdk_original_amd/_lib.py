@@ -7,6 +7,7 @@ allocates the workspace, phase 2 enqueues on the current stream.
 
 There is no fallback: if the shared library is missing or a call fails, an exception is raised.
 """
+import contextlib
 import ctypes
 import os
 
@@ -98,7 +99,9 @@ SIGNATURES = {
                           _TP, _TP, _TP],
     "MoeCombineNormal": [_TP, _TP, _TP, _TP, _TP, _STR, _I64, _I64, _STR, _I64, _I64, _I64, _I64, _TP],
     "MoeCombineIndex": [_TP, _I64, _TP],
-    "MoeCombineGather": [_TP, _TP, _TP, _TP, _TP, _TP],
+    "MoeCombineGather": [_TP, _TP, _TP, _TP, _TP, _TP, _TP],
+    "MoeDispatchShmem": [_TP, _TP, _TP, _TP] + [_I64] * 12 + [_TP] * 6,
+    "MoeCombineShmem": [_TP] * 11 + [_I64] * 13 + [_TP],
     "PrepackWeight": [_TP, _I64, _TP],
     "GroupedMatmulSwigluQuant": [_TP, _TP, _LP, _LP, _TP, _I64, _TP, _TP],
     "GroupedMatmulDequant": [_TP, _TP, _LP, _LP, _TP, _I64, _TP],
@@ -115,7 +118,7 @@ DIRECT_SIGNATURES = {
     "MoeDispatchPlanNoAlloc": [_TP, _I64, _I64, _I64, _TP, _TP, _TP, _TP, _TP, _TP, _TP, _TP],
 }
 
-EXPORTS = ["camGetRecentErrMsg", "camDestroyExecutor", "camGetVersion", "camSetDispatchLaunchMode"] + [
+EXPORTS = ["camGetRecentErrMsg", "camDestroyExecutor", "camGetVersion"] + [
     "cam%s" % op for op in DIRECT_SIGNATURES] + [
     "cam%s%s" % (op, suffix) for op in SIGNATURES for suffix in ("GetWorkspaceSize", "")
 ]
@@ -135,8 +138,6 @@ def lib():
         handle.camGetRecentErrMsg.restype = ctypes.c_char_p
         handle.camGetVersion.restype = ctypes.c_char_p
         handle.camDestroyExecutor.argtypes = [ctypes.c_void_p]
-        handle.camSetDispatchLaunchMode.argtypes = [ctypes.c_int32]
-        handle.camSetDispatchLaunchMode.restype = ctypes.c_int32
         for op, argtypes in SIGNATURES.items():
             f1 = getattr(handle, "cam%sGetWorkspaceSize" % op)
             f1.argtypes = argtypes + _PHASE1_TAIL
@@ -272,7 +273,9 @@ def call_direct(op, args, stream=None):
             cargs.append(int(a))
     if stream is None:
         stream = torch.cuda.current_stream(device).cuda_stream if device is not None else 0
-    st = getattr(handle, "cam%s" % op)(*cargs, ctypes.c_void_p(stream))
+    # a single-call entry point resolves library-owned device memory for the CURRENT device
+    with torch.cuda.device(device) if device is not None else contextlib.nullcontext():
+        st = getattr(handle, "cam%s" % op)(*cargs, ctypes.c_void_p(stream))
     if st != CAM_OK:
         raise CamError(st, recent_error())
 

@@ -8,7 +8,7 @@ _PKG = os.path.dirname(os.path.abspath(__file__))
 _CSRC = os.path.join(_PKG, "csrc")
 LIB_DIR = os.path.join(_PKG, "lib")
 LIB_PATH = os.path.join(LIB_DIR, "libcam_mi355x.so")
-SOURCES = ["abi.cpp", "plan.hip", "dispatch.hip", "dispatch_fused.hip", "combine.hip", "gemm.hip"]
+SOURCES = ["abi.cpp", "plan.hip", "dispatch.hip", "combine.hip", "gemm.hip"]
 
 # -packed-fp32-ops is switched off on purpose: packed fp32 VALU forms are not used by this library.
 HIPCC_FLAGS = [

@@ -9,7 +9,6 @@
 //   AK/fused_deep_moe/op_host/fused_deep_moe_tiling.cpp:49-61,83-348
 //   src/cam/comm_operator/pybind/moe_dispatch_prefill.cpp:44-70
 #include <algorithm>
-#include <atomic>
 #include <cstdarg>
 #include <cstdio>
 #include <cstring>
@@ -54,7 +53,9 @@ enum OpTag {
     kOpFused = 0x46555345,
     kOpGmmFp8 = 0x474d4638,
     kOpQuantFp8 = 0x51544638,
-    kOpFusedFp8 = 0x46554638
+    kOpFusedFp8 = 0x46554638,
+    kOpDispShmem = 0x4453484d,
+    kOpCombShmem = 0x4353484d
 };
 
 constexpr uint64_t kAlign = 256;
@@ -297,35 +298,11 @@ cam::SchedSpec sched_spec(int64_t rows, int64_t G, int64_t N)
     return sp;
 }
 
-std::atomic<int32_t> g_dispatch_launch_mode{CAM_DISPATCH_LAUNCH_AUTO};
-
-// One launch for plan + permute (dispatch_fused.hip), or the plan's launches and then the permute's.  Measured
-// (int8 rows, top-8, microseconds single / separate): 1024 x 7168: 24.1 / 20.9, 2048 x 7168: 39.7 / 33.4,
-// 4096 x 4096: 40.2 / 38.3, 4096 x 7168: 61.0 / 59.4, 8192 x 4096: 105.7 / 77.4, 8192 x 7168: 132.6 / 126.8.  The
-// single launch saves two launch latencies but its token workgroups sit idle until the ranking is through and
-// read the hand-over tables past the L2; since the permute keeps four workgroups per CU resident the separate
-// form is ahead at every size, and in a fused layer its permute launch also builds the GEMM schedules.  The
-// single launch therefore runs only when it is asked for.
-bool single_launch_dispatch(int64_t T, int64_t K)
-{
-    return g_dispatch_launch_mode.load(std::memory_order_relaxed) == CAM_DISPATCH_LAUNCH_SINGLE &&
-           cam::fused_dispatch_fits(T, K);
-}
-
 }  // namespace
 
 extern "C" {
 
 const char *camGetRecentErrMsg(void) { return g_err.c_str(); }
-
-camStatus camSetDispatchLaunchMode(int32_t mode)
-{
-    if (mode < CAM_DISPATCH_LAUNCH_AUTO || mode > CAM_DISPATCH_LAUNCH_SEPARATE) {
-        return fail(CAM_ERR_RANGE, "camSetDispatchLaunchMode: mode must be 0 (auto), 1 (single) or 2 (separate)");
-    }
-    g_dispatch_launch_mode.store(mode, std::memory_order_relaxed);
-    return CAM_OK;
-}
 
 const char *camGetVersion(void) { return "cam-mi355x 0.1 (gfx950)"; }
 
@@ -869,46 +846,39 @@ camStatus camMoeDispatchPrefillGetWorkspaceSize(const camTensor *x, const camTen
             return fail(CAM_ERR_SHAPE, "totalRecvTokens must hold one element");
         }
     }
-    cam::FusedDispatchArgs f{};
-    f.p.idx = topkIdx->data;
-    f.p.idx_is64 = topkIdx->dtype == CAM_DT_INT64;
-    f.p.T = (int)T;
-    f.p.K = (int)K;
-    f.p.E = (int)numExperts;
-    f.p.R = 1;
-    f.p.pos = (int32_t *)sendTokenIdx->data;
-    f.p.dst_row = slotRowOptional ? (int32_t *)slotRowOptional->data : nullptr;
-    f.p.cnt = numTokensPerExpertOptional ? (int32_t *)numTokensPerExpertOptional->data : nullptr;
-    f.p.off = sendOffsetOptional ? (int32_t *)sendOffsetOptional->data : nullptr;
-    f.p.recv_count = recvCountOptional ? (int32_t *)recvCountOptional->data : nullptr;
-    f.p.tokens_per_expert =
+    cam::PlanArgs p{};
+    p.idx = topkIdx->data;
+    p.idx_is64 = topkIdx->dtype == CAM_DT_INT64;
+    p.T = (int)T;
+    p.K = (int)K;
+    p.E = (int)numExperts;
+    p.R = 1;
+    p.pos = (int32_t *)sendTokenIdx->data;
+    p.dst_row = slotRowOptional ? (int32_t *)slotRowOptional->data : nullptr;
+    p.cnt = numTokensPerExpertOptional ? (int32_t *)numTokensPerExpertOptional->data : nullptr;
+    p.off = sendOffsetOptional ? (int32_t *)sendOffsetOptional->data : nullptr;
+    p.recv_count = recvCountOptional ? (int32_t *)recvCountOptional->data : nullptr;
+    p.tokens_per_expert =
         numRecvTokensPerExpertOptional ? (int64_t *)numRecvTokensPerExpertOptional->data : nullptr;
-    f.p.total = totalRecvTokensOptional ? (int64_t *)totalRecvTokensOptional->data : nullptr;
-    f.x = (const uint16_t *)x->data;
-    f.x_is_fp16 = x->dtype == CAM_DT_FLOAT16;
-    f.H = (int)H;
-    f.A = A;
-    f.quant = quantMode == 0 ? 0 : (quantMode == 2 ? 1 : (quantMode == 4 ? 3 : 2));
-    f.out = recvX->data;
-    f.scales = quant ? (float *)recvXScalesOptional->data : nullptr;
-    f.src_info = (int32_t *)expandIdx->data;
-    f.src_rank = (int)rankId;
+    p.total = totalRecvTokensOptional ? (int64_t *)totalRecvTokensOptional->data : nullptr;
+    cam::DispatchArgs d{};
+    d.x = (const uint16_t *)x->data;
+    d.x_is_fp16 = x->dtype == CAM_DT_FLOAT16;
+    d.T = (int)T;
+    d.K = (int)K;
+    d.H = (int)H;
+    d.E = (int)numExperts;
+    d.A = A;
+    d.quant = quantMode == 0 ? 0 : (quantMode == 2 ? 1 : (quantMode == 4 ? 3 : 2));
+    d.out = recvX->data;
+    d.scales = quant ? (float *)recvXScalesOptional->data : nullptr;
+    d.src_info = (int32_t *)expandIdx->data;
+    d.src_rank = (int)rankId;
+    // The plan's launches, then the permute's.
     Carver c;
-    if (single_launch_dispatch(T, K)) {
-        const uint64_t o_ctrl = c.take(cam::fused_dispatch_ctrl_bytes());
-        const uint64_t o_table = c.take(cam::fused_dispatch_table_bytes(T, K, (int)numExperts));
-        auto run = [f, o_ctrl, o_table](void *ws, hipStream_t s) mutable -> hipError_t {
-            f.ctrl = (unsigned long long *)((char *)ws + o_ctrl);
-            f.p.hist_ws = (int32_t *)((char *)ws + o_table);
-            return cam::launch_dispatch_fused(f, s);
-        };
-        return finish_phase1(kOpPrefill, c.off, run, workspaceSize, executor);
-    }
-    // The plan and the permute as separate launches.
     const uint64_t o_hist = c.take(cam::plan_workspace_bytes(T, K, (int)numExperts));
     const uint64_t o_row = c.take((uint64_t)T * K * 4);
-    auto run = [f, o_hist, o_row](void *ws, hipStream_t s) mutable -> hipError_t {
-        cam::PlanArgs p = f.p;
+    auto run = [p, d, o_hist, o_row](void *ws, hipStream_t s) mutable -> hipError_t {
         p.hist_ws = (int32_t *)((char *)ws + o_hist);
         if (p.dst_row == nullptr) {
             p.dst_row = (int32_t *)((char *)ws + o_row);
@@ -917,20 +887,7 @@ camStatus camMoeDispatchPrefillGetWorkspaceSize(const camTensor *x, const camTen
         if (e != hipSuccess) {
             return e;
         }
-        cam::DispatchArgs d{};
-        d.x = f.x;
-        d.x_is_fp16 = f.x_is_fp16;
         d.dst_row = p.dst_row;
-        d.T = p.T;
-        d.K = p.K;
-        d.H = f.H;
-        d.E = p.E;
-        d.A = f.A;
-        d.quant = f.quant;
-        d.out = f.out;
-        d.scales = f.scales;
-        d.src_info = f.src_info;
-        d.src_rank = f.src_rank;
         return cam::launch_dispatch(d, s);
     };
     return finish_phase1(kOpPrefill, c.off, run, workspaceSize, executor);
@@ -1067,8 +1024,9 @@ camStatus camMoeCombineIndex(void *workspace, uint64_t workspaceSize, camOpExecu
 
 camStatus camMoeCombineGatherGetWorkspaceSize(const camTensor *recvX, const camTensor *tokenSrcInfoOptional,
                                               const camTensor *slotRow, const camTensor *epRecvCountsOptional,
-                                              const camTensor *recvTopkWeights, const camTensor *out,
-                                              uint64_t *workspaceSize, camOpExecutor **executor)
+                                              const camTensor *recvTopkWeights, const camTensor *sharedXOptional,
+                                              const camTensor *out, uint64_t *workspaceSize,
+                                              camOpExecutor **executor)
 {
     // recvX: bf16 rows [A,H], or rows quantised for the wire, int8 [A, H + H/4] (the int8 communication
     // quantisation of AK/moe_combine_shmem/op_kernel/moe_combine_shmem.h:564-592, dequantised as :755-773).
@@ -1114,7 +1072,17 @@ camStatus camMoeCombineGatherGetWorkspaceSize(const camTensor *recvX, const camT
     }
     CAM_TRY(check_aligned(recvX, "recvX", 16));
     CAM_TRY(check_aligned(out, "out", 16));
+    if (sharedXOptional != nullptr) {
+        // the shared expert's output rows, one per token, in the output's type; added un-weighted after the routed
+        // rows (FDM/raw_distributed/cam_moe_distribute_combine.h:757-774)
+        CAM_TRY(check_tensor(sharedXOptional, "sharedX", 2, out->dtype));
+        if (sharedXOptional->sizes[0] != T || sharedXOptional->sizes[1] != H) {
+            return fail(CAM_ERR_SHAPE, "sharedX must be [T,H] like out");
+        }
+        CAM_TRY(check_aligned(sharedXOptional, "sharedX", 16));
+    }
     cam::CombineArgs g{};
+    g.shared = sharedXOptional ? (const uint16_t *)sharedXOptional->data : nullptr;
     g.y = (const uint16_t *)recvX->data;
     g.slot_row = (const int32_t *)slotRow->data;
     g.src_info = tokenSrcInfoOptional ? (const int32_t *)tokenSrcInfoOptional->data : nullptr;
@@ -1136,6 +1104,289 @@ camStatus camMoeCombineGatherGetWorkspaceSize(const camTensor *recvX, const camT
 camStatus camMoeCombineGather(void *workspace, uint64_t workspaceSize, camOpExecutor *executor, camStream_t stream)
 {
     return run_phase2(kOpCombGather, "camMoeCombineGather", workspace, workspaceSize, executor, stream);
+}
+
+// ------------------------------------------------------------------------------------------------
+// The SHMEM operator pair on one rank.  Validation follows AK/moe_dispatch_shmem/op_host/
+// moe_dispatch_shmem_tiling.cpp:123-215,365-535 and AK/moe_combine_shmem/op_host/moe_combine_shmem_tiling.cpp:
+// 120-200; the limits tied to the transport (epWorldSize in {8,...,288}, H == 7168) are lifted, epWorldSize > 1 is
+// refused.
+camStatus camMoeDispatchShmemGetWorkspaceSize(const camTensor *x, const camTensor *expertIds,
+                                              const camTensor *scalesOptional,
+                                              const camTensor *xActiveMaskOptional, int64_t epWorldSize,
+                                              int64_t epRankId, int64_t moeExpertNum, int64_t tpWorldSize,
+                                              int64_t tpRankId, int64_t expertShardType, int64_t sharedExpertNum,
+                                              int64_t sharedExpertRankNum, int64_t quantMode, int64_t globalBs,
+                                              int64_t expertTokenNumsType, int64_t extInfo,
+                                              const camTensor *expandXOut, const camTensor *dynamicScalesOut,
+                                              const camTensor *expandIdxOut, const camTensor *expertTokenNumsOut,
+                                              const camTensor *epRecvCountOut, const camTensor *tpRecvCountOut,
+                                              uint64_t *workspaceSize, camOpExecutor **executor)
+{
+    (void)tpRankId;
+    (void)sharedExpertNum;
+    (void)extInfo;         // the reference's handle of its symmetric heap
+    (void)tpRecvCountOut;  // written only when tpWorldSize == 2 (moe_dispatch_shmem.h:1078-1086)
+    CAM_TRY(check_tensor(x, "x", 2, CAM_DT_BF16, CAM_DT_FLOAT16));
+    CAM_TRY(check_tensor(expertIds, "expertIds", 2, CAM_DT_INT32));
+    if (epWorldSize <= 0 || epWorldSize > cam::kMaxRanks) {
+        return fail(CAM_ERR_RANGE, "epWorldSize %lld outside (0, %d]", (long long)epWorldSize, cam::kMaxRanks);
+    }
+    if (epRankId < 0 || epRankId >= epWorldSize) {
+        return fail(CAM_ERR_RANGE, "epRankId %lld outside [0, epWorldSize)", (long long)epRankId);
+    }
+    if (moeExpertNum <= 0 || moeExpertNum > cam::kMaxExperts) {
+        return fail(CAM_ERR_RANGE, "moeExpertNum %lld outside (0, %d]", (long long)moeExpertNum, cam::kMaxExperts);
+    }
+    if (tpWorldSize < 0 || tpWorldSize > 2) {
+        return fail(CAM_ERR_RANGE, "tpWorldSize %lld outside [0, 2]", (long long)tpWorldSize);
+    }
+    if (expertShardType != 0) {
+        return fail(CAM_ERR_RANGE, "expertShardType must be 0");
+    }
+    if (sharedExpertRankNum < 0 || sharedExpertRankNum >= epWorldSize) {
+        return fail(CAM_ERR_RANGE, "sharedExpertRankNum %lld outside [0, epWorldSize)", (long long)sharedExpertRankNum);
+    }
+    if (quantMode < 0 || quantMode > 2) {
+        return fail(CAM_ERR_RANGE, "quantMode %lld outside [0, 2]", (long long)quantMode);
+    }
+    if (expertTokenNumsType != 0 && expertTokenNumsType != 1) {
+        return fail(CAM_ERR_RANGE, "expertTokenNumsType must be 0 (running totals) or 1 (counts)");
+    }
+    if (quantMode == 1) {
+        return fail(CAM_ERR_UNSUPPORTED, "quantMode 1 (static quantisation) is not built");
+    }
+    if (epWorldSize != 1 || sharedExpertRankNum != 0 || tpWorldSize > 1) {
+        return fail(CAM_ERR_UNSUPPORTED, "MoeDispatchShmem: epWorldSize must be 1, sharedExpertRankNum 0 and "
+                                         "tpWorldSize at most 1 (single-GPU library)");
+    }
+    if (xActiveMaskOptional != nullptr) {
+        return fail(CAM_ERR_UNSUPPORTED, "MoeDispatchShmem: xActiveMask is reserved in the reference; pass NULL");
+    }
+    const int64_t T = x->sizes[0], H = x->sizes[1], K = expertIds->sizes[1];
+    if (T < 1) {
+        return fail(CAM_ERR_RANGE, "batch size must be at least 1");
+    }
+    if (H < 1024 || H > 7168 || H % 8 != 0) {
+        return fail(CAM_ERR_RANGE, "hidden size %lld must be a multiple of 8 in [1024, 7168]", (long long)H);
+    }
+    if (expertIds->sizes[0] != T) {
+        return fail(CAM_ERR_SHAPE, "x and expertIds must agree on dimension 0");
+    }
+    if (K <= 0 || K > cam::kMaxTopk || K > moeExpertNum) {
+        return fail(CAM_ERR_RANGE, "top-k %lld outside (0, min(%d, moeExpertNum)]", (long long)K, cam::kMaxTopk);
+    }
+    if (globalBs != 0 && (globalBs < T * epWorldSize || globalBs % epWorldSize != 0)) {
+        return fail(CAM_ERR_RANGE, "globalBs must be 0 or a multiple of epWorldSize that is >= epWorldSize * bs");
+    }
+    if (T * K > 0x7fffffffll) {
+        return fail(CAM_ERR_RANGE, "tokens * top-k does not fit 32 bits");
+    }
+    const bool quant = quantMode == 2;
+    if (scalesOptional != nullptr) {
+        CAM_TRY(check_tensor(scalesOptional, "scales", 2, CAM_DT_FLOAT));
+        if (scalesOptional->sizes[0] != moeExpertNum || scalesOptional->sizes[1] != H) {
+            return fail(CAM_ERR_SHAPE, "scales must be fp32 [moeExpertNum, H]");
+        }
+        CAM_TRY(check_aligned(scalesOptional, "scales", 16));
+    }
+    CAM_TRY(check_tensor(expandXOut, "expandXOut", 2, quant ? CAM_DT_INT8 : x->dtype));
+    if (expandXOut->sizes[1] != H) {
+        return fail(CAM_ERR_SHAPE, "expandXOut dimension 1 must equal the hidden size");
+    }
+    const int64_t A = expandXOut->sizes[0];
+    CAM_TRY(check_aligned(x, "x", 16));
+    CAM_TRY(check_aligned(expandXOut, "expandXOut", 16));
+    CAM_TRY(check_tensor(dynamicScalesOut, "dynamicScalesOut", 1, CAM_DT_FLOAT));
+    if (quant && dynamicScalesOut->sizes[0] < A) {
+        return fail(CAM_ERR_SHAPE, "dynamicScalesOut must hold one value per expandXOut row");
+    }
+    CAM_TRY(check_tensor(expandIdxOut, "expandIdxOut", 1, CAM_DT_INT32));
+    if (expandIdxOut->sizes[0] != T * K) {
+        return fail(CAM_ERR_SHAPE, "expandIdxOut must hold bs * K elements");
+    }
+    CAM_TRY(check_tensor(expertTokenNumsOut, "expertTokenNumsOut", 1, CAM_DT_INT64));
+    CAM_TRY(check_tensor(epRecvCountOut, "epRecvCountOut", 1, CAM_DT_INT32));
+    if (expertTokenNumsOut->sizes[0] != moeExpertNum || epRecvCountOut->sizes[0] != moeExpertNum) {
+        return fail(CAM_ERR_SHAPE, "expertTokenNumsOut and epRecvCountOut must hold one value per local expert");
+    }
+    cam::PlanArgs p{};
+    p.idx = expertIds->data;
+    p.idx_is64 = 0;
+    p.T = (int)T;
+    p.K = (int)K;
+    p.E = (int)moeExpertNum;
+    p.R = 1;
+    p.pos = (int32_t *)expandIdxOut->data;
+    p.recv_count = (int32_t *)epRecvCountOut->data;
+    if (expertTokenNumsType == 0) {
+        p.group_list = (int64_t *)expertTokenNumsOut->data;
+    } else {
+        p.tokens_per_expert = (int64_t *)expertTokenNumsOut->data;
+    }
+    cam::DispatchArgs d{};
+    d.x = (const uint16_t *)x->data;
+    d.x_is_fp16 = x->dtype == CAM_DT_FLOAT16;
+    d.idx = (const int32_t *)expertIds->data;
+    d.T = (int)T;
+    d.K = (int)K;
+    d.H = (int)H;
+    d.E = (int)moeExpertNum;
+    d.A = A;
+    d.quant = quant ? 2 : 0;  // the variant without the epsilon (moe_dispatch_shmem.h:720)
+    d.out = expandXOut->data;
+    d.scales = quant ? (float *)dynamicScalesOut->data : nullptr;
+    d.src_rank = (int)epRankId;
+    d.smooth = quant && scalesOptional ? (const float *)scalesOptional->data : nullptr;
+    Carver c;
+    const uint64_t o_hist = c.take(cam::plan_workspace_bytes(T, K, (int)moeExpertNum));
+    const uint64_t o_row = c.take((uint64_t)T * K * 4);
+    auto run = [p, d, o_hist, o_row](void *ws, hipStream_t s) mutable -> hipError_t {
+        p.hist_ws = (int32_t *)((char *)ws + o_hist);
+        p.dst_row = (int32_t *)((char *)ws + o_row);
+        hipError_t e = cam::launch_plan(p, s);
+        if (e != hipSuccess) {
+            return e;
+        }
+        d.dst_row = p.dst_row;
+        return cam::launch_dispatch(d, s);
+    };
+    return finish_phase1(kOpDispShmem, c.off, run, workspaceSize, executor);
+}
+
+camStatus camMoeDispatchShmem(void *workspace, uint64_t workspaceSize, camOpExecutor *executor, camStream_t stream)
+{
+    return run_phase2(kOpDispShmem, "camMoeDispatchShmem", workspace, workspaceSize, executor, stream);
+}
+
+camStatus camMoeCombineShmemGetWorkspaceSize(
+    const camTensor *expandX, const camTensor *expertIds, const camTensor *expandIdx, const camTensor *epSendCounts,
+    const camTensor *expertScales, const camTensor *tpSendCountsOptional, const camTensor *xActiveMaskOptional,
+    const camTensor *activationScaleOptional, const camTensor *weightScaleOptional,
+    const camTensor *groupListOptional, const camTensor *expandScalesOptional, int64_t epWorldSize,
+    int64_t epRankId, int64_t moeExpertNum, int64_t tpWorldSize, int64_t tpRankId, int64_t expertShardType,
+    int64_t sharedExpertNum, int64_t sharedExpertRankNum, int64_t globalBs, int64_t commQuantMode, int64_t extInfo,
+    int64_t outDtype, int64_t groupListType, const camTensor *out, uint64_t *workspaceSize,
+    camOpExecutor **executor)
+{
+    (void)tpSendCountsOptional;
+    (void)tpRankId;
+    (void)sharedExpertNum;
+    (void)extInfo;
+    (void)outDtype;
+    (void)groupListType;
+    if (xActiveMaskOptional != nullptr || activationScaleOptional != nullptr || weightScaleOptional != nullptr ||
+        groupListOptional != nullptr || expandScalesOptional != nullptr) {
+        return fail(CAM_ERR_UNSUPPORTED, "MoeCombineShmem: xActiveMask, activationScale, weightScale, groupList and "
+                                         "expandScales are reserved in the reference; pass NULL");
+    }
+    CAM_TRY(check_tensor(expandX, "expandX", 2, CAM_DT_BF16, CAM_DT_FLOAT16));
+    CAM_TRY(check_tensor(expertIds, "expertIds", 2, CAM_DT_INT32));
+    CAM_TRY(check_tensor(expandIdx, "expandIdx", 1, CAM_DT_INT32));
+    CAM_TRY(check_tensor(epSendCounts, "epSendCounts", 1, CAM_DT_INT32));
+    CAM_TRY(check_tensor(expertScales, "expertScales", 2, CAM_DT_FLOAT));
+    CAM_TRY(check_tensor(out, "out", 2, expandX->dtype));
+    if (epWorldSize <= 0 || epWorldSize > cam::kMaxRanks) {
+        return fail(CAM_ERR_RANGE, "epWorldSize %lld outside (0, %d]", (long long)epWorldSize, cam::kMaxRanks);
+    }
+    if (epRankId < 0 || epRankId >= epWorldSize) {
+        return fail(CAM_ERR_RANGE, "epRankId %lld outside [0, epWorldSize)", (long long)epRankId);
+    }
+    if (moeExpertNum <= 0 || moeExpertNum > cam::kMaxExperts) {
+        return fail(CAM_ERR_RANGE, "moeExpertNum %lld outside (0, %d]", (long long)moeExpertNum, cam::kMaxExperts);
+    }
+    if (tpWorldSize < 0 || tpWorldSize > 2) {
+        return fail(CAM_ERR_RANGE, "tpWorldSize %lld outside [0, 2]", (long long)tpWorldSize);
+    }
+    if (expertShardType != 0) {  // moe_combine_shmem_tiling.cpp:174
+        return fail(CAM_ERR_RANGE, "expertShardType must be 0");
+    }
+    if (sharedExpertRankNum < 0 || sharedExpertRankNum >= epWorldSize) {
+        return fail(CAM_ERR_RANGE, "sharedExpertRankNum %lld outside [0, epWorldSize)", (long long)sharedExpertRankNum);
+    }
+    if (commQuantMode != 0 && commQuantMode != 2) {  // moe_combine_shmem_tiling.cpp:190-191
+        return fail(CAM_ERR_RANGE, "commQuantMode must be 0 or 2, is %lld", (long long)commQuantMode);
+    }
+    if (epWorldSize != 1 || sharedExpertRankNum != 0 || tpWorldSize > 1) {
+        return fail(CAM_ERR_UNSUPPORTED, "MoeCombineShmem: epWorldSize must be 1, sharedExpertRankNum 0 and "
+                                         "tpWorldSize at most 1 (single-GPU library)");
+    }
+    const int64_t A = expandX->sizes[0], H = expandX->sizes[1];
+    const int64_t T = expertIds->sizes[0], K = expertIds->sizes[1];
+    if (T < 1) {
+        return fail(CAM_ERR_RANGE, "batch size must be at least 1");
+    }
+    if (H < 1024 || H > 7168 || H % 8 != 0) {
+        return fail(CAM_ERR_RANGE, "hidden size %lld must be a multiple of 8 in [1024, 7168]", (long long)H);
+    }
+    if (K <= 0 || K > cam::kMaxTopk) {
+        return fail(CAM_ERR_RANGE, "top-k %lld outside (0, %d]", (long long)K, cam::kMaxTopk);
+    }
+    if (expandIdx->sizes[0] != T * K) {
+        return fail(CAM_ERR_SHAPE, "expandIdx must hold bs * K elements");
+    }
+    if (expertScales->sizes[0] != T || expertScales->sizes[1] != K) {
+        return fail(CAM_ERR_SHAPE, "expertScales must be [bs, K]");
+    }
+    if (epSendCounts->sizes[0] != moeExpertNum) {
+        return fail(CAM_ERR_SHAPE, "epSendCounts must hold one value per local expert");
+    }
+    if (out->sizes[0] != T || out->sizes[1] != H) {
+        return fail(CAM_ERR_SHAPE, "out must be [bs, H]");
+    }
+    if (globalBs != 0 && (globalBs < T * epWorldSize || globalBs % epWorldSize != 0)) {
+        return fail(CAM_ERR_RANGE, "globalBs must be 0 or a multiple of epWorldSize that is >= epWorldSize * bs");
+    }
+    if (T * K > 0x7fffffffll || A > 0x7fffffffll) {
+        return fail(CAM_ERR_RANGE, "row counts do not fit 32 bits");
+    }
+    const bool wire = commQuantMode == 2;
+    if (wire && expandX->dtype != CAM_DT_BF16) {
+        return fail(CAM_ERR_UNSUPPORTED, "MoeCombineShmem: commQuantMode 2 is built for bf16 rows only");
+    }
+    CAM_TRY(check_aligned(expandX, "expandX", 16));
+    CAM_TRY(check_aligned(out, "out", 16));
+    Carver c;
+    const uint64_t o_slot = c.take((uint64_t)T * K * 4);
+    const uint64_t o_wire = wire ? c.take((uint64_t)A * (uint64_t)(H + H / 4)) : 0;
+    cam::CombineArgs g{};
+    g.y = (const uint16_t *)expandX->data;
+    g.w = (const float *)expertScales->data;
+    g.T = (int)T;
+    g.K = (int)K;
+    g.H = (int)H;
+    g.A = A;
+    g.act_fp16 = expandX->dtype == CAM_DT_FLOAT16;
+    g.out = (uint16_t *)out->data;
+    const int32_t *ids = (const int32_t *)expertIds->data;
+    const int32_t *eidx = (const int32_t *)expandIdx->data;
+    const int32_t *counts = (const int32_t *)epSendCounts->data;
+    const int iE = (int)moeExpertNum;
+    auto run = [=](void *ws, hipStream_t s) mutable -> hipError_t {
+        int32_t *slot = (int32_t *)((char *)ws + o_slot);
+        hipError_t e = cam::launch_rows_from_counts(ids, eidx, counts, (int64_t)g.T * g.K, iE, g.A, slot, s);
+        if (e != hipSuccess) {
+            return e;
+        }
+        g.slot_row = slot;
+        if (wire) {  // every row takes the int8 wire format on its way (moe_combine_shmem.h:567-592,755-773)
+            uint8_t *rows = (uint8_t *)ws + o_wire;
+            e = cam::launch_comm_quant(g.y, g.A, g.H, counts + (iE - 1), rows, s);
+            if (e != hipSuccess) {
+                return e;
+            }
+            g.y = (const uint16_t *)rows;
+            g.wire_rows = 1;
+            g.row_limit = counts + (iE - 1);
+        }
+        return cam::launch_combine(g, s);
+    };
+    return finish_phase1(kOpCombShmem, c.off, run, workspaceSize, executor);
+}
+
+camStatus camMoeCombineShmem(void *workspace, uint64_t workspaceSize, camOpExecutor *executor, camStream_t stream)
+{
+    return run_phase2(kOpCombShmem, "camMoeCombineShmem", workspace, workspaceSize, executor, stream);
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -1436,8 +1687,8 @@ camStatus camFusedDeepMoeGetWorkspaceSize(const camTensor *x, const camTensor *e
     if (moeExpertNum <= 0 || moeExpertNum > cam::kMaxExperts) {
         return fail(CAM_ERR_RANGE, "moeExpertNum %lld outside (0, %d]", (long long)moeExpertNum, cam::kMaxExperts);
     }
-    if (sharedExpertNum != 1 && sharedExpertNum != 0) {
-        return fail(CAM_ERR_RANGE, "sharedExpertNum must be 1 (0 is tolerated), is %lld", (long long)sharedExpertNum);
+    if (sharedExpertNum != 1) {  // AK/fused_deep_moe/op_host/fused_deep_moe_tiling.cpp:345
+        return fail(CAM_ERR_RANGE, "sharedExpertNum must be 1, is %lld", (long long)sharedExpertNum);
     }
     if (sharedExpertRankNum < 0 || sharedExpertRankNum >= epRankSize) {
         return fail(CAM_ERR_RANGE, "sharedExpertRankNum %lld outside [0, epRankSize)", (long long)sharedExpertRankNum);
@@ -1520,10 +1771,7 @@ camStatus camFusedDeepMoeGetWorkspaceSize(const camTensor *x, const camTensor *e
     const uint64_t o_meta = c.take(cam::kPlanMeta * 4);
     const uint64_t o_sched1 = c.take(cam::sched_bytes(A, (int)Epr, (int)(2 * I)));
     const uint64_t o_sched2 = c.take(cam::sched_bytes(A, (int)Epr, (int)H));
-    const bool fused_dispatch = single_launch_dispatch(T, K);
-    const uint64_t o_hist = c.take(fused_dispatch ? cam::fused_dispatch_table_bytes(T, K, (int)Epr)
-                                                  : cam::plan_workspace_bytes(T, K, (int)Epr));
-    const uint64_t o_ctrl = c.take(cam::fused_dispatch_ctrl_bytes());
+    const uint64_t o_hist = c.take(cam::plan_workspace_bytes(T, K, (int)Epr));
     // The bf16 rows GMM2 writes (2*A*H bytes) live where the quantised rows (A*H) and the fp32 SwiGLU products
     // (4*A*I) lived: both are dead once the re-quantisation has run (the reference overlays its stages the same
     // way, AK/fused_deep_moe/op_kernel/fused_deep_moe.h:362-391).  GMM2's own input stays apart.
@@ -1574,50 +1822,31 @@ camStatus camFusedDeepMoeGetWorkspaceSize(const camTensor *x, const camTensor *e
         cam::SchedSpec specs[2] = {sp1, sp2};  // both GEMM schedules come from the per-expert counts of the plan
         specs[0].sched = (int32_t *)(w + o_sched1);
         specs[1].sched = (int32_t *)(w + o_sched2);
-        if (fused_dispatch) {
-            cam::FusedDispatchArgs f{};
-            f.p = p;
-            f.x = xp;
-            f.x_is_fp16 = x_is_fp16;
-            f.H = iH;
-            f.A = A;
-            f.quant = 2;
-            f.out = x1;
-            f.scales = x1s;
-            f.ctrl = (unsigned long long *)(w + o_ctrl);
-            e = cam::launch_dispatch_fused(f, s);
-            if (e != hipSuccess) return e;
-        } else {
-            e = cam::launch_plan(p, s);
-            if (e != hipSuccess) return e;
-            cam::DispatchArgs d{};
-            d.x = xp;
-            d.x_is_fp16 = x_is_fp16;
-            d.idx = ids;
-            d.dst_row = row;
-            d.T = iT;
-            d.K = iK;
-            d.H = iH;
-            d.E = iE;
-            d.A = A;
-            d.quant = 2;
-            d.out = x1;
-            d.scales = x1s;
-            // the plan has written the per-expert counts: spare workgroups of the permute build both schedules
-            d.sched.group_list = etn;
-            d.sched.cumulative = 0;
-            d.sched.G = iE;
-            d.sched.nspec = 2;
-            d.sched.max_rows = A;
-            d.sched.spec[0] = specs[0];
-            d.sched.spec[1] = specs[1];
-            e = cam::launch_dispatch(d, s);
-            if (e != hipSuccess) return e;
-        }
-        if (fused_dispatch) {  // the counts exist only once the single launch is over
-            e = cam::launch_build_sched(etn, 0, iE, A, 2, specs, s);
-            if (e != hipSuccess) return e;
-        }
+        e = cam::launch_plan(p, s);
+        if (e != hipSuccess) return e;
+        cam::DispatchArgs d{};
+        d.x = xp;
+        d.x_is_fp16 = x_is_fp16;
+        d.idx = ids;
+        d.dst_row = row;
+        d.T = iT;
+        d.K = iK;
+        d.H = iH;
+        d.E = iE;
+        d.A = A;
+        d.quant = 2;
+        d.out = x1;
+        d.scales = x1s;
+        // the plan has written the per-expert counts: spare workgroups of the permute build both schedules
+        d.sched.group_list = etn;
+        d.sched.cumulative = 0;
+        d.sched.G = iE;
+        d.sched.nspec = 2;
+        d.sched.max_rows = A;
+        d.sched.spec[0] = specs[0];
+        d.sched.spec[1] = specs[1];
+        e = cam::launch_dispatch(d, s);
+        if (e != hipSuccess) return e;
 
         cam::GemmArgs g1{};
         g1.a = x1;
@@ -1903,10 +2132,7 @@ camStatus camFusedDeepMoeFp8GetWorkspaceSize(const camTensor *x, const camTensor
     const uint64_t o_meta = c.take(cam::kPlanMeta * 4);
     const uint64_t o_sched1 = c.take(cam::sched_bytes(A, (int)E, (int)(2 * I)));
     const uint64_t o_sched2 = c.take(cam::sched_bytes(A, (int)E, (int)H));
-    const bool fused_dispatch = single_launch_dispatch(T, K);
-    const uint64_t o_hist = c.take(fused_dispatch ? cam::fused_dispatch_table_bytes(T, K, (int)E)
-                                                  : cam::plan_workspace_bytes(T, K, (int)E));
-    const uint64_t o_ctrl = c.take(cam::fused_dispatch_ctrl_bytes());
+    const uint64_t o_hist = c.take(cam::plan_workspace_bytes(T, K, (int)E));
     // as in the int8 layer, the bf16 rows of GMM2 overlay the quantised input rows and the fp32 products
     const uint64_t x1_bytes = align_up((uint64_t)A * H);
     const uint64_t shared_bytes = std::max<uint64_t>((uint64_t)A * H * 2, x1_bytes + (uint64_t)A * I * 4);
@@ -1955,49 +2181,30 @@ camStatus camFusedDeepMoeFp8GetWorkspaceSize(const camTensor *x, const camTensor
         cam::SchedSpec specs[2] = {sp1, sp2};
         specs[0].sched = (int32_t *)(w + o_sched1);
         specs[1].sched = (int32_t *)(w + o_sched2);
-        if (fused_dispatch) {
-            cam::FusedDispatchArgs f{};
-            f.p = p;
-            f.x = xp;
-            f.x_is_fp16 = x_is_fp16;
-            f.H = iH;
-            f.A = A;
-            f.quant = 3;
-            f.out = x1;
-            f.scales = (float *)x1s;
-            f.ctrl = (unsigned long long *)(w + o_ctrl);
-            e = cam::launch_dispatch_fused(f, s);
-            if (e != hipSuccess) return e;
-        } else {
-            e = cam::launch_plan(p, s);
-            if (e != hipSuccess) return e;
-            cam::DispatchArgs d{};
-            d.x = xp;
-            d.x_is_fp16 = x_is_fp16;
-            d.idx = ids;
-            d.dst_row = row;
-            d.T = iT;
-            d.K = iK;
-            d.H = iH;
-            d.E = iE;
-            d.A = A;
-            d.quant = 3;
-            d.out = x1;
-            d.scales = (float *)x1s;
-            d.sched.group_list = etn;  // spare workgroups of the permute build both schedules
-            d.sched.cumulative = 0;
-            d.sched.G = iE;
-            d.sched.nspec = 2;
-            d.sched.max_rows = A;
-            d.sched.spec[0] = specs[0];
-            d.sched.spec[1] = specs[1];
-            e = cam::launch_dispatch(d, s);
-            if (e != hipSuccess) return e;
-        }
-        if (fused_dispatch) {  // the counts exist only once the single launch is over
-            e = cam::launch_build_sched(etn, 0, iE, A, 2, specs, s);
-            if (e != hipSuccess) return e;
-        }
+        e = cam::launch_plan(p, s);
+        if (e != hipSuccess) return e;
+        cam::DispatchArgs d{};
+        d.x = xp;
+        d.x_is_fp16 = x_is_fp16;
+        d.idx = ids;
+        d.dst_row = row;
+        d.T = iT;
+        d.K = iK;
+        d.H = iH;
+        d.E = iE;
+        d.A = A;
+        d.quant = 3;
+        d.out = x1;
+        d.scales = (float *)x1s;
+        d.sched.group_list = etn;  // spare workgroups of the permute build both schedules
+        d.sched.cumulative = 0;
+        d.sched.G = iE;
+        d.sched.nspec = 2;
+        d.sched.max_rows = A;
+        d.sched.spec[0] = specs[0];
+        d.sched.spec[1] = specs[1];
+        e = cam::launch_dispatch(d, s);
+        if (e != hipSuccess) return e;
 
         cam::GemmArgs g1{};
         g1.a = (const int8_t *)x1;

@@ -109,6 +109,9 @@ struct DispatchArgs {
     float *scales;       // [A]   (quant only)
     int32_t *src_info;   // [3A]  optional
     int src_rank;
+    // quant == 2 only: optional per-expert smooth scales fp32 [E,H].  Copy (t,k) is then quantised on its own,
+    // from float(x[t]) * smooth[idx[t,k]] (moe_dispatch_shmem.h:693-733); idx must be set.
+    const float *smooth;
     // GEMM schedules to build in the same launch (sched.nspec > 0): sched.nspec * sched_parts extra workgroups
     // do what launch_build_sched would, beside the ones that move rows.  The group list must be complete before
     // the launch (it is when it comes from launch_plan on the same stream).  sched_parts is set by the launcher.
@@ -116,30 +119,6 @@ struct DispatchArgs {
     int sched_parts;
 };
 hipError_t launch_dispatch(const DispatchArgs &a, hipStream_t stream);
-
-// Plan + permute in one launch (dispatch_fused.hip).  `p` is the plan (pos required; hist_ws must hold
-// fused_dispatch_table_bytes()); ctrl points at fused_dispatch_ctrl_bytes() of workspace, 8-byte aligned, whose
-// content is arbitrary on the first use and is left cleared by every launch.
-constexpr int kFusedMaxChunks = 256;                 // chunks of 2048 flat ids: T*K <= 524288
-constexpr int kFusedCtrlWords = kFusedMaxChunks + 4;
-struct FusedDispatchArgs {
-    PlanArgs p;
-    const uint16_t *x;   // [T,H] bf16 or fp16 bits
-    int x_is_fp16;
-    int H;
-    int64_t A;           // rows in the outputs
-    int quant;           // as DispatchArgs
-    void *out;
-    float *scales;
-    int32_t *src_info;   // optional
-    int src_rank;
-    unsigned long long *ctrl;
-    int nb;              // set by the launcher
-};
-bool fused_dispatch_fits(int64_t T, int64_t K);
-uint64_t fused_dispatch_table_bytes(int64_t T, int64_t K, int E);
-uint64_t fused_dispatch_ctrl_bytes();
-hipError_t launch_dispatch_fused(FusedDispatchArgs a, hipStream_t stream);
 
 // ---------------------------------------------------------------------------------------------
 // Combine.
@@ -157,9 +136,14 @@ struct CombineArgs {
     int64_t A;
     const int32_t *row_limit; // optional device scalar: rows >= *row_limit are never read
     const int32_t *t_active;  // optional device scalar: tokens >= *t_active produce zero rows
+    const uint16_t *shared;   // optional [T,H] rows of the output's type, added un-weighted after the routed rows
     uint16_t *out;            // [T,H]
 };
 hipError_t launch_combine(const CombineArgs &a, hipStream_t stream);
+// slot_row[i] = (e ? ep_send_counts[e-1] : 0) + expand_idx[i] for e = ids[i] in [0,E) and a row below A, else -1
+// (how the SHMEM combine finds the row of slot i: moe_combine_shmem.h:514-556,833-837).
+hipError_t launch_rows_from_counts(const int32_t *ids, const int32_t *expand_idx, const int32_t *ep_send_counts,
+                                   int64_t n, int E, int64_t A, int32_t *slot_row, hipStream_t stream);
 // bf16 rows [A,H] -> wire rows [A, H + H/4] bytes: per block of 8 columns int8 values and one bf16 scale.
 // row_limit: optional device scalar; rows >= *row_limit are left untouched.
 hipError_t launch_comm_quant(const uint16_t *y, int64_t A, int H, const int32_t *row_limit, uint8_t *out,

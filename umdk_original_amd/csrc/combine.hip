@@ -48,6 +48,25 @@ __global__ void invert_src_info_kernel(const int32_t *src_info, long long A, con
     }
 }
 
+__global__ void rows_from_counts_kernel(const int32_t *__restrict__ ids, const int32_t *__restrict__ expand_idx,
+                                        const int32_t *__restrict__ ep_send_counts, long long n, int E, long long A,
+                                        int32_t *__restrict__ slot_row)
+{
+    const long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n) {
+        return;
+    }
+    const int e = ids[i];
+    long long row = -1;
+    if (e >= 0 && e < E) {
+        row = (long long)(e == 0 ? 0 : ep_send_counts[e - 1]) + expand_idx[i];
+        if (row < 0 || row >= A) {
+            row = -1;
+        }
+    }
+    slot_row[i] = (int32_t)row;
+}
+
 // bf16 rows -> wire rows.  One thread per block of 8 columns.
 __global__ __launch_bounds__(256) void comm_quant_kernel(const uint16_t *__restrict__ y, long long A, int H,
                                                          const int32_t *__restrict__ row_limit,
@@ -111,6 +130,11 @@ __global__ __launch_bounds__(kCombThreads) void combine_kernel(CombineArgs a, in
     }
     const bool live = a.t_active == nullptr || t < *a.t_active;
     const long long rows = a.row_limit == nullptr ? a.A : min(a.A, (long long)*a.row_limit);
+    const bool add_shared = live && a.shared != nullptr;
+    v4u sh = {0u, 0u, 0u, 0u};
+    if (add_shared) {  // requested with the routed rows, used after them
+        sh = __builtin_nontemporal_load((const v4u *)(a.shared + (long long)t * a.H + col));
+    }
     if (live) {
         for (int k0 = 0; k0 < a.K; k0 += kCombBatch) {
             v4u v[kCombBatch];  // WIRE: x, y = the 8 int8 values, z = the block's scale (bf16 bits)
@@ -164,6 +188,13 @@ __global__ __launch_bounds__(kCombThreads) void combine_kernel(CombineArgs a, in
                     }
                 }
             }
+        }
+    }
+    if (add_shared) {  // the shared expert's row: un-weighted, after the routed rows
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+            acc[2 * c] = __fadd_rn(acc[2 * c], comb_act_to_f32<ACT>(sh[c] & 0xffffu));
+            acc[2 * c + 1] = __fadd_rn(acc[2 * c + 1], comb_act_to_f32<ACT>(sh[c] >> 16));
         }
     }
     v4u o;
@@ -249,6 +280,15 @@ __global__ __launch_bounds__(kCombThreads) void combine_wire16_kernel(CombineArg
             }
         }
     }
+    if (live && a.shared != nullptr) {
+        const v4u *sp = (const v4u *)(a.shared + (long long)t * a.H + col);
+        const v4u s[2] = {__builtin_nontemporal_load(sp), __builtin_nontemporal_load(sp + 1)};
+#pragma unroll
+        for (int c = 0; c < 8; ++c) {
+            acc[2 * c] = __fadd_rn(acc[2 * c], bf16_bits_to_f32(s[c >> 2][c & 3] & 0xffffu));
+            acc[2 * c + 1] = __fadd_rn(acc[2 * c + 1], bf16_bits_to_f32(s[c >> 2][c & 3] >> 16));
+        }
+    }
     v4u o[2];
 #pragma unroll
     for (int c = 0; c < 8; ++c) {
@@ -269,6 +309,17 @@ hipError_t launch_invert_src_info(const int32_t *src_info, int64_t A, const int3
     }
     hipLaunchKernelGGL(invert_src_info_kernel, dim3((unsigned)((A + 255) / 256)), dim3(256), 0, stream, src_info,
                        (long long)A, row_limit, T, K, slot_row);
+    return hipGetLastError();
+}
+
+hipError_t launch_rows_from_counts(const int32_t *ids, const int32_t *expand_idx, const int32_t *ep_send_counts,
+                                   int64_t n, int E, int64_t A, int32_t *slot_row, hipStream_t stream)
+{
+    if (n <= 0) {
+        return hipSuccess;
+    }
+    hipLaunchKernelGGL(rows_from_counts_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, stream, ids,
+                       expand_idx, ep_send_counts, (long long)n, E, (long long)A, slot_row);
     return hipGetLastError();
 }
 

@@ -72,6 +72,30 @@ __global__ __launch_bounds__(kDispWaves * kWave, QUANT == 3 ? 3 : 4) void dispat
     }
 }
 
+// The quantising permute with per-expert smooth scales: every copy of a token is quantised on its own, under the
+// scale row of its destination expert (moe_dispatch_shmem.h:492-549,693-733).  One wave per token; the token row
+// is loaded once and stays in registers across its copies.
+template <int ACT>
+__global__ __launch_bounds__(kDispWaves * kWave) void dispatch_smooth_kernel(DispatchArgs a)
+{
+    const int t = (int)blockIdx.x * kDispWaves + (threadIdx.x >> 6);
+    const int lane = threadIdx.x & (kWave - 1);
+    if (t >= a.T) {
+        return;
+    }
+    TokenRow r;
+    load_token_row(a.x, t, a.H, lane, r);
+    for (int k = 0; k < a.K; ++k) {
+        const long long row = dispatch_row(a, t, k);
+        const int e = a.idx[(long long)t * a.K + k];
+        if (row < 0 || row >= a.A || e < 0 || e >= a.E) {
+            continue;
+        }
+        quant_token_row_smooth<ACT>(r, a.smooth + (long long)e * a.H, a.H, lane);
+        store_token_row<2>(r, a.out, a.scales, a.src_info, a.src_rank, row, t, k, a.H, lane);
+    }
+}
+
 }  // namespace
 
 hipError_t launch_dispatch(const DispatchArgs &a_in, hipStream_t stream)
@@ -99,6 +123,17 @@ hipError_t launch_dispatch(const DispatchArgs &a_in, hipStream_t stream)
         a.sched_parts = a.sched_parts > 8 ? 8 : a.sched_parts;
     }
     dim3 grid((a.T + kDispWaves - 1) / kDispWaves + a.sched.nspec * a.sched_parts), block(kDispWaves * kWave);
+    if (a.smooth != nullptr) {
+        if (a.quant != 2 || a.idx == nullptr || a.sched.nspec != 0) {
+            return hipErrorInvalidValue;
+        }
+        if (a.x_is_fp16) {
+            hipLaunchKernelGGL((dispatch_smooth_kernel<1>), grid, block, 0, stream, a);
+        } else {
+            hipLaunchKernelGGL((dispatch_smooth_kernel<0>), grid, block, 0, stream, a);
+        }
+        return hipGetLastError();
+    }
     if (a.quant == 0) {
         hipLaunchKernelGGL((dispatch_kernel<0, 0>), grid, block, 0, stream, a);  // a copy does not look at the format
     } else if (a.quant == 1) {

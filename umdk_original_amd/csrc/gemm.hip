@@ -50,6 +50,8 @@
 //     their last sub-steps, where tall items keep a branch-free loop body and fetch the last sub-step again;
 //     and between the K loop and the epilogue of a flat item the workgroup takes its next item and, if that
 //     is flat too, touches the lines of its first stages so that they travel to L2 under the epilogue.
+#include <atomic>
+
 #include "cam_device.h"
 #include "cam_kernels.h"
 #include "rank_device.h"
@@ -96,10 +98,6 @@ __device__ __forceinline__ void dma16_stream(const void *base, unsigned voff, un
                  : "s"(lds_addr), "v"(voff), "s"((unsigned long long)base)
                  : "memory", "m0");
 }
-
-#ifndef CAM_TALL_WEIGHTS_STREAM
-#define CAM_TALL_WEIGHTS_STREAM 0
-#endif
 
 template <int N>
 __device__ __forceinline__ void wait_loads_outstanding()
@@ -222,7 +220,7 @@ __device__ __forceinline__ void run_item(const GemmArgs &a, const ItemCtx &t, in
             const int8_t *bb = b_base + (long long)s * b_step;
 #pragma unroll
             for (int j = 0; j < NB; ++j) {
-                if (FLAT || CAM_TALL_WEIGHTS_STREAM) {  // a flat item is the only reader of its weight panel
+                if (FLAT) {  // a flat item is the only reader of its weight panel
                     dma16_stream(bb + j * 1024, b_voff, sbase + b_dst + j * 1024);
                 } else {
                     dma16(bb + j * 1024, b_voff, sbase + b_dst + j * 1024);
@@ -971,7 +969,32 @@ __global__ __launch_bounds__(256) void prepack_kernel(const int8_t *__restrict__
     *((v4u *)(dst + (long long)g * Kd * N) + q) = o;
 }
 
-int g_num_cus = 0;  // workgroups of the persistent kernel: one per CU of the current device
+// Workgroups of the persistent kernel: one per CU of the device the launch goes to (looked up once per device).
+constexpr int kMaxDevices = 64;
+std::atomic<int> g_num_cus[kMaxDevices];
+
+hipError_t cus_of_current_device(int *out)
+{
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) {
+        return e;
+    }
+    if (dev < 0 || dev >= kMaxDevices) {
+        return hipErrorInvalidDevice;
+    }
+    int n = g_num_cus[dev].load(std::memory_order_relaxed);
+    if (n == 0) {
+        e = hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev);
+        if (e != hipSuccess) {
+            return e;
+        }
+        n = n > 0 ? n : 256;
+        g_num_cus[dev].store(n, std::memory_order_relaxed);
+    }
+    *out = n;
+    return hipSuccess;
+}
 
 }  // namespace
 
@@ -1024,16 +1047,10 @@ hipError_t launch_gemm(const GemmArgs &a, hipStream_t stream)
     if (a.Kd % kBK != 0 || a.Kd < kBK || a.N % 64 != 0 || (a.gate_up && a.N % 128 != 0)) {
         return hipErrorInvalidValue;
     }
-    if (g_num_cus == 0) {
-        int dev = 0, n = 0;
-        hipError_t e = hipGetDevice(&dev);
-        if (e == hipSuccess) {
-            e = hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev);
-        }
-        if (e != hipSuccess) {
-            return e;
-        }
-        g_num_cus = n > 0 ? n : 256;
+    int num_cus = 0;
+    const hipError_t ce = cus_of_current_device(&num_cus);
+    if (ce != hipSuccess) {
+        return ce;
     }
     if (a.fp8) {
         if (a.Kd % 128 != 0 || a.N % 128 != 0 || (a.gate_up && a.N % 256 != 0) || a.Kd / 128 > kScaleKb ||
@@ -1043,12 +1060,12 @@ hipError_t launch_gemm(const GemmArgs &a, hipStream_t stream)
         if (a.epilogue == kEpiSwigluFp8 && (!a.gate_up || a.out_scale8 == nullptr)) {
             return hipErrorInvalidValue;
         }
-        hipLaunchKernelGGL(gemm_kernel<true>, dim3((unsigned)g_num_cus), dim3(kThreads), 0, stream, a);
+        hipLaunchKernelGGL(gemm_kernel<true>, dim3((unsigned)num_cus), dim3(kThreads), 0, stream, a);
     } else {
         if (a.epilogue == kEpiSwigluFp8) {
             return hipErrorInvalidValue;
         }
-        hipLaunchKernelGGL(gemm_kernel<false>, dim3((unsigned)g_num_cus), dim3(kThreads), 0, stream, a);
+        hipLaunchKernelGGL(gemm_kernel<false>, dim3((unsigned)num_cus), dim3(kThreads), 0, stream, a);
     }
     return hipGetLastError();
 }

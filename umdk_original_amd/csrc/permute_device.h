@@ -171,6 +171,50 @@ __device__ __forceinline__ void quant_token_row(TokenRow &r)
     }
 }
 
+// Quantisation of one COPY of a token row under a per-expert smooth scale
+// (src/cam/comm_operator/ascend_kernels/moe_dispatch_shmem/op_kernel/moe_dispatch_shmem.h:693-733):
+// xf = float(x) * smooth[h] (one rounded multiply), then the no-epsilon variant on xf.  r.raw is left untouched.
+template <int ACT>
+__device__ __forceinline__ void quant_token_row_smooth(TokenRow &r, const float *__restrict__ smooth, int H, int lane)
+{
+    const int nch = H >> 3;
+    float m = 0.0f;
+#pragma unroll
+    for (int j = 0; j < kDispMaxChunks; ++j) {
+        const int c = j * kWave + lane;
+        if (c < nch) {
+            const v4f s0 = *(const v4f *)(smooth + c * 8);
+            const v4f s1 = *(const v4f *)(smooth + c * 8 + 4);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const float sa = i < 2 ? s0[2 * i] : s1[2 * i - 4], sb = i < 2 ? s0[2 * i + 1] : s1[2 * i - 3];
+                m = fmaxf(m, fabsf(__fmul_rn(act_bits_to_f32<ACT>(r.raw[j][i] & 0xffffu), sa)));
+                m = fmaxf(m, fabsf(__fmul_rn(act_bits_to_f32<ACT>(r.raw[j][i] >> 16), sb)));
+            }
+        }
+    }
+    m = wave_max(m);
+    const bool zero_row = m == 0.0f;
+    const float s = zero_row ? 0.0f : __fdiv_rn(127.0f, m);
+    r.scale_out = zero_row ? 0.0f : __fdiv_rn(1.0f, s);
+#pragma unroll
+    for (int j = 0; j < kDispMaxChunks; ++j) {
+        const int c = j * kWave + lane;
+        int v[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+        if (c < nch) {
+            const v4f s0 = *(const v4f *)(smooth + c * 8);
+            const v4f s1 = *(const v4f *)(smooth + c * 8 + 4);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const float sa = i < 2 ? s0[2 * i] : s1[2 * i - 4], sb = i < 2 ? s0[2 * i + 1] : s1[2 * i - 3];
+                v[2 * i] = (int)rintf(__fmul_rn(__fmul_rn(act_bits_to_f32<ACT>(r.raw[j][i] & 0xffffu), sa), s));
+                v[2 * i + 1] = (int)rintf(__fmul_rn(__fmul_rn(act_bits_to_f32<ACT>(r.raw[j][i] >> 16), sb), s));
+            }
+        }
+        r.q[j] = v2u{pack4(v[0], v[1], v[2], v[3]), pack4(v[4], v[5], v[6], v[7])};
+    }
+}
+
 // Stores the row (quantised or raw) to output row `row`, with its scale and triple.
 template <int QUANT>
 __device__ __forceinline__ void store_token_row(const TokenRow &r, void *out, float *scales, int32_t *src_info,

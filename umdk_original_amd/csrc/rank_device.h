@@ -1,4 +1,4 @@
-// Device code shared by the routing-plan kernels and the single-launch dispatch: id loading, workgroup
+// Device code shared by the routing-plan kernels: id loading, workgroup
 // scans and the stable ranking of one chunk of the flat (token, k) id sequence.
 #ifndef CAM_RANK_DEVICE_H_
 #define CAM_RANK_DEVICE_H_
@@ -78,9 +78,8 @@ __device__ __forceinline__ int count_active(const uint8_t *mask, int T, int tid,
 // group, and the group's highest lane publishes the new count.  A scan over the 4 waves' histograms
 // turns wave-local ranks into chunk-local ones.  Writes the chunk-local rank of every entry below
 // n_all to pos_out (-1 for skipped entries and entries at or beyond n) and the chunk's per-expert
-// histogram to hist_row[0..E).  `hist` is LDS, kLocalWaves * kMaxExperts ints.  WRITE_THROUGH: the results
-// are for other workgroups of the same launch and are stored with device-scope write-through stores.
-template <typename IdT, int IT, bool WRITE_THROUGH = false>
+// histogram to hist_row[0..E).  `hist` is LDS, kLocalWaves * kMaxExperts ints.
+template <typename IdT, int IT>
 __device__ __forceinline__ void rank_chunk(const IdT *__restrict__ idx, int b, long long n, long long n_all, int E,
                                            int *hist, int32_t *pos_out, int32_t *hist_row)
 {
@@ -135,11 +134,7 @@ __device__ __forceinline__ void rank_chunk(const IdT *__restrict__ idx, int b, l
             hist[ww * kMaxExperts + ee] = run;
             run += t;
         }
-        if (WRITE_THROUGH) {
-            __hip_atomic_store(&hist_row[ee], run, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        } else {
-            hist_row[ee] = run;
-        }
+        hist_row[ee] = run;
     }
     __syncthreads();
 #pragma unroll
@@ -147,11 +142,7 @@ __device__ __forceinline__ void rank_chunk(const IdT *__restrict__ idx, int b, l
         const long long i = base + it * kWave + lane;
         if (i < n_all) {
             const int v = e[it] >= 0 ? r[it] + my_hist[e[it]] : -1;
-            if (WRITE_THROUGH) {
-                __hip_atomic_store(&pos_out[i], v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            } else {
-                pos_out[i] = v;
-            }
+            pos_out[i] = v;
         }
     }
 }

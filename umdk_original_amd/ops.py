@@ -27,6 +27,7 @@ from ._lib import CamError, CAM_FORMAT_MFMA_B
 
 __all__ = [
     "CamError", "get_dispatch_layout", "moe_dispatch_plan", "moe_dispatch_fused", "moe_dispatch_prefill", "moe_dispatch_normal",
+    "moe_dispatch_shmem", "moe_combine_shmem",
     "moe_combine_prefill", "moe_combine_normal", "moe_combine_index", "moe_combine_gather", "notify_dispatch", "prepack_weight",
     "grouped_matmul_swiglu_quant", "grouped_matmul_dequant", "grouped_matmul_int32", "fused_deep_moe",
 ]
@@ -98,17 +99,6 @@ def moe_dispatch_plan(topk_idx, num_experts, num_ranks=1, rank=0):
                                   out["recv_count"], out["num_recv_tokens_per_expert"], out["total"],
                                   out["slot_row"]])
     return out
-
-
-DISPATCH_LAUNCH_AUTO, DISPATCH_LAUNCH_SINGLE, DISPATCH_LAUNCH_SEPARATE = 0, 1, 2
-
-
-def set_dispatch_launch_mode(mode):
-    """Process-wide choice between the single-launch dispatch and the plan's and the permute's own launches
-    (camSetDispatchLaunchMode); the results do not depend on it."""
-    status = _lib.lib().camSetDispatchLaunchMode(int(mode))
-    if status != 0:
-        raise CamError("camSetDispatchLaunchMode failed (%d): %s" % (status, _lib.recent_error()))
 
 
 def moe_dispatch_fused(x, topk_idx, num_experts, quant_mode=0, num_rows=None, rank=0, num_ranks=1):
@@ -235,11 +225,13 @@ def moe_combine_index(token_src_info, num_rows, num_tokens, top_k):
     return slot_row
 
 
-def moe_combine_gather(recv_x, token_src_info, slot_row, topk_weights, out=None, ep_recv_counts=None):
+def moe_combine_gather(recv_x, token_src_info, slot_row, topk_weights, out=None, ep_recv_counts=None,
+                       shared_x=None):
     """Weighted gather-reduce with a prebuilt map: -> combined bf16 [T,H].
 
     token_src_info=None trusts slot_row as it stands (the dispatch operators' slot_row output); with the
     triples given, entries whose row does not point back at the slot are skipped (a map from moe_combine_index).
+    shared_x [T,H]: the shared expert's rows, added un-weighted after the routed rows, before the rounding.
     """
     _require_gpu(recv_x, "recv_x")
     if out is None:
@@ -247,7 +239,49 @@ def moe_combine_gather(recv_x, token_src_info, slot_row, topk_weights, out=None,
         h = recv_x.size(1) // 5 * 4 if recv_x.dtype == torch.int8 else recv_x.size(1)
         out = torch.empty((topk_weights.size(0), h),
                           dtype=torch.bfloat16 if recv_x.dtype == torch.int8 else recv_x.dtype, device=recv_x.device)
-    _lib.call("MoeCombineGather", [recv_x, token_src_info, slot_row, ep_recv_counts, topk_weights, out])
+    _lib.call("MoeCombineGather", [recv_x, token_src_info, slot_row, ep_recv_counts, topk_weights, shared_x, out])
+    return out
+
+
+def moe_dispatch_shmem(x, expertIds, scales=None, xActiveMask=None, epWorldSize=1, epRankId=0, moeExpertNum=0,
+                       tpWorldSize=1, tpRankId=0, expertShardType=0, sharedExpertNum=1, sharedExpertRankNum=0,
+                       quantMode=0, globalBS=0, expertTokenNumsType=1, extInfo=0):
+    """The reference's moe_dispatch_shmem on one rank (src/cam/comm_operator/pybind/moe_dispatch_shmem.cpp:27-153).
+    -> [expandX [bs*min(K, experts), H], dynamicScales fp32, expandIdx int32 [bs*K], expertTokenNums int64,
+        epRecvCount int32, tpRecvCount int32 [tpWorldSize]]"""
+    _require_gpu(x, "x")
+    bs, h = x.shape
+    k = expertIds.size(1)
+    _bind_assert(epWorldSize != sharedExpertRankNum, "epWorldSize != sharedExpertRankNum")
+    per_rank = moeExpertNum // (epWorldSize - sharedExpertRankNum)
+    rows = bs * epWorldSize * min(per_rank, k)
+    dev = x.device
+    expand_x = torch.empty((rows, h), dtype=torch.int8 if quantMode == 2 else x.dtype, device=dev)
+    dyn = torch.empty(rows, dtype=torch.float32, device=dev)
+    expand_idx = torch.empty(bs * k, dtype=torch.int32, device=dev)
+    etn = torch.empty(per_rank, dtype=torch.int64, device=dev)
+    ep_cnt = torch.empty(epWorldSize * per_rank, dtype=torch.int32, device=dev)
+    tp_cnt = torch.empty(tpWorldSize, dtype=torch.int32, device=dev)
+    _lib.call("MoeDispatchShmem", [x, expertIds, scales, xActiveMask, epWorldSize, epRankId, moeExpertNum, tpWorldSize,
+                                   tpRankId, expertShardType, sharedExpertNum, sharedExpertRankNum, quantMode,
+                                   globalBS, expertTokenNumsType, extInfo, expand_x, dyn, expand_idx, etn, ep_cnt,
+                                   tp_cnt])
+    return [expand_x, dyn, expand_idx, etn, ep_cnt, tp_cnt]
+
+
+def moe_combine_shmem(expandX, expertIds, expandIdx, epSendCounts, expertScales, tpSendCounts=None,
+                      xActiveMask=None, activationScale=None, weightScale=None, groupList=None, expandScales=None,
+                      epWorldSize=1, epRankId=0, moeExpertNum=0, tpWorldSize=1, tpRankId=0, expertShardType=0,
+                      sharedExpertNum=1, sharedExpertRankNum=0, globalBS=0, commQuantMode=0, extInfo=0, outDtype=0,
+                      groupListType=0):
+    """The reference's moe_combine_shmem on one rank (src/cam/comm_operator/pybind/moe_combine_shmem.cpp:27-86).
+    -> out [bs,H], dtype of expandX."""
+    _require_gpu(expandX, "expandX")
+    out = torch.empty((expertIds.size(0), expandX.size(1)), dtype=expandX.dtype, device=expandX.device)
+    _lib.call("MoeCombineShmem", [expandX, expertIds, expandIdx, epSendCounts, expertScales, tpSendCounts, xActiveMask,
+                                  activationScale, weightScale, groupList, expandScales, epWorldSize, epRankId,
+                                  moeExpertNum, tpWorldSize, tpRankId, expertShardType, sharedExpertNum,
+                                  sharedExpertRankNum, globalBS, commQuantMode, extInfo, outDtype, groupListType, out])
     return out
 
 
@@ -418,6 +452,16 @@ def register_torch_ops():
                "int rank, int num_ranks) -> (Tensor, Tensor, Tensor, Tensor)")
     lib.define("moe_combine_prefill(Tensor x, Tensor topk_idx, Tensor topk_weights, Tensor src_idx, "
                "Tensor send_head, str group_ep, int rank, int num_ranks) -> Tensor")
+    lib.define("moe_dispatch_shmem(Tensor x, Tensor expertIds, Tensor? scales, Tensor? xActiveMask, "
+               "int epWorldSize, int epRankId, int moeExpertNum, int tpWorldSize, int tpRankId, "
+               "int expertShardType, int sharedExpertNum, int sharedExpertRankNum, int quantMode, int globalBS, "
+               "int expertTokenNumsType, int extInfo) -> Tensor[]")
+    lib.define("moe_combine_shmem(Tensor expandX, Tensor expertIds, Tensor expandIdx, Tensor epSendCounts, "
+               "Tensor expertScales, Tensor? tpSendCounts, Tensor? xActiveMask, Tensor? activationScale, "
+               "Tensor? weightScale, Tensor? groupList, Tensor? expandScales, int epWorldSize, int epRankId, "
+               "int moeExpertNum, int tpWorldSize, int tpRankId, int expertShardType, int sharedExpertNum, "
+               "int sharedExpertRankNum, int globalBS, int commQuantMode, int extInfo, int outDtype, "
+               "int groupListType) -> Tensor")
 
     def _fused(x, expertIds, w1, w1s, w2, w2s, expertScales, smooth, mask, groupEp, epRankSize, epRankId,
                moeExpertNum, sharedExpertNum, sharedExpertRankNum, quantMode, globalBs):
@@ -440,6 +484,8 @@ def register_torch_ops():
     lib.impl("moe_dispatch_prefill",
              lambda *a: tuple(moe_dispatch_prefill(*a)), "CUDA")
     lib.impl("moe_combine_prefill", moe_combine_prefill, "CUDA")
+    lib.impl("moe_dispatch_shmem", moe_dispatch_shmem, "CUDA")
+    lib.impl("moe_combine_shmem", moe_combine_shmem, "CUDA")
     _torch_lib = lib
     return lib
 
