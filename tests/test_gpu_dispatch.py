@@ -280,7 +280,7 @@ def test_dispatch_prefill_full_size_config(gpu, oracle):
 @pytest.mark.parametrize("quant_mode", [0, 2, 3])
 def test_dispatch_fp16_activations(gpu, oracle, quant_mode):
     """fp16 activations (moe_dispatch_normal.cpp op_host :17-22 lists them beside bf16), both dispatch operators."""
-    announce("dispatch fp16 quant=%d (%s)" % (quant_mode))
+    announce("dispatch fp16 quant=%d" % quant_mode)
     T, K, E, H = 70, 4, 16, 2048
     ids = _random_ids(T, K, E, seed=61, neg_frac=0.1)
     x = (torch.randn(T, H, generator=torch.Generator().manual_seed(62)) * 4).half()

@@ -312,14 +312,93 @@ def test_expf_scaling_by_two_multiplies_equals_ldexp():
             assert np.array_equal(two_step.view(np.uint32), one_step.view(np.uint32)), n
 
 
-def test_silu_against_float64(oracle):
-    ts = _rng(11).normal(0, 4, 5000).astype(np.float32)
+def _silu64(t):
+    t = np.asarray(t, np.float64)
+    with np.errstate(over="ignore"):
+        return t / (1.0 + np.exp(-t))
+
+
+def test_silu_spec_accuracy_against_float64(oracle):
+    """The bounds the specification states (include/cam_expf_spec.h): 6e-6 relative for |t| <= 20, 1.2e-5 for
+    |t| <= 86, below 4e-36 absolute beyond; exact at 0 and at +inf."""
+    rng = _rng(11)
+    ts = np.concatenate([np.linspace(-86, 86, 60001), rng.normal(0, 4, 30000), rng.uniform(-20, 20, 30000),
+                         [2.0 ** -k for k in range(0, 140, 3)], [-(2.0 ** -k) for k in range(0, 140, 3)]]).astype(np.float32)
     got = np.array([oracle.silu(float(t)) for t in ts], np.float64)
-    want = ts.astype(np.float64) / (1.0 + np.exp(-ts.astype(np.float64)))
-    assert np.allclose(got, want, rtol=5e-7, atol=1e-30)
-    assert oracle.silu(0.0) == 0.0
-    assert oracle.silu(-1000.0) == 0.0 or oracle.silu(-1000.0) == -0.0
-    assert oracle.silu(1000.0) == 1000.0
+    want = _silu64(ts)
+    err = np.abs(got - want)
+    near = np.abs(ts) <= 20
+    assert (err[near] <= 6e-6 * np.abs(want[near]) + 1e-45).all(), (err[near] / np.abs(want[near]).clip(1e-300)).max()
+    assert (err <= 1.2e-5 * np.abs(want) + 1e-45).all(), (err / np.abs(want).clip(1e-300)).max()
+    far = np.array([87.0, 100.0, 1e4, 1e30, 3e38], np.float32)
+    for t in far:
+        assert oracle.silu(float(t)) == float(t)                       # t - 86 q with q ~ 4e-38
+        assert abs(oracle.silu(-float(t)) - _silu64(-float(t))) < 4e-36
+    assert oracle.silu(0.0) == 0.0 and oracle.silu(-0.0) == 0.0
+    assert math.isinf(oracle.silu(float("inf"))) and oracle.silu(float("inf")) > 0
+    assert abs(oracle.silu(float("-inf"))) < 4e-36
+    # silu(t) - silu(-t) == t up to the roundings of the two results
+    pos = np.abs(ts[:60001:7])
+    d = np.array([oracle.silu(float(t)) - oracle.silu(-float(t)) for t in pos])
+    assert np.allclose(d, pos, rtol=3e-7, atol=1e-37)
+
+
+def _round_f32(fr):
+    """Correctly rounded (nearest, ties to even) binary32 value of an exact Fraction, as np.float32 (normal range)."""
+    from fractions import Fraction
+    if fr == 0:
+        return np.float32(0.0)
+    sign = -1 if fr < 0 else 1
+    fr = abs(fr)
+    e = fr.numerator.bit_length() - fr.denominator.bit_length()
+    if Fraction(2) ** e > fr:
+        e -= 1
+    assert -126 <= e <= 127, e                      # the specification never leaves the normal range
+    scaled = fr / Fraction(2) ** (e - 23)           # in [2^23, 2^24)
+    m = scaled.numerator // scaled.denominator
+    rem = scaled - m
+    if rem > Fraction(1, 2) or (rem == Fraction(1, 2) and m % 2 == 1):
+        m += 1
+    return np.float32(sign * float(m) * 2.0 ** (e - 23))   # m <= 2^24 and the power are exact in a double
+
+
+def test_silu_spec_is_the_written_operation_sequence_bit_for_bit(oracle):
+    """An independent restatement in exact rational arithmetic, every written operation rounded to binary32 once
+    (a fused multiply-add is ONE rounding of a*b + c).  It fails if the C build splits a fused operation, fuses a
+    split one, evaluates the polynomial in another order or scales by the power of two inexactly."""
+    from fractions import Fraction as F
+
+    def fr(v):
+        return F(float(v))
+
+    def fma(a, b, c):
+        return _round_f32(fr(a) * fr(b) + fr(c))
+
+    def spec(t):
+        t = np.float32(t)
+        a = np.float32(min(abs(float(t)), 86.0))
+        z = _round_f32(fr(a) * fr(np.float32(-1.44269504088896341)))
+        n = np.float32(np.rint(z))
+        f = _round_f32(fr(z) - fr(n))
+        p = fma(f, np.float32(9.570102e-3), np.float32(5.591786e-2))
+        p = fma(f, p, np.float32(2.4024744e-1))
+        p = fma(f, p, np.float32(6.931218e-1))
+        p = fma(f, p, np.float32(9.999993e-1))
+        e = _round_f32(fr(p) * F(2) ** int(n))
+        d = _round_f32(fr(e) + 1)
+        r = fma(d, np.float32(3.2323232e-1), np.float32(-1.4545455))
+        r = fma(d, r, np.float32(2.121212))
+        u = fma(-d, r, np.float32(1.0))
+        r = fma(fma(u, u, u), r, r)
+        q = _round_f32(fr(e) * fr(r))
+        return fma(-a, q, np.float32(max(float(t), 0.0)))
+
+    rng = _rng(12)
+    ts = np.concatenate([rng.normal(0, 3, 1500), rng.uniform(-90, 90, 600), [0.5, -0.5, 1.0, -1.0, 86.0, -86.0, 1e-20, 20.0, -20.0],
+                         np.float32(np.arange(-40, 41)) * np.float32(0.6931472)]).astype(np.float32)
+    for t in ts:
+        got, want = np.float32(oracle.silu(float(t))), spec(t)
+        assert got.view(np.uint32) == want.view(np.uint32), (float(t), float(got), float(want))
 
 
 def test_gmm1_epilogue_halves_scale_order_and_grouping(oracle):
