@@ -290,10 +290,12 @@ camStatus check_gemm_dims(const char *op, int64_t Kd, int64_t N, bool gate_up)
 }
 
 // One schedule for a GEMM of N packed columns over `rows` rows of G experts, carved out of a workspace.
-cam::SchedSpec sched_spec(int64_t rows, int64_t G, int64_t N)
+cam::SchedSpec sched_spec(int64_t rows, int64_t G, int64_t N, int64_t Kd, bool swiglu)
 {
     cam::SchedSpec sp{};
     sp.N = (int)N;
+    sp.Kd = (int)Kd;
+    sp.swiglu = swiglu ? 1 : 0;
     sp.max_items = cam::sched_max_items(rows, (int)G, (int)N);
     return sp;
 }
@@ -1498,7 +1500,7 @@ camStatus camGroupedMatmulSwigluQuantGetWorkspaceSize(const camTensor *x, const 
     WeightSet ws{};
     CAM_TRY(resolve_weights(weight, weightScale, "weight", gc.G, gc.Kd, 2 * I, true, &ws));
     CAM_TRY(check_aligned(y, "y", 16));
-    cam::SchedSpec sp = sched_spec(gc.A, gc.G, 2 * I);
+    cam::SchedSpec sp = sched_spec(gc.A, gc.G, 2 * I, gc.Kd, true);
     Carver c;
     const uint64_t o_sched = c.take(cam::sched_bytes(gc.A, (int)gc.G, (int)(2 * I)));
     const uint64_t o_prod = c.take((uint64_t)gc.A * I * 4);
@@ -1562,7 +1564,7 @@ camStatus camGroupedMatmulDequantGetWorkspaceSize(const camTensor *x, const camT
     CAM_TRY(check_aligned(out, "out", 16));
     WeightSet ws{};
     CAM_TRY(resolve_weights(weight, weightScale, "weight", gc.G, gc.Kd, N, true, &ws));
-    cam::SchedSpec sp = sched_spec(gc.A, gc.G, N);
+    cam::SchedSpec sp = sched_spec(gc.A, gc.G, N, gc.Kd, false);
     Carver c;
     const uint64_t o_sched = c.take(cam::sched_bytes(gc.A, (int)gc.G, (int)N));
     const uint64_t o_rows = wire ? c.take((uint64_t)gc.A * N * 2) : 0;  // the bf16 rows before quantisation
@@ -1623,7 +1625,7 @@ camStatus camGroupedMatmulInt32GetWorkspaceSize(const camTensor *x, const camTen
     CAM_TRY(check_aligned(out, "out", 16));
     WeightSet ws{};
     CAM_TRY(resolve_weights(weight, nullptr, "weight", gc.G, gc.Kd, N, false, &ws));
-    cam::SchedSpec sp = sched_spec(gc.A, gc.G, N);
+    cam::SchedSpec sp = sched_spec(gc.A, gc.G, N, gc.Kd, false);
     Carver c;
     const uint64_t o_sched = c.take(cam::sched_bytes(gc.A, (int)gc.G, (int)N));
     cam::GemmArgs g{};
@@ -1763,8 +1765,8 @@ camStatus camFusedDeepMoeGetWorkspaceSize(const camTensor *x, const camTensor *e
     CAM_TRY(check_aligned(output, "output", 16));
 
     const int64_t A = T * K;  // maxTokenNum of AK/fused_deep_moe/op_kernel/fused_deep_moe.h:336 for one rank
-    cam::SchedSpec sp1 = sched_spec(A, Epr, 2 * I);
-    cam::SchedSpec sp2 = sched_spec(A, Epr, H);
+    cam::SchedSpec sp1 = sched_spec(A, Epr, 2 * I, H, true);
+    cam::SchedSpec sp2 = sched_spec(A, Epr, H, I, false);
     Carver c;
     const uint64_t o_pos = c.take((uint64_t)A * 4);
     const uint64_t o_row = c.take((uint64_t)A * 4);
@@ -2003,7 +2005,7 @@ camStatus camGroupedMatmulFp8GetWorkspaceSize(const camTensor *x, const camTenso
     CAM_TRY(check_aligned(out, "out", 16));
     Fp8Weight fw{};
     CAM_TRY(check_fp8_weight(weight, weightScale, "weight", G, Kd, N, &fw));
-    cam::SchedSpec sp = sched_spec(A, G, N);
+    cam::SchedSpec sp = sched_spec(A, G, N, Kd, gate_up);
     Carver c;
     const uint64_t o_sched = c.take(cam::sched_bytes(A, (int)G, (int)N));
     cam::GemmArgs g{};
@@ -2124,8 +2126,8 @@ camStatus camFusedDeepMoeFp8GetWorkspaceSize(const camTensor *x, const camTensor
     CAM_TRY(check_aligned(output, "output", 16));
 
     const int64_t A = T * K;
-    cam::SchedSpec sp1 = sched_spec(A, E, 2 * I);
-    cam::SchedSpec sp2 = sched_spec(A, E, H);
+    cam::SchedSpec sp1 = sched_spec(A, E, 2 * I, H, true);
+    cam::SchedSpec sp2 = sched_spec(A, E, H, I, false);
     Carver c;
     const uint64_t o_pos = c.take((uint64_t)A * 4);
     const uint64_t o_row = c.take((uint64_t)A * 4);

@@ -13,15 +13,18 @@ constexpr int kMaxRanks = 384;
 constexpr int kMaxTopk = 16;
 constexpr int kMaxListExperts = 64;  // per-expert weight tensors that fit in the kernel arguments
 // GEMM schedule (device-built, one per GEMM launch): kSchedHeader ints, then the work items.
-//   [0] item count  [1] total rows  [2], [3] 0
-//   [kSchedQueueStart .. +8]  first item of each of the 8 queues, and the end of the last
-//   [kSchedQueueCount + 32 x] items already taken from queue x (zeroed by the builder, advanced by the GEMM);
-//                             one counter per 128-byte line, so that the queues do not share a line
-constexpr int kNumXcd = 8;  // queues of a schedule: workgroup i of a launch runs on XCD i % 8
-constexpr int kSchedHeader = 32 + 8 * 32;
+//   [0] item count  [1] total rows  [2] queues in use  [3] 0
+//   [kSchedQueueStart + w]     first item of the queue of workgroup w (w = 0 .. kMaxQueues; the last entry is
+//                              the end of the last queue)
+//   [kSchedQueueCount + 32 w]  items already handed out from queue w (set to 1 by the builder: the first item is
+//                              its workgroup's without asking; advanced by the GEMM); one counter per 128-byte
+//                              line, so that the queues do not share a line
+constexpr int kNumXcd = 8;       // workgroup i of a launch runs on XCD i % 8
+constexpr int kMaxQueues = 512;  // one queue per workgroup of the persistent GEMM (one workgroup per CU)
 constexpr int kSchedQueueStart = 4;
-constexpr int kSchedQueueCount = 32;
+constexpr int kSchedQueueCount = 544;
 constexpr int kSchedQueueStride = 32;
+constexpr int kSchedHeader = kSchedQueueCount + kMaxQueues * kSchedQueueStride;
 // One work item: rows [m0, m0 + rows) of expert g times column block nb.  flat != 0: at most 128 rows x 512
 // packed columns, the two wave teams split the columns; flat == 0: at most 256 rows x 256 packed columns, team
 // 0 takes tile rows [0, split), team 1 the rest.
@@ -76,6 +79,8 @@ hipError_t launch_notify_scan(const int32_t *cnt, int E, int num_tokens, int32_t
 // one or two GEMMs over the same rows (they differ in the number of weight columns).
 struct SchedSpec {
     int N;             // packed weight columns of the GEMM
+    int Kd;            // its reduction length (the cost model of the builder needs it)
+    int swiglu;        // its epilogue forms SiLU(gate) * up (costlier per row than a plain dequantisation)
     int max_items;     // capacity of the item table (sched_max_items)
     int32_t *sched;    // sched_bytes() of device memory
 };
@@ -87,11 +92,12 @@ hipError_t launch_build_sched(const int64_t *group_list, int cumulative, int G, 
 struct SchedBuild {
     const int64_t *group_list;
     int cumulative, G, nspec;
+    int queues;        // workgroups of the GEMM launch the schedule is for (set by the launchers: CUs of the device)
     long long max_rows;
     SchedSpec spec[2];
 };
-// Workgroups that share the building of one schedule of sb (each writes every parts-th batch of 256 items).
-int sched_build_parts(const SchedBuild &sb);
+// CUs of the current device = workgroups of a GEMM launch = queues of its schedule.
+hipError_t gemm_workgroups(int *out);
 
 // ---------------------------------------------------------------------------------------------
 // Permute (+ per-token int8 quantisation).
@@ -112,11 +118,10 @@ struct DispatchArgs {
     // quant == 2 only: optional per-expert smooth scales fp32 [E,H].  Copy (t,k) is then quantised on its own,
     // from float(x[t]) * smooth[idx[t,k]] (moe_dispatch_shmem.h:693-733); idx must be set.
     const float *smooth;
-    // GEMM schedules to build in the same launch (sched.nspec > 0): sched.nspec * sched_parts extra workgroups
-    // do what launch_build_sched would, beside the ones that move rows.  The group list must be complete before
-    // the launch (it is when it comes from launch_plan on the same stream).  sched_parts is set by the launcher.
+    // GEMM schedules to build in the same launch (sched.nspec > 0): sched.nspec extra workgroups do what
+    // launch_build_sched would, beside the ones that move rows.  The group list must be complete before the
+    // launch (it is when it comes from launch_plan on the same stream).  sched.queues is set by the launcher.
     SchedBuild sched;
-    int sched_parts;
 };
 hipError_t launch_dispatch(const DispatchArgs &a, hipStream_t stream);
 

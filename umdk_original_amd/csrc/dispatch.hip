@@ -47,10 +47,9 @@ __global__ __launch_bounds__(kDispWaves * kWave, QUANT == 3 ? 3 : 4) void dispat
     // The first workgroups of the launch build the GEMM schedules (they start first and finish under the row
     // traffic of the others); they depend on nothing this launch writes.
     __shared__ SchedShared sched_s;
-    const int builders = a.sched.nspec * a.sched_parts;
+    const int builders = a.sched.nspec;
     if ((int)blockIdx.x < builders) {
-        build_sched_part<kDispWaves * kWave>(sched_s, a.sched, (int)blockIdx.x / a.sched_parts,
-                                             (int)blockIdx.x % a.sched_parts, a.sched_parts);
+        build_sched_part<kDispWaves * kWave>(sched_s, a.sched, (int)blockIdx.x, 0, 1);
         return;
     }
     const int t = ((int)blockIdx.x - builders) * kDispWaves + (threadIdx.x >> 6);
@@ -112,17 +111,17 @@ hipError_t launch_dispatch(const DispatchArgs &a_in, hipStream_t stream)
         return hipErrorInvalidValue;
     }
     DispatchArgs a = a_in;
-    a.sched_parts = 0;
     if (a.sched.nspec != 0) {
         if (a.sched.nspec < 0 || a.sched.nspec > 2 || a.sched.G <= 0 || a.sched.G > kMaxExperts ||
             a.sched.group_list == nullptr) {
             return hipErrorInvalidValue;
         }
-        // Few builders: every one repeats the per-expert tables, and the row traffic hides them anyway.
-        a.sched_parts = sched_build_parts(a.sched);
-        a.sched_parts = a.sched_parts > 8 ? 8 : a.sched_parts;
+        const hipError_t qe = gemm_workgroups(&a.sched.queues);
+        if (qe != hipSuccess) {
+            return qe;
+        }
     }
-    dim3 grid((a.T + kDispWaves - 1) / kDispWaves + a.sched.nspec * a.sched_parts), block(kDispWaves * kWave);
+    dim3 grid((a.T + kDispWaves - 1) / kDispWaves + a.sched.nspec), block(kDispWaves * kWave);
     if (a.smooth != nullptr) {
         if (a.quant != 2 || a.idx == nullptr || a.sched.nspec != 0) {
             return hipErrorInvalidValue;

@@ -50,6 +50,7 @@
 //     their last sub-steps, where tall items keep a branch-free loop body and fetch the last sub-step again;
 //     and between the K loop and the epilogue of a flat item the workgroup takes its next item and, if that
 //     is flat too, touches the lines of its first stages so that they travel to L2 under the epilogue.
+#include <algorithm>
 #include <atomic>
 
 #include "cam_device.h"
@@ -627,51 +628,72 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_kernel(GemmArgs a)
     const int32_t *qstart = sched + kSchedQueueStart;
     int32_t *qcount = sched + kSchedQueueCount;
     const SchedItem *items = (const SchedItem *)(sched + kSchedHeader);
-    const int q = blockIdx.x % kNumXcd;  // workgroup i runs on XCD i % 8
-    bool own_empty = false;
+    const int me = (int)blockIdx.x;            // this workgroup's queue
+    const int q0 = qstart[min(me, kMaxQueues)];
+    const int qlen = me < kMaxQueues ? qstart[me + 1] - q0 : 0;
+    bool own_empty = qlen <= 1;                // the first item needs no asking; there may be nothing after it
 
-    // Takes the next item (thread 0 only).  A device-scope atomic on a queue counter is a round trip to the
-    // memory side and atomics on one line are served one after the other, so: every queue counter has a line
-    // of its own, the take from the own queue is issued at the START of an item and looked at only when the
-    // item is done (take_begin / take_end), and other queues are tried only after a plain load has shown that
-    // they still hold items.  Every queue runs dry, so every workgroup leaves.
-    auto take_begin = [&]() -> int {
-        return own_empty ? 0 : atomicAdd(&qcount[q * kSchedQueueStride], 1);
+    // Work items.  Every workgroup has a queue of its own, built to last as long as the others (sched_device.h).
+    // Its first item is its own without asking; for the following ones it advances its queue's counter with a
+    // device-scope atomic, a round trip to the memory side that is issued at the START of an item and looked at
+    // only when the item is done (take_begin / take_end).  Every counter has a cache line of its own.  A
+    // workgroup whose queue has run out helps the queue with the most items left (its own XCD's first, so that
+    // what it fetches is likely to be in its L2): wave 0 looks at every counter at once, one round trip, and its
+    // first lane then advances the chosen one.  A counter only ever grows and every queue is finite, so every
+    // workgroup leaves.
+    auto take_begin = [&]() -> int {  // thread 0
+        return own_empty ? 0 : atomicAdd(&qcount[me * kSchedQueueStride], 1);
     };
-    auto take_end = [&](int taken) -> int {
-        if (!own_empty) {
-            const int i = qstart[q] + taken;
-            if (i < qstart[q + 1]) {
-                return i;
-            }
-            own_empty = true;
-        }
-        // Look at all the other queues at once: a look is a round trip to the memory side (1-2 us), and a
-        // workgroup that finds nothing does this before it leaves, so seven looks in a row would be the tail of
-        // every launch.
-        int seen[kNumXcd - 1], len[kNumXcd - 1];
-#pragma unroll
-        for (int k = 1; k < kNumXcd; ++k) {
-            const int qq = (q + k) % kNumXcd;
-            seen[k - 1] = __hip_atomic_load(&qcount[qq * kSchedQueueStride], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            len[k - 1] = qstart[qq + 1] - qstart[qq];
-        }
-#pragma unroll
-        for (int k = 1; k < kNumXcd; ++k) {
-            const int qq = (q + k) % kNumXcd;
-            if (seen[k - 1] < len[k - 1]) {
-                const int i = atomicAdd(&qcount[qq * kSchedQueueStride], 1);
-                if (i < len[k - 1]) {
-                    return qstart[qq] + i;
+    auto steal = [&]() -> int {  // all lanes of wave 0; the result is valid in every lane
+        const int lane = tid & (kWave - 1);
+        const int nq = min(sched[2], kMaxQueues);
+        for (int attempt = 0; attempt < 4; ++attempt) {
+            int best = -1;  // (items left, same XCD, queue) packed so that the maximum is the choice
+            for (int v = lane; v < nq; v += kWave) {
+                const int len = qstart[v + 1] - qstart[v];
+                const int seen = __hip_atomic_load(&qcount[v * kSchedQueueStride], __ATOMIC_RELAXED,
+                                                   __HIP_MEMORY_SCOPE_AGENT);
+                const int left = len - seen;
+                if (left > 0 && v != me) {
+                    best = max(best, (min(left, 1023) << 11) | ((v % kNumXcd == me % kNumXcd ? 1 : 0) << 10) | v);
                 }
+            }
+#pragma unroll
+            for (int off = 32; off > 0; off >>= 1) {
+                best = max(best, __shfl_xor(best, off, kWave));
+            }
+            if (best < 0) {
+                return -1;
+            }
+            // the queue number fits ten bits only below 1024 queues, which kMaxQueues guarantees
+            const int v = best & 1023;
+            int got = -1;
+            if (lane == 0) {
+                const int i = atomicAdd(&qcount[v * kSchedQueueStride], 1);
+                got = i < qstart[v + 1] - qstart[v] ? qstart[v] + i : -1;
+            }
+            got = __shfl(got, 0, kWave);
+            if (got >= 0) {
+                return got;
             }
         }
         return -1;
     };
+    // The item after the one whose take was `taken`; called by all threads of wave 0 (the answer is for thread 0).
+    auto take_end = [&](int taken) -> int {
+        taken = __shfl(taken, 0, kWave);
+        if (!own_empty) {
+            if (taken < qlen) {
+                return q0 + taken;
+            }
+            own_empty = true;
+        }
+        return steal();
+    };
 
     int next = -1;
-    if (tid == 0) {
-        next = take_end(take_begin());
+    if (tid < kWave) {
+        next = qlen > 0 ? q0 : steal();
     }
     for (;;) {
         if (tid == 0) {
@@ -687,6 +709,11 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_kernel(GemmArgs a)
             taken = take_begin();  // in flight while this item runs
         }
         SchedItem it = items[idx];
+#ifdef CAM_GEMM_TIMELINE
+        // Build option for profiling only: thread 0 leaves the item's start and end times (wall_clock64, 100 MHz)
+        // and the workgroup that ran it in the item's two spare words.
+        const long long timeline_t0 = wall_clock64();
+#endif
         const int g = __builtin_amdgcn_readfirstlane(it.g);
         const int m0 = __builtin_amdgcn_readfirstlane(it.m0);
         const int rows = __builtin_amdgcn_readfirstlane(it.rows);
@@ -747,9 +774,11 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_kernel(GemmArgs a)
         // one word of every 128-byte line of its first stages -- so that they are on their way to this XCD's L2
         // while the epilogue computes, and the next item's first direct-to-LDS loads find them there.
         auto between = [&]() -> int {
-            if (tid == 0) {
+            if (tid < kWave) {
                 next = take_end(taken);
-                next_s = next;
+                if (tid == 0) {
+                    next_s = next;
+                }
             }
             __syncthreads();
             const int nidx = next_s;
@@ -802,7 +831,15 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_kernel(GemmArgs a)
                 run_item_mf<1, false, FP8>(mf, a, t, nb, lds, row_scale_s, a_scale8_s, w_scale8_s, between, stage_scales);
             }
         }
-        if (!flat && tid == 0) {  // a flat item has taken its successor between its K loop and its epilogue
+#ifdef CAM_GEMM_TIMELINE
+        if (tid == 0) {
+            int32_t *stamp = (int32_t *)&items[idx];
+            stamp[6] = (int32_t)timeline_t0;
+            stamp[7] = (int32_t)wall_clock64();
+            stamp[3] = (stamp[3] & 0xffff) | ((int)blockIdx.x << 16);  // split is read at the start of the item only
+        }
+#endif
+        if (!flat && tid < kWave) {  // a flat item has taken its successor between its K loop and its epilogue
             next = take_end(taken);
         }
     }
@@ -811,7 +848,7 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_kernel(GemmArgs a)
 __global__ __launch_bounds__(1024) void build_sched_kernel(SchedBuild sb)
 {
     __shared__ SchedShared sh;
-    build_sched_part<1024>(sh, sb, (int)blockIdx.y, (int)blockIdx.x, (int)gridDim.x);
+    build_sched_part<1024>(sh, sb, (int)blockIdx.x, 0, 1);
 }
 
 // SwiGLU product rows (fp32) -> int8 rows + per-row scale:
@@ -1000,7 +1037,7 @@ hipError_t cus_of_current_device(int *out)
 
 int sched_max_items(int64_t max_rows, int G, int N)
 {
-    // tall tiles hold more than 128 rows each, flat tiles are one per expert
+    // tall experts own at most max_rows / 129 + G row tiles between them, flat experts one each
     const int64_t tiles = max_rows / 129 + G;
     return (int)(tiles * ((N + 255) / 256));
 }
@@ -1010,14 +1047,14 @@ uint64_t sched_bytes(int64_t max_rows, int G, int N)
     return (uint64_t)(kSchedHeader + (int64_t)sched_max_items(max_rows, G, N) * (int)(sizeof(SchedItem) / 4)) * 4;
 }
 
-int sched_build_parts(const SchedBuild &sb)
+hipError_t gemm_workgroups(int *out)
 {
-    int most = 0;
-    for (int i = 0; i < sb.nspec; ++i) {
-        most = sb.spec[i].max_items > most ? sb.spec[i].max_items : most;
+    int n = 0;
+    const hipError_t e = cus_of_current_device(&n);
+    if (e == hipSuccess) {
+        *out = n < kMaxQueues ? n : kMaxQueues;
     }
-    const int parts = (most + 255) / 256;
-    return parts < 1 ? 1 : (parts > 64 ? 64 : parts);
+    return e;
 }
 
 hipError_t launch_build_sched(const int64_t *group_list, int cumulative, int G, int64_t max_rows, int nspec,
@@ -1034,8 +1071,11 @@ hipError_t launch_build_sched(const int64_t *group_list, int cumulative, int G, 
     sb.max_rows = (long long)max_rows;
     sb.spec[0] = specs[0];
     sb.spec[1] = nspec > 1 ? specs[1] : specs[0];
-    hipLaunchKernelGGL(build_sched_kernel, dim3((unsigned)sched_build_parts(sb), (unsigned)nspec), dim3(1024), 0,
-                       stream, sb);
+    const hipError_t qe = gemm_workgroups(&sb.queues);
+    if (qe != hipSuccess) {
+        return qe;
+    }
+    hipLaunchKernelGGL(build_sched_kernel, dim3((unsigned)nspec), dim3(1024), 0, stream, sb);
     return hipGetLastError();
 }
 
@@ -1048,7 +1088,7 @@ hipError_t launch_gemm(const GemmArgs &a, hipStream_t stream)
         return hipErrorInvalidValue;
     }
     int num_cus = 0;
-    const hipError_t ce = cus_of_current_device(&num_cus);
+    const hipError_t ce = gemm_workgroups(&num_cus);
     if (ce != hipSuccess) {
         return ce;
     }
