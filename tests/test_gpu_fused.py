@@ -156,3 +156,29 @@ def test_torch_ops_are_the_cpp_library_and_check_the_weight_mark(gpu, oracle):
         torch.ops.umdk_cam_op_lib.fused_deep_moe(*args(w1p, w2.to(gpu)))
     with pytest.raises(RuntimeError, match="prepack_weight"):
         torch.ops.umdk_cam_op_lib.fused_deep_moe(*args(w2p, w2p))   # packed for the other projection
+
+
+@pytest.mark.parametrize("T", [8192, 128])
+def test_fused_layer_at_the_benchmarked_qwen3_shapes_sampled_tokens(gpu, oracle, T):
+    """The w8a8 layer at the shapes whose time is reported (hidden 4096, 128 experts, top-8, intermediate 1536;
+    8192 and 128 tokens).  A token's output depends on its own row, its routing and the weights only, so the oracle
+    runs on a sample of tokens and must reproduce those rows of the full-size result bit for bit; the per-expert
+    totals are checked against a bincount of all ids."""
+    announce("fused w8a8 layer at the benchmarked shape, T=%d, sampled tokens" % T)
+    H, E, K, I = 4096, 128, 8, 1536
+    ids, gates = synth.sigmoid_zipf_routing(T, E, K, seed=47)
+    g = torch.Generator().manual_seed(471)
+    w1 = torch.randint(-127, 128, (E, H, 2 * I), generator=g, dtype=torch.int8)
+    w2 = torch.randint(-127, 128, (E, I, H), generator=g, dtype=torch.int8)
+    w1s = synth.channel_scales((E, 2 * I), 472)
+    w2s = synth.channel_scales((E, H), 473)
+    x = synth.normal_bf16(T, H, seed=474)
+    out, etn = cam.fused_deep_moe(x.to(gpu), ids.to(torch.int32).to(gpu), [cam.prepack_weight(w1.to(gpu), True)],
+                                  [w1s.to(gpu)], [cam.prepack_weight(w2.to(gpu), False)], [w2s.to(gpu)],
+                                  gates.to(gpu), None, None, "", 1, 0, E, 1, 0, 0, 0)
+    assert np.array_equal(etn.cpu().numpy(), np.bincount(ids.numpy().reshape(-1), minlength=E))
+    pick = np.unique(np.concatenate([[0, 1, T - 1], np.random.default_rng(12).integers(0, T, 37)]))
+    want, _ = oracle.fused_layer(synth.bf16_bits(x)[pick], ids.numpy()[pick].astype(np.int64), gates.numpy()[pick],
+                                 w1.numpy(), w1s.numpy(), w2.numpy(), w2s.numpy())
+    assert_bits_equal(to_np(out)[pick], want, "layer output rows of the sampled tokens")
+    assert torch.isfinite(out.float()).all()

@@ -13,7 +13,7 @@ constexpr int kMaxRanks = 384;
 constexpr int kMaxTopk = 16;
 constexpr int kMaxListExperts = 64;  // per-expert weight tensors that fit in the kernel arguments
 // GEMM schedule (device-built, one per GEMM launch): kSchedHeader ints, then the work items.
-//   [0] item count  [1] total rows  [2] queues in use  [3] 0
+//   [0] item count  [1] total rows  [2] queues in use  [3] 1 when no queue holds more than one item
 //   [kSchedQueueStart + w]     first item of the queue of workgroup w (w = 0 .. kMaxQueues; the last entry is
 //                              the end of the last queue)
 //   [kSchedQueueCount + 32 w]  items already handed out from queue w (set to 1 by the builder: the first item is

@@ -647,6 +647,9 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_kernel(GemmArgs a)
     auto steal = [&]() -> int {  // all lanes of wave 0; the result is valid in every lane
         const int lane = tid & (kWave - 1);
         const int nq = min(sched[2], kMaxQueues);
+        if (sched[3] != 0) {  // every queue's only item is its workgroup's own: there is nothing to take over
+            return -1;
+        }
         for (int attempt = 0; attempt < 4; ++attempt) {
             int best = -1;  // (items left, same XCD, queue) packed so that the maximum is the choice
             for (int v = lane; v < nq; v += kWave) {

@@ -248,11 +248,11 @@ __device__ __forceinline__ void build_sched_part(SchedShared &sh, const SchedBui
         sched[0] = min(n_items, spec.max_items);
         sched[1] = sh.total_rows;
         sched[2] = m;
-        sched[3] = 0;
+        sched[3] = R + (b > 0 ? 1 : 0) <= 1 ? 1 : 0;  // no queue holds a second item: nothing can be taken over
     }
-    for (int w = tid; w <= kMaxQueues; w += NT) {
+    for (int w = tid; w <= m; w += NT) {  // the launch has m workgroups: the entries beyond are never read
         sched[kSchedQueueStart + w] = min(sh.qstart[w], spec.max_items);
-        if (w < kMaxQueues) {
+        if (w < m) {
             // the first item of a queue belongs to its workgroup without asking; the counter starts behind it
             sched[kSchedQueueCount + w * kSchedQueueStride] = 1;
         }
