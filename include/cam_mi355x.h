@@ -166,7 +166,9 @@ CAM_API camStatus camMoeDispatchPlan(void *workspace, uint64_t workspaceSize, ca
  * device image; every GPU the library runs on holds its own copy until the process ends.  Limit: at most
  * 131072 (token, k) entries (T*K); more returns CAM_ERR_RANGE.  Every call on a GPU uses that GPU's one
  * array, so calls that overlap on one GPU (two streams, two threads) race; calls on one stream do not.
- * Nothing in the array has to start at zero.  The call must be made with the target device current. */
+ * Nothing in the array has to start at zero.  The call must be made with the target device current.  The first
+ * call on a device looks up the array's address in the library's device image (hipGetSymbolAddress): make it
+ * once outside any stream capture; every later call on that device only enqueues kernels and may be captured. */
 CAM_API camStatus camMoeDispatchPlanNoAlloc(const camTensor *topkIdx, int64_t numExperts, int64_t numRanks,
                                             int64_t rankId, const camTensor *sendTokenIdx,
                                             const camTensor *numTokensPerExpert, const camTensor *sendOffset,

@@ -598,11 +598,18 @@ camStatus camMoeDispatchPlanNoAlloc(const camTensor *topkIdx, int64_t numExperts
     CAM_TRY(validate_plan(topkIdx, numExperts, numRanks, rankId, sendTokenIdx, numTokensPerExpert, sendOffset,
                           recvOffset, recvCount, numRecvTokensPerExpert, totalRecvTokens, slotRowOptional, &p));
     const int64_t entries = (int64_t)p.T * p.K;
-    if (entries > kNoAllocMaxEntries || cam::plan_workspace_bytes(p.T, p.K, p.E) > kNoAllocScratchBytes) {
+    if (entries > kNoAllocMaxEntries) {
         return fail(CAM_ERR_RANGE,
                     "MoeDispatchPlanNoAlloc: %lld (token, k) entries exceed the %lld the built-in scratch holds; "
                     "use MoeDispatchPlan with a workspace",
                     (long long)entries, (long long)kNoAllocMaxEntries);
+    }
+    const uint64_t need = cam::plan_workspace_bytes(p.T, p.K, p.E);
+    if (need > kNoAllocScratchBytes) {  // cannot happen within the entry limit; guards a change of the plan's chunking
+        return fail(CAM_ERR_RANGE,
+                    "MoeDispatchPlanNoAlloc: the plan needs %llu bytes of scratch, the built-in array holds %llu; "
+                    "use MoeDispatchPlan with a workspace",
+                    (unsigned long long)need, (unsigned long long)kNoAllocScratchBytes);
     }
     void *ptr = nullptr;
     hipError_t e = scratch_on_current_device(&ptr);
