@@ -19,6 +19,7 @@ import os
 import sys
 import time
 
+import numpy as np
 import torch
 
 ROOT = os.path.dirname(os.path.abspath(__file__))
@@ -93,7 +94,8 @@ def main():
     ap.add_argument("--skip-cpu", action="store_true")
     ap.add_argument("--layers", default="", help="comma list of substrings: only the fused layers whose name holds one of them")
     ap.add_argument("--only", default="", help="comma list of sections: step (the timed dispatch + combine step and its two kernels), "
-                         "dispatch / combine (those plus the other operator forms of each), gemm, layer, copy")
+                         "dispatch / combine (those plus the other operator forms of each), gemm, layer, copy; "
+                         "timeline (with gemm, on a clock-stamping build of the library: per-tile times)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build is single-GPU; every figure is measured on one MI355X. "
@@ -420,6 +422,45 @@ def main():
                                                                                    ops1 / s_u["mean"] / 1e12))
         except cam.CamError as ex:  # the slice lost its format tag
             log("uniform-expert GEMM skipped: %s" % ex)
+        if "timeline" in only:
+            # Per-tile device clock stamps (only in a library built with -DCAM_GEMM_TIMELINE and named by
+            # CAM_MI355X_LIB): how long each class of tile ran and when the workgroups of each XCD went idle.
+            tl, head_words, item_words, sched_at = _lib.gemm_timeline_info()
+            if not tl:
+                log("timeline: this library has no clock stamps; build one with `python -m umdk_original_amd.build "
+                    "--timeline` and run with CAM_MI355X_LIB=umdk_original_amd/lib/libcam_mi355x_timeline.so")
+            else:
+                for opname, fn, ws in (("GroupedMatmulSwigluQuant", gmm1, ws1), ("GroupedMatmulDequant", gmm2, ws2)):
+                    for j in range(PG + 1):
+                        fn(j)
+                    torch.cuda.synchronize()
+                    words = ws[sched_at:].view(torch.int32)
+                    n_items, n_q = int(words[0]), int(words[2])
+                    rec = words[head_words:head_words + n_items * item_words].cpu().numpy().reshape(n_items, item_words)
+                    t0 = rec[:, 6].astype(np.int64).min()
+                    beg = (rec[:, 6].astype(np.int64) - t0) / 100.0
+                    end = (rec[:, 7].astype(np.int64) - t0) / 100.0
+                    wg = (rec[:, 3].astype(np.int64) & 0xffffffff) >> 16
+                    cls = np.where(rec[:, 5] != 0, 0, (rec[:, 2] + 31) // 32)
+                    log("timeline of %s: %d tiles on %d workgroups, first begin to last end %.1f us" %
+                        (opname, n_items, n_q, end.max()))
+                    table = {}
+                    for c in sorted(set(cls.tolist())):
+                        d = (end - beg)[cls == c]
+                        table["flat" if c == 0 else "tall_%d_units" % c] = dict(tiles=int(d.size), mean_us=float(d.mean()),
+                                                                               max_us=float(d.max()))
+                        log("  %-14s %4d tiles  mean %6.1f us  max %6.1f us" %
+                            ("flat" if c == 0 else "tall, %d units" % c, d.size, d.mean(), d.max()))
+                    fin = np.zeros(n_q)
+                    busy = np.zeros(n_q)
+                    np.maximum.at(fin, wg, end)
+                    np.add.at(busy, wg, end - beg)
+                    per_xcd = [float(fin[x::8].max()) for x in range(8)]
+                    log("  workgroups go idle between %.1f and %.1f us; mean busy %.1f us; last end per XCD: %s" %
+                        (fin.min(), fin.max(), busy.mean(), " ".join("%.0f" % v for v in per_xcd)))
+                    result.setdefault("gemm_timeline", {})[opname] = dict(
+                        span_us=float(end.max()), tiles=table, mean_busy_us=float(busy.mean()),
+                        last_end_per_xcd_us=per_xcd)
         del gsets, ws1, ws2
         torch.cuda.empty_cache()
         # Calibration only, never a product path: what the vendor's dense int8 GEMM (hipBLASLt behind
@@ -549,7 +590,6 @@ def main():
     if not args.skip_cpu and want("step"):
         sys.path.insert(0, os.path.join(ROOT, "oracle"))
         import cam_oracle
-        import numpy as np
         ids_np = ids64.numpy()
         x_np = synth.bf16_bits(synth.normal_bf16(T, H, seed=44))
         y_np = synth.bf16_bits(synth.normal_bf16(A, H, seed=46))

@@ -427,6 +427,9 @@ def test_fp8_operator_validation():
     a = list(fused)
     a[8] = 513
     assert _lib.phase1("FusedDeepMoeFp8", a)[0] == CAM_ERR_RANGE
+    a = list(fused)
+    a[0] = _t((T, H), torch.float16)                   # the block-scaled layer takes bf16 activations only
+    assert _lib.phase1("FusedDeepMoeFp8", a)[0] == CAM_ERR_DTYPE
     # quantMode 4 of MoeDispatchPrefill: FP8 rows with uint8 block scales
     pre = _prefill_args()
     pre[5] = 4

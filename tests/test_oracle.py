@@ -420,7 +420,8 @@ def test_gmm1_epilogue_halves_scale_order_and_grouping(oracle):
     assert not np.array_equal(t_other[:, I:].view(np.uint32), t32[:, I:].view(np.uint32))
     # left half is SiLU of the dequantised value
     t64 = t32[:, :I].astype(np.float64)
-    assert np.allclose(d[:, :I], t64 / (1 + np.exp(-t64)), rtol=1e-6, atol=1e-30)
+    # (the specified SiLU is within 1.2e-5 relative of the exact one over this range; its own tests pin that)
+    assert np.allclose(d[:, :I], t64 / (1 + np.exp(-t64)), rtol=1.5e-5, atol=1e-30)
     assert not np.allclose(d[:, :I], t32[:, :I])  # and not the identity
 
 

@@ -14,7 +14,9 @@ import os
 import torch
 
 _PKG = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_PKG, "lib", "libcam_mi355x.so")
+# CAM_MI355X_LIB names another build of the same library (the clock-stamping profiling build); the default is the
+# product library beside this file.
+LIB_PATH = os.environ.get("CAM_MI355X_LIB") or os.path.join(_PKG, "lib", "libcam_mi355x.so")
 
 CAM_MAX_DIMS = 8
 
@@ -118,7 +120,7 @@ DIRECT_SIGNATURES = {
     "MoeDispatchPlanNoAlloc": [_TP, _I64, _I64, _I64, _TP, _TP, _TP, _TP, _TP, _TP, _TP, _TP],
 }
 
-EXPORTS = ["camGetRecentErrMsg", "camDestroyExecutor", "camGetVersion"] + [
+EXPORTS = ["camGetRecentErrMsg", "camDestroyExecutor", "camGetVersion", "camGemmTimelineInfo"] + [
     "cam%s" % op for op in DIRECT_SIGNATURES] + [
     "cam%s%s" % (op, suffix) for op in SIGNATURES for suffix in ("GetWorkspaceSize", "")
 ]
@@ -155,6 +157,16 @@ def lib():
 
 def recent_error():
     return lib().camGetRecentErrMsg().decode("utf-8", "replace")
+
+
+def gemm_timeline_info():
+    """camGemmTimelineInfo: (stamps compiled in, words before the first tile record, words per record, byte
+    offset of the schedule in a grouped-GEMM operator's workspace)."""
+    info = (ctypes.c_int32 * 4)()
+    st = lib().camGemmTimelineInfo(info)
+    if st != CAM_OK:
+        raise CamError(st, recent_error())
+    return tuple(int(v) for v in info)
 
 
 def as_cam_tensor(t, fmt=CAM_FORMAT_ND):

@@ -1,5 +1,9 @@
 """Builds libcam_mi355x.so (HIP kernels + C ABI) for gfx950 with hipcc, and libcam_torch_ops.so (the C++
-registration of torch.ops.umdk_cam_op_lib on top of that ABI) with the host compiler, both in-tree."""
+registration of torch.ops.umdk_cam_op_lib on top of that ABI) with the host compiler, both in-tree.
+
+`python -m umdk_original_amd.build --timeline` builds a second library beside them, libcam_mi355x_timeline.so:
+the same sources with -DCAM_GEMM_TIMELINE, whose grouped-GEMM kernel stamps every tile of its schedule with
+the device clock.  It is a profiling aid and is only loaded when CAM_MI355X_LIB names it."""
 import os
 import subprocess
 import sys
@@ -8,6 +12,7 @@ _PKG = os.path.dirname(os.path.abspath(__file__))
 _CSRC = os.path.join(_PKG, "csrc")
 LIB_DIR = os.path.join(_PKG, "lib")
 LIB_PATH = os.path.join(LIB_DIR, "libcam_mi355x.so")
+TIMELINE_LIB_PATH = os.path.join(LIB_DIR, "libcam_mi355x_timeline.so")
 SOURCES = ["abi.cpp", "plan.hip", "dispatch.hip", "combine.hip", "gemm.hip"]
 
 # -packed-fp32-ops is switched off on purpose: packed fp32 VALU forms are not used by this library.
@@ -21,15 +26,16 @@ HIPCC_FLAGS = [
 ]
 
 
-def build(verbose=False):
+def build(verbose=False, timeline=False):
     """Compile every source and link the shared library. Always recompiles."""
     os.makedirs(LIB_DIR, exist_ok=True)
     hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
     objs = []
     procs = []
+    extra = ["-DCAM_GEMM_TIMELINE"] if timeline else []
     for src in SOURCES:
-        obj = os.path.join(LIB_DIR, os.path.splitext(src)[0] + ".o")
-        cmd = [hipcc] + HIPCC_FLAGS + ["-x", "hip", "-c", os.path.join(_CSRC, src), "-o", obj]
+        obj = os.path.join(LIB_DIR, os.path.splitext(src)[0] + (".timeline.o" if timeline else ".o"))
+        cmd = [hipcc] + HIPCC_FLAGS + extra + ["-x", "hip", "-c", os.path.join(_CSRC, src), "-o", obj]
         if verbose:
             print(" ".join(cmd), flush=True)
         procs.append((src, subprocess.Popen(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)))
@@ -41,12 +47,14 @@ def build(verbose=False):
             raise RuntimeError("hipcc failed on %s:\n%s" % (src, out))
         if verbose and out.strip():
             print(out)
-    cmd = [hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB_PATH] + objs
+    out_path = TIMELINE_LIB_PATH if timeline else LIB_PATH
+    cmd = [hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", out_path] + objs
     subprocess.check_call(cmd)
     for o in objs:
         os.remove(o)
-    build_torch_ops(verbose)
-    return LIB_PATH
+    if not timeline:
+        build_torch_ops(verbose)
+    return out_path
 
 
 TORCH_OPS_PATH = os.path.join(LIB_DIR, "libcam_torch_ops.so")
@@ -75,4 +83,4 @@ def build_torch_ops(verbose=False):
 
 
 if __name__ == "__main__":
-    print(build(verbose="-v" in sys.argv))
+    print(build(verbose="-v" in sys.argv, timeline="--timeline" in sys.argv))

@@ -308,6 +308,22 @@ const char *camGetRecentErrMsg(void) { return g_err.c_str(); }
 
 const char *camGetVersion(void) { return "cam-mi355x 0.1 (gfx950)"; }
 
+camStatus camGemmTimelineInfo(int32_t info[4])
+{
+    if (info == nullptr) {
+        return fail(CAM_ERR_NULL, "info is NULL");
+    }
+#ifdef CAM_GEMM_TIMELINE
+    info[0] = 1;
+#else
+    info[0] = 0;
+#endif
+    info[1] = cam::kSchedHeader;
+    info[2] = (int32_t)(sizeof(cam::SchedItem) / sizeof(int32_t));
+    info[3] = 0;  // every camGroupedMatmul* phase 1 carves its schedule first
+    return CAM_OK;
+}
+
 camStatus camDestroyExecutor(camOpExecutor *executor)
 {
     delete executor;
@@ -2089,7 +2105,7 @@ camStatus camFusedDeepMoeFp8GetWorkspaceSize(const camTensor *x, const camTensor
                                              const camTensor *expertTokenNums, uint64_t *workspaceSize,
                                              camOpExecutor **executor)
 {
-    CAM_TRY(check_tensor(x, "x", 2, CAM_DT_BF16, CAM_DT_FLOAT16));
+    CAM_TRY(check_tensor(x, "x", 2, CAM_DT_BF16));  // the block-scaled layer is specified for bf16 activations only
     CAM_TRY(check_tensor(expertIds, "expertIds", 2, CAM_DT_INT32));
     CAM_TRY(check_tensor(expertScales, "expertScales", 2, CAM_DT_FLOAT));
     if (moeExpertNum <= 0 || moeExpertNum > cam::kMaxExperts) {
@@ -2153,7 +2169,7 @@ camStatus camFusedDeepMoeFp8GetWorkspaceSize(const camTensor *x, const camTensor
     const uint64_t o_x2s = c.take((uint64_t)A * (I / 128));
 
     const uint16_t *xp = (const uint16_t *)x->data;
-    const int x_is_fp16 = x->dtype == CAM_DT_FLOAT16;
+    const int x_is_fp16 = 0;
     const int32_t *ids = (const int32_t *)expertIds->data;
     const float *gates = (const float *)expertScales->data;
     const uint8_t *mask = xActiveMaskOptional ? (const uint8_t *)xActiveMaskOptional->data : nullptr;

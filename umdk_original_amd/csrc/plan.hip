@@ -45,8 +45,9 @@ __global__ __launch_bounds__(kLocalThreads) void plan_local_kernel(PlanArgs a, i
 
 // Phase 2.  Every workgroup sums the histogram columns (all rows for the per-expert count, the rows
 // before its own for its base), scans the counts into offsets, and finishes its own chunk:
-// pos += base[e], dst_row = off[e] + pos.  Workgroup 0 also writes the per-expert outputs and the
-
+// pos += base[e], dst_row = off[e] + pos.  Workgroup 0 also writes the per-expert outputs (counts, offsets,
+// cumulative group list, receive bookkeeping), the total row count, the zeroed per-rank counters and the
+// four words of the receive metadata.
 template <typename IdT>
 __global__ __launch_bounds__(kGlobalThreads) void plan_global_kernel(PlanArgs a, int chunk, const int32_t *hist_in)
 {
