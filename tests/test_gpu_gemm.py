@@ -257,3 +257,26 @@ def test_many_flat_items_per_workgroup_bit_exact(gpu, oracle, Kd, N, gate_up):
         xs = synth.channel_scales((max(A, 1),), seed=42, lo=0.001, hi=0.01)
         out = cam.grouped_matmul_dequant(a.to(gpu), xs.to(gpu), wp, ws.to(gpu), gl.to(gpu))
         assert_bits_equal(to_np(out)[:A], oracle.gmm2_epilogue(want, ws.numpy(), xs.numpy(), gl.numpy())[:A], "bf16 output")
+
+
+def test_long_schedule_shared_queues_bit_exact(gpu, oracle):
+    """A schedule of more than eight items per workgroup (tall experts of 2-6 row tiles with flat and empty ones
+    in between): the builder then deals the items to one shared queue per XCD, flat items spread among the tall
+    ones, and every workgroup asks for every item.  Every accumulator is checked."""
+    rng = np.random.default_rng(77)
+    sizes = []
+    for _ in range(150):
+        sizes.append(int(rng.integers(300, 1500)))
+        if rng.random() < 0.3:
+            sizes.append(int(rng.integers(0, 129)))
+    Kd, N = 128, 1024
+    items = sum(((s + 255) // 256) * (N // 256) if s > 128 else ((N + 511) // 512 if s > 0 else 0) for s in sizes)
+    cus = torch.cuda.get_device_properties(gpu).multi_processor_count
+    announce("gemm long schedule: %d experts, %d rows, %d items on %d workgroups" % (len(sizes), sum(sizes), items, cus))
+    if items < 8 * cus:
+        pytest.skip("this device has too many CUs for the shape to reach the shared-queue form")
+    a, w, gl, A = _inputs(sizes, Kd, N, seed=177)
+    wp = cam.prepack_weight(w.to(gpu), False)
+    got = cam.grouped_matmul_int32(a.to(gpu), wp, gl.to(gpu))
+    want = oracle.gmm_int32(a.numpy(), w.numpy(), gl.numpy())
+    assert_bits_equal(to_np(got)[:A], want[:A], "int32 accumulators")

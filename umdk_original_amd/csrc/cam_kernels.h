@@ -13,12 +13,14 @@ constexpr int kMaxRanks = 384;
 constexpr int kMaxTopk = 16;
 constexpr int kMaxListExperts = 64;  // per-expert weight tensors that fit in the kernel arguments
 // GEMM schedule (device-built, one per GEMM launch): kSchedHeader ints, then the work items.
-//   [0] item count  [1] total rows  [2] queues in use  [3] 1 when no queue holds more than one item
-//   [kSchedQueueStart + w]     first item of the queue of workgroup w (w = 0 .. kMaxQueues; the last entry is
-//                              the end of the last queue)
-//   [kSchedQueueCount + 32 w]  items already handed out from queue w (set to 1 by the builder: the first item is
-//                              its workgroup's without asking; advanced by the GEMM); one counter per 128-byte
-//                              line, so that the queues do not share a line
+//   [0] item count  [1] total rows  [2] queues in use
+//   [3] bit 0: no queue holds more than one item; bit 1: one queue per XCD, shared by its workgroups, instead
+//       of one queue per workgroup
+//   [kSchedQueueStart + w]     first item of queue w (w = 0 .. queues in use; the last entry is the end of the
+//                              last queue)
+//   [kSchedQueueCount + 32 w]  items already handed out from queue w (a workgroup's own queue starts at 1: the
+//                              first item is its workgroup's without asking; a shared queue at 0; advanced by
+//                              the GEMM); one counter per 128-byte line, so that the queues do not share a line
 constexpr int kNumXcd = 8;       // workgroup i of a launch runs on XCD i % 8
 constexpr int kMaxQueues = 512;  // one queue per workgroup of the persistent GEMM (one workgroup per CU)
 constexpr int kSchedQueueStart = 4;

@@ -628,15 +628,17 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_kernel(GemmArgs a)
     const int32_t *qstart = sched + kSchedQueueStart;
     int32_t *qcount = sched + kSchedQueueCount;
     const SchedItem *items = (const SchedItem *)(sched + kSchedHeader);
-    const int me = (int)blockIdx.x;            // this workgroup's queue
+    const bool shared = (sched[3] & 2) != 0;   // long schedules: one queue per XCD, every item asked for
+    const int me = shared ? (int)blockIdx.x % max(min(sched[2], kMaxQueues), 1) : (int)blockIdx.x;  // this workgroup's queue
     const int q0 = qstart[min(me, kMaxQueues)];
     const int qlen = me < kMaxQueues ? qstart[me + 1] - q0 : 0;
-    bool own_empty = qlen <= 1;                // the first item needs no asking; there may be nothing after it
+    bool own_empty = qlen <= (shared ? 0 : 1);  // an own queue's first item needs no asking; there may be nothing after it
 
-    // Work items.  Every workgroup has a queue of its own, built to last as long as the others (sched_device.h).
-    // Its first item is its own without asking; for the following ones it advances its queue's counter with a
-    // device-scope atomic, a round trip to the memory side that is issued at the START of an item and looked at
-    // only when the item is done (take_begin / take_end).  Every counter has a cache line of its own.  A
+    // Work items.  Short schedules: every workgroup has a queue of its own, built to last as long as the others
+    // (sched_device.h).  Its first item is its own without asking; for the following ones it advances its queue's
+    // counter with a device-scope atomic, a round trip to the memory side that is issued at the START of an item
+    // and looked at only when the item is done (take_begin / take_end).  Long schedules: the workgroups of an XCD
+    // share one queue and ask for every item, the first included.  Every counter has a cache line of its own.  A
     // workgroup whose queue has run out helps the queue with the most items left (its own XCD's first, so that
     // what it fetches is likely to be in its L2): wave 0 looks at every counter at once, one round trip, and its
     // first lane then advances the chosen one.  A counter only ever grows and every queue is finite, so every
@@ -647,7 +649,7 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_kernel(GemmArgs a)
     auto steal = [&]() -> int {  // all lanes of wave 0; the result is valid in every lane
         const int lane = tid & (kWave - 1);
         const int nq = min(sched[2], kMaxQueues);
-        if (sched[3] != 0) {  // every queue's only item is its workgroup's own: there is nothing to take over
+        if ((sched[3] & 1) != 0) {  // every queue's only item is its workgroup's own: there is nothing to take over
             return -1;
         }
         for (int attempt = 0; attempt < 4; ++attempt) {
@@ -696,7 +698,15 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_kernel(GemmArgs a)
 
     int next = -1;
     if (tid < kWave) {
-        next = qlen > 0 ? q0 : steal();
+        if (shared) {
+            int taken = 0;
+            if (tid == 0) {
+                taken = take_begin();
+            }
+            next = take_end(taken);
+        } else {
+            next = qlen > 0 ? q0 : steal();
+        }
     }
     for (;;) {
         if (tid == 0) {
