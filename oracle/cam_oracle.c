@@ -12,12 +12,15 @@
  * Parity status.  Integer functions (layout, offsets, ranks, receive bookkeeping, int32 GEMM) and the
  * dispatch quantisation are pinned by closed forms and brute-force definitions in tests/test_oracle.py.
  * The reference ships no golden vectors for this path, and its kernels cannot be built without the
- * Ascend toolkit, so no function here is checked against reference *outputs*.  Two functions rest on
+ * Ascend toolkit, so no function here is checked against reference *outputs*.  These functions rest on
  * a deliberate definition the reference does not give portably and are therefore "parity unpinned"
  * against the Ascend hardware bit-for-bit:
- *   - cam_oracle_gmm1_epilogue: SiLU uses cam_expf_spec() in place of the Ascend Exp instruction;
+ *   - cam_oracle_gmm1_epilogue: SiLU is cam_silu_spec() (a fixed sequence of 19 rounded operations, within
+ *     1.2e-5 relative of the exact function) in place of the Ascend Exp and Div instructions;
  *   - everything downstream of it (cam_oracle_swiglu_quant's int8 values, the bf16 layer output)
- *     inherits that; the reference's own acceptance bound there is atol 2.0 / rtol 0.02.
+ *     inherits that; the reference's own acceptance bound there is atol 2.0 / rtol 0.02;
+ *   - cam_oracle_comm_quant_rows and cam_oracle_dispatch_shmem take the Ascend Div to be the IEEE quotient
+ *     and every written operation to round once.
  * All-zero rows (division by zero in the reference, AK/.../grouped_matmul_slice_m_per_token_dequant_
  * swiglu_quant_multistage_workspace.h:804 and :252-255) are defined here as q = 0, scale = 0.
  */
