@@ -52,7 +52,7 @@ constexpr float kTallUnitStep = 92.0f;
 constexpr float kFlatFixed = 22400.0f;
 constexpr float kFlatStep = 862.0f;
 constexpr int kClasses = 9;  // item kinds: 0 = flat, h = 1..8 = tall tile of h row units
-constexpr int kSharedFrom = 8;                        // items per workgroup from which the queues are shared
+constexpr int kSharedFrom = 12;                       // items per workgroup from which the queues are shared
 constexpr int kTallTail = 24;                        // tall items a shared queue ends with
 
 struct ExpertShape {
