@@ -146,7 +146,7 @@ def test_moe_dispatch_prefill_validation():
     for i in (10, 11, 12, 13, 14, 15):  # every optional output may be absent
         a[i] = None
     assert _lib.phase1("MoeDispatchPrefill", a)[0] == CAM_OK
-    # more (token, k) entries than the single launch is built for still validates (two-launch fallback)
+    # a long id sequence (many ranking chunks) validates like a short one
     assert _lib.phase1("MoeDispatchPrefill", _prefill_args(T=40000, K=16, E=32))[0] == CAM_OK
 
 

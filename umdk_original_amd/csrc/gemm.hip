@@ -10,11 +10,12 @@
 //
 // Design (not a translation of the cube/vector split above).
 //   * Persistent kernel, one workgroup of 8 waves per CU.  Work items (one row tile of ONE expert x one
-//     block of packed weight columns) come from eight device-built queues, one per XCD; a workgroup
-//     takes items from the queue of the XCD it runs on and helps the other queues when its own is empty.
-//     The row tiles of an expert that read the same weight columns sit next to each other in one queue,
-//     so the CUs working on them share one L2, and the queues list big experts first, which leaves the
-//     small items for the end, where they even out the finishing times.
+//     block of packed weight columns) come from a device-built schedule (sched_device.h).  Short schedules
+//     give every workgroup a queue of its own, dealt so that the queues last equally long and that the
+//     workgroups of an XCD work on tiles which share operands; a workgroup whose queue runs out takes from
+//     the fullest one.  Long schedules use one queue per XCD, shared by its workgroups, in which the row
+//     tiles of an expert that read the same weight columns sit next to each other and big experts come
+//     first, which leaves the small items for the end, where they even out the finishing times.
 //   * Two tile shapes.  Tall tiles (129..256 rows) x 256 columns: the two teams of four waves split the
 //     rows, every wave owns 64 columns.  Flat tiles (<= 128 rows) x 512 columns: the teams split the
 //     columns, so that the weights, which is all such an expert streams from HBM, feed every wave and
