@@ -442,7 +442,7 @@ def main():
                     end = (rec[:, 7].astype(np.int64) - t0) / 100.0
                     wg = (rec[:, 3].astype(np.int64) & 0xffffffff) >> 16
                     cls = np.where(rec[:, 5] != 0, 0, (rec[:, 2] + 31) // 32)
-                    log("timeline of %s: %d tiles on %d workgroups, first begin to last end %.1f us" %
+                    log("timeline of %s: %d tiles in %d queues, first begin to last end %.1f us" %
                         (opname, n_items, n_q, end.max()))
                     table = {}
                     for c in sorted(set(cls.tolist())):
@@ -451,8 +451,9 @@ def main():
                                                                                max_us=float(d.max()))
                         log("  %-14s %4d tiles  mean %6.1f us  max %6.1f us" %
                             ("flat" if c == 0 else "tall, %d units" % c, d.size, d.mean(), d.max()))
-                    fin = np.zeros(n_q)
-                    busy = np.zeros(n_q)
+                    n_wg = int(wg.max()) + 1  # (a long schedule has eight shared queues, not one per workgroup)
+                    fin = np.zeros(n_wg)
+                    busy = np.zeros(n_wg)
                     np.maximum.at(fin, wg, end)
                     np.add.at(busy, wg, end - beg)
                     per_xcd = [float(fin[x::8].max()) for x in range(8)]
