@@ -95,7 +95,8 @@ def main():
     ap.add_argument("--layers", default="", help="comma list of substrings: only the fused layers whose name holds one of them")
     ap.add_argument("--only", default="", help="comma list of sections: step (the timed dispatch + combine step and its two kernels), "
                          "dispatch / combine (those plus the other operator forms of each), gemm, layer, copy; "
-                         "timeline (with gemm, on a clock-stamping build of the library: per-tile times)")
+                         "timeline (with gemm, on a clock-stamping build of the library: per-tile times); "
+                         "calib (micro-benchmarks of the part's ceilings from libcam_calib.so)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build is single-GPU; every figure is measured on one MI355X. "
@@ -128,6 +129,44 @@ def main():
 
     result = {}
     kernels = {}
+
+    # ------------------------------------------------------------------ ceilings of the part (on request)
+    if "calib" in only:
+        # Micro-benchmarks from libcam_calib.so (csrc/calib.hip; not part of the product library): what the matrix
+        # cores, scattered row stores and streaming reads reach on this box, and the dispatch in destination order.
+        import ctypes
+        from umdk_original_amd import build as cam_build
+        clib = ctypes.CDLL(cam_build.CALIB_LIB_PATH)
+        dbl4 = ctypes.c_double * 4
+
+        def calib(fn, *args):
+            out = dbl4()
+            rc = getattr(clib, fn)(*args, out)
+            assert rc == 0, "%s failed with HIP error %d" % (fn, rc)
+            return [float(v) for v in out]
+
+        m0 = calib("camCalibMfmaInt8", 0)
+        m1 = calib("camCalibMfmaInt8", 1)
+        m2 = calib("camCalibMfmaInt8", 2)
+        log("calib: v_mfma_i32_32x32x32_i8 alone %.2f POP/s at %.2f GHz; with LDS fragment reads of the same bytes "
+            "%.2f POP/s at %.2f GHz; of changing random bytes %.2f POP/s at %.2f GHz"
+            % (m0[0], m0[1], m1[0], m1[1], m2[0], m2[1]))
+        s_nt = calib("camCalibRowStores", 1)
+        s_pl = calib("camCalibRowStores", 0)
+        log("calib: 32768 rows of 7168 B stored to scattered row slots %.2f TB/s (plain stores %.2f), to consecutive "
+            "slots %.2f TB/s (plain %.2f)" % (s_nt[0], s_pl[0], s_nt[1], s_pl[1]))
+        rd = calib("camCalibStreamRead")
+        log("calib: streaming read of 1.5 GiB %.2f TB/s with plain loads, %.2f TB/s non-temporal" % (rd[0], rd[1]))
+        do = calib("camCalibDestinationOrder")
+        log("calib: dispatch in destination order (4096 x 7168, top-8): one pass %.1f us; token-major quantisation "
+            "%.1f us + row copy %.1f us = %.1f us back to back" % (do[0], do[1], do[2], do[3]))
+        result["calibration"] = dict(
+            mfma_int8_alone=dict(pops=m0[0], ghz=m0[1]), mfma_int8_with_lds_reads=dict(pops=m1[0], ghz=m1[1]),
+            mfma_int8_with_random_operands=dict(pops=m2[0], ghz=m2[1]),
+            row_stores_tb_per_s=dict(scattered_nt=s_nt[0], scattered_plain=s_pl[0], linear_nt=s_nt[1],
+                                     linear_plain=s_pl[1]),
+            stream_read_tb_per_s=dict(plain=rd[0], non_temporal=rd[1]),
+            destination_order_us=dict(one_pass=do[0], quantise_tokens=do[1], row_copy=do[2], two_passes=do[3]))
 
     # ------------------------------------------------------------------ counter calibration (on request)
     if "copy" in only:

@@ -29,6 +29,13 @@ def test_library_exports_every_declared_symbol():
     assert sorted(_lib.EXPORTS) == names
 
 
+def test_calibration_library_loads_and_exports_its_entry_points():
+    from umdk_original_amd import build
+    handle = ctypes.CDLL(build.CALIB_LIB_PATH)
+    for n in ("camCalibMfmaInt8", "camCalibRowStores", "camCalibStreamRead", "camCalibDestinationOrder"):
+        assert hasattr(handle, n), n
+
+
 def test_version_and_error_string():
     assert b"gfx950" in _lib.lib().camGetVersion()
     st, _, msg = _lib.phase1("DispatchLayout", [None, 1, 1, 1, 1, None, None, None])
