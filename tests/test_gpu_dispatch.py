@@ -298,3 +298,14 @@ def test_dispatch_fp16_activations(gpu, oracle, quant_mode):
     assert torch.equal(assist[:3 * total], d["expand_idx"][:3 * total])
     if quant_mode:
         assert torch.equal(scales[:total], d["recv_x_scales"][:total])
+
+
+def test_plain_c_caller_runs_layout_and_notify(gpu):
+    """The C ABI called from a program in plain C (csrc/abi_consumer.c; no torch, no C++): DispatchLayout and
+    NotifyDispatch on device memory from hipMalloc, compared with loops on the host."""
+    import subprocess
+    from umdk_original_amd import build
+    announce("plain C caller of the ABI")
+    p = subprocess.run([build.ABI_CONSUMER_PATH, "run"], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True,
+                       timeout=120)
+    assert p.returncode == 0 and "run ok" in p.stdout, p.stdout

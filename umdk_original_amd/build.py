@@ -15,6 +15,7 @@ LIB_DIR = os.path.join(_PKG, "lib")
 LIB_PATH = os.path.join(LIB_DIR, "libcam_mi355x.so")
 TIMELINE_LIB_PATH = os.path.join(LIB_DIR, "libcam_mi355x_timeline.so")
 CALIB_LIB_PATH = os.path.join(LIB_DIR, "libcam_calib.so")  # calibration micro-benchmarks, loaded by bench.py only
+ABI_CONSUMER_PATH = os.path.join(LIB_DIR, "abi_consumer")  # plain-C caller of the ABI (csrc/abi_consumer.c), for tests
 SOURCES = ["abi.cpp", "plan.hip", "dispatch.hip", "combine.hip", "gemm.hip"]
 
 # -packed-fp32-ops is switched off on purpose: packed fp32 VALU forms are not used by this library.
@@ -56,8 +57,25 @@ def build(verbose=False, timeline=False):
         os.remove(o)
     if not timeline:
         build_calib(verbose)
+        build_abi_consumer(verbose)
         build_torch_ops(verbose)
     return out_path
+
+
+def build_abi_consumer(verbose=False):
+    """csrc/abi_consumer.c, compiled as C by the host compiler: the header has to be a C header, and the library has
+    to be usable with nothing but the HIP runtime beside it."""
+    cc = os.environ.get("CC", "gcc")
+    cmd = [cc, "-std=c11", "-O1", "-Wall", "-Wextra", "-Werror", "-I", "/opt/rocm/include",
+           os.path.join(_CSRC, "abi_consumer.c"), "-o", ABI_CONSUMER_PATH,
+           "-L", LIB_DIR, "-lcam_mi355x", "-L", "/opt/rocm/lib", "-lamdhip64",
+           "-Wl,-rpath,$ORIGIN", "-Wl,-rpath,/opt/rocm/lib"]
+    if verbose:
+        print(" ".join(cmd), flush=True)
+    p = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    if p.returncode != 0:
+        raise RuntimeError("building %s failed:\n%s" % (ABI_CONSUMER_PATH, p.stdout))
+    return ABI_CONSUMER_PATH
 
 
 def build_calib(verbose=False):
