@@ -425,7 +425,9 @@ __device__ __forceinline__ void run_item(const GemmArgs &a, const ItemCtx &t, in
                 const v4u v = *(const v4u *)(slice + row * kEpiRowBytes + piece * 16);
                 const int trow = mf * 32 + row;
                 if (trow < t.my_rows) {
-                    *(v4u *)(dst + (long long)(t.m0 + t.a_row0 + trow) * row_pitch_bytes + piece * 16) = v;
+                    // the next kernel reads these rows once; stored non-temporally they do not push weight panels
+                    // and activation tiles out of the L2 (C3 both operators 519 -> 506 us, decode layer 427 -> 420 us)
+                    __builtin_nontemporal_store(v, (v4u *)(dst + (long long)(t.m0 + t.a_row0 + trow) * row_pitch_bytes + piece * 16));
                 }
             }
         };
