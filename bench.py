@@ -480,7 +480,11 @@ def main():
                     beg = (rec[:, 6].astype(np.int64) - t0) / 100.0
                     end = (rec[:, 7].astype(np.int64) - t0) / 100.0
                     wg = (rec[:, 3].astype(np.int64) & 0xffffffff) >> 16
-                    cls = np.where(rec[:, 5] != 0, 0, (rec[:, 2] + 31) // 32)
+                    flat_w = rec[:, 5].astype(np.int64) & 0xffffffff
+                    nb_w = rec[:, 4].astype(np.int64) & 0xffffffff
+                    to_first = (nb_w >> 16) / 100.0           # start of the tile -> its first multiply
+                    to_loop_end = ((flat_w >> 16) & 0x7fff) / 100.0  # start of the tile -> end of its K loop
+                    cls = np.where((flat_w & 0xffff) != 0, 0, (rec[:, 2] + 31) // 32)
                     log("timeline of %s: %d tiles in %d queues, first begin to last end %.1f us" %
                         (opname, n_items, n_q, end.max()))
                     table = {}
@@ -488,8 +492,14 @@ def main():
                         d = (end - beg)[cls == c]
                         table["flat" if c == 0 else "tall_%d_units" % c] = dict(tiles=int(d.size), mean_us=float(d.mean()),
                                                                                max_us=float(d.max()))
-                        log("  %-14s %4d tiles  mean %6.1f us  max %6.1f us" %
-                            ("flat" if c == 0 else "tall, %d units" % c, d.size, d.mean(), d.max()))
+                        sel = cls == c
+                        pro, loop = to_first[sel].mean(), (to_loop_end - to_first)[sel].mean()
+                        table["flat" if c == 0 else "tall_%d_units" % c].update(
+                            before_first_multiply_us=float(pro), k_loop_us=float(loop),
+                            after_k_loop_us=float(d.mean() - pro - loop))
+                        log("  %-14s %4d tiles  mean %6.1f us  max %6.1f us   (to the first multiply %.1f, K loop %.1f, "
+                            "epilogue and hand-over %.1f)" % ("flat" if c == 0 else "tall, %d units" % c, d.size, d.mean(),
+                                                              d.max(), pro, loop, d.mean() - pro - loop))
                     n_wg = int(wg.max()) + 1  # (a long schedule has eight shared queues, not one per workgroup)
                     fin = np.zeros(n_wg)
                     busy = np.zeros(n_wg)

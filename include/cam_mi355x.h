@@ -98,7 +98,8 @@ CAM_API const char *camGetVersion(void);
 
 /* Profiling aid with no counterpart in the reference.  A library built with -DCAM_GEMM_TIMELINE makes the
  * grouped-GEMM kernel stamp every tile of its schedule with the device's wall clock (100 MHz): begin and end in
- * words 6 and 7 of the tile's 8-word record, the workgroup that ran it in the upper 16 bits of word 3.  The
+ * words 6 and 7 of the tile's 8-word record, the workgroup that ran it in the upper 16 bits of word 3, and the ticks
+ * from its begin to its first multiply and to the end of its K loop in the upper 16 bits of words 4 and 5.  The
  * schedule is the first region of the workspace of every camGroupedMatmul* operator, so a caller that owns the
  * workspace can read the stamps back after a call.  info[0] = 1 when the stamps are compiled in (0 in a normal
  * build, whose kernel writes nothing to the schedule), info[1] = 32-bit words before the first tile record,

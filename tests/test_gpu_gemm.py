@@ -315,7 +315,7 @@ def test_schedule_covers_every_tile_exactly_once(gpu, name, sizes, N):
     nb_tall, nb_flat = (N + 255) // 256, (N + 511) // 512
     cover = {}
     for g, m0, rows, split, nb, flat, _, _ in rec.tolist():
-        split &= 0xffff  # a clock-stamping build keeps the workgroup in the upper half
+        split, nb, flat = split & 0xffff, nb & 0xffff, flat & 0xffff  # a clock-stamping build uses the upper halves
         assert 0 <= g < len(sizes) and sizes[g] > 0
         rel = m0 - int(first[g])
         if flat:
@@ -342,3 +342,16 @@ def test_schedule_covers_every_tile_exactly_once(gpu, name, sizes, N):
     shared = bool(flags & 2)
     assert n_queues == (8 if shared else cus)
     assert shared == (len(rec) // cus >= 12)
+
+
+def test_hardware_bf16_conversion_equals_the_definition_on_all_inputs(gpu):
+    """The GEMM and combine epilogues round fp32 to bf16 with the hardware's packed conversion; the oracle rounds by
+    the arithmetic definition (nearest even on the bit pattern, NaN -> truncated payload with the quiet bit).  The
+    calibration library compares the two over every one of the 2^32 bit patterns."""
+    import ctypes
+    from umdk_original_amd import build
+    announce("hardware bf16 conversion against its definition, all 2^32 patterns")
+    lib = ctypes.CDLL(build.CALIB_LIB_PATH)
+    out = (ctypes.c_double * 4)()
+    assert lib.camCalibBf16Conversion(out) == 0
+    assert out[0] == 0.0, "first differing pattern 0x%08x" % int(out[1])

@@ -280,6 +280,34 @@ __global__ __launch_bounds__(256) void dest_copy_kernel(const int8_t *q, const f
     }
 }
 
+// ---------------------------------------------------------------------------------------------------------------
+// fp32 -> bf16: the library's arithmetic definition (round to nearest even on the bit pattern, NaN -> truncated payload
+// with the quiet bit set) against the hardware conversion instruction, over every one of the 2^32 bit patterns.
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+
+__device__ __forceinline__ unsigned bf16_by_definition(unsigned u)
+{
+    const unsigned rounded = (u + 0x7fffu + ((u >> 16) & 1u)) >> 16;
+    const unsigned quiet = (u >> 16) | 0x0040u;
+    return ((u & 0x7fffffffu) > 0x7f800000u ? quiet : rounded) & 0xffffu;
+}
+
+__global__ __launch_bounds__(256) void bf16_check_kernel(unsigned long long *mismatches, unsigned *first)
+{
+    // thread i checks patterns 2i and 2i + 1 of this launch's quarter of the space
+    const unsigned long long i = ((unsigned long long)blockIdx.y << 31) + ((unsigned long long)blockIdx.x * 256 + threadIdx.x) * 2;
+    const unsigned u0 = (unsigned)i, u1 = (unsigned)i + 1u;
+    const f32x2 p = {__uint_as_float(u0), __uint_as_float(u1)};
+    const bf16x2 h = __builtin_convertvector(p, bf16x2);
+    const unsigned packed = __builtin_bit_cast(unsigned, h);
+    const unsigned want = bf16_by_definition(u0) | (bf16_by_definition(u1) << 16);
+    if (packed != want) {
+        atomicAdd(mismatches, 1ull);
+        atomicMin(first, (packed & 0xffffu) != (want & 0xffffu) ? u0 : u1);
+    }
+}
+
 }  // namespace
 
 #define CALIB_API extern "C" __attribute__((visibility("default")))
@@ -455,4 +483,28 @@ CALIB_API int camCalibDestinationOrder(double *out)
             hipLaunchKernelGGL(dest_copy_kernel, dim3(kA / 4), dim3(256), 0, 0, q, qs, dtor, o[i % rot], sc);
         },
         8, 40, &out[3]);
+}
+
+// out[0] = bit patterns (in pairs) on which the hardware fp32 -> bf16 conversion differs from the definition above,
+// out[1] = the smallest such pattern (as an unsigned value) or 2^32 - 1 when there is none.
+CALIB_API int camCalibBf16Conversion(double *out)
+{
+    Buffers b;
+    unsigned long long *mism;
+    unsigned *first;
+    CALIB_TRY(b.get((void **)&mism, 8));
+    CALIB_TRY(b.get((void **)&first, 4));
+    CALIB_TRY(hipMemset(mism, 0, 8));
+    CALIB_TRY(hipMemset(first, 0xff, 4));
+    // 2^32 patterns = 2 (grid y) x 2^31; a thread takes two: 2^30 threads per y = 2^22 workgroups of 256
+    hipLaunchKernelGGL(bf16_check_kernel, dim3(1u << 22, 2), dim3(256), 0, 0, mism, first);
+    CALIB_TRY(hipGetLastError());
+    CALIB_TRY(hipDeviceSynchronize());
+    unsigned long long hm = 0;
+    unsigned hf = 0;
+    CALIB_TRY(hipMemcpy(&hm, mism, 8, hipMemcpyDeviceToHost));
+    CALIB_TRY(hipMemcpy(&hf, first, 4, hipMemcpyDeviceToHost));
+    out[0] = (double)hm;
+    out[1] = (double)hf;
+    return 0;
 }

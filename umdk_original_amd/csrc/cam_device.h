@@ -32,6 +32,18 @@ __device__ __forceinline__ uint32_t f32_to_bf16_bits(float f)
     return (u & 0x7fffffffu) > 0x7f800000u ? quiet : rounded;  // both sides computed: a select, no branch
 }
 
+// Two fp32 values -> two bf16 bit patterns (lo in bits 0..15) with ONE hardware conversion instruction.  Its results
+// equal f32_to_bf16_bits on every one of the 2^32 inputs, NaNs included (checked exhaustively on the GPU by
+// camCalibBf16Conversion and tests/test_gpu_gemm.py); it takes one vector instruction where the arithmetic form
+// takes nine per value.
+typedef float cam_f32x2 __attribute__((ext_vector_type(2)));
+typedef __bf16 cam_bf16x2 __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ uint32_t f32x2_to_bf16x2_bits(float lo, float hi)
+{
+    const cam_f32x2 p = {lo, hi};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(p, cam_bf16x2));
+}
+
 // Round-to-nearest-even fp32 -> IEEE fp16 bit pattern (the hardware conversion; overflow gives infinity).
 __device__ __forceinline__ uint32_t f32_to_fp16_bits(float f)
 {

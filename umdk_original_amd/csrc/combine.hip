@@ -200,7 +200,7 @@ __global__ __launch_bounds__(kCombThreads) void combine_kernel(CombineArgs a, in
     v4u o;
 #pragma unroll
     for (int c = 0; c < 4; ++c) {
-        o[c] = ACT == 0 ? f32_to_bf16_bits(acc[2 * c]) | (f32_to_bf16_bits(acc[2 * c + 1]) << 16)
+        o[c] = ACT == 0 ? f32x2_to_bf16x2_bits(acc[2 * c], acc[2 * c + 1])
                         : f32_to_fp16_bits(acc[2 * c]) | (f32_to_fp16_bits(acc[2 * c + 1]) << 16);
     }
     __builtin_nontemporal_store(o, (v4u *)(a.out + (long long)t * a.H + col));
@@ -292,7 +292,7 @@ __global__ __launch_bounds__(kCombThreads) void combine_wire16_kernel(CombineArg
     v4u o[2];
 #pragma unroll
     for (int c = 0; c < 8; ++c) {
-        o[c >> 2][c & 3] = f32_to_bf16_bits(acc[2 * c]) | (f32_to_bf16_bits(acc[2 * c + 1]) << 16);
+        o[c >> 2][c & 3] = f32x2_to_bf16x2_bits(acc[2 * c], acc[2 * c + 1]);
     }
     v4u *dst = (v4u *)(a.out + (long long)t * a.H + col);
     __builtin_nontemporal_store(o[0], dst);

@@ -132,6 +132,9 @@ struct ItemCtx {
     bool wave_live;         // the group exists (ragged last column block)
     int stage_a, stage_bytes;
     int Kd, N;
+#ifdef CAM_GEMM_TIMELINE
+    int *phase_s;           // LDS: wall clock at the first multiply and after the K loop (written by thread 0)
+#endif
 };
 
 // One wave's part of one item.  TEAM 0 multiplies in the first phase of every sub-step, TEAM 1 in the second.
@@ -333,6 +336,11 @@ __device__ __forceinline__ void run_item(const GemmArgs &a, const ItemCtx &t, in
         wait_loads_outstanding<(NS - 1) * LPS>();
     }
     barrier_no_fence();  // stage 0 has landed and every wave's share of the scales is in LDS
+#ifdef CAM_GEMM_TIMELINE
+    if (tid == 0) {
+        t.phase_s[0] = (int)wall_clock64();
+    }
+#endif
     int slot = 0;        // slot of stage s
     const int steady = FLAT ? KT - NS : KT;  // sub-steps that request the stage NS ahead
     if (TEAM == 0) {
@@ -376,6 +384,11 @@ __device__ __forceinline__ void run_item(const GemmArgs &a, const ItemCtx &t, in
         wait_loads_outstanding<0>();
     }
     barrier_no_fence();  // nobody reads or fills the stages any more: the epilogue may stage through them
+#ifdef CAM_GEMM_TIMELINE
+    if (tid == 0) {
+        t.phase_s[1] = (int)wall_clock64();
+    }
+#endif
 
     // ---- epilogue, accumulators in registers.
     // Lane l holds activation row (l & 31) of each 32x32 fragment; registers 4j .. 4j+3 hold the four
@@ -504,18 +517,24 @@ __device__ __forceinline__ void run_item(const GemmArgs &a, const ItemCtx &t, in
                 for (int nf = 0; nf < 2; ++nf) {
 #pragma unroll
                     for (int j = 0; j < 4; ++j) {
-                        uint32_t b[4];
+                        float f[4];
 #pragma unroll
                         for (int e = 0; e < 4; ++e) {
-                            float v;
                             if constexpr (FP8) {
-                                v = acc[mf][nf][4 * j + e];
+                                f[e] = acc[mf][nf][4 * j + e];
                             } else {
-                                v = __fmul_rn(__fmul_rn((float)acc[mf][nf][4 * j + e], ws[nf][j][e]), xs);
+                                f[e] = __fmul_rn(__fmul_rn((float)acc[mf][nf][4 * j + e], ws[nf][j][e]), xs);
                             }
-                            b[e] = a.out_fp16 ? f32_to_fp16_bits(v) : f32_to_bf16_bits(v);
                         }
-                        const v2u v = {b[0] | (b[1] << 16), b[2] | (b[3] << 16)};
+                        // two values per conversion instruction: with the rounding spelled out in integer
+                        // arithmetic this epilogue took a quarter of a short-K tile's time in the vector ALU
+                        v2u v;
+                        if (a.out_fp16) {
+                            v = v2u{f32_to_fp16_bits(f[0]) | (f32_to_fp16_bits(f[1]) << 16),
+                                    f32_to_fp16_bits(f[2]) | (f32_to_fp16_bits(f[3]) << 16)};
+                        } else {
+                            v = v2u{f32x2_to_bf16x2_bits(f[0], f[1]), f32x2_to_bf16x2_bits(f[2], f[3])};
+                        }
                         *(v2u *)(slice + row_in * kEpiRowBytes + (nf * 32 + 8 * j + col_half) * 2) = v;
                     }
                 }
@@ -623,6 +642,9 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_kernel(GemmArgs a)
     __shared__ uint8_t w_scale8_s[FP8 ? 16 * kScaleKb : 4];
     __shared__ int item_s;
     __shared__ int next_s;
+#ifdef CAM_GEMM_TIMELINE
+    __shared__ int phase_s[2];
+#endif
 
     const int tid = threadIdx.x;
     const int team = __builtin_amdgcn_readfirstlane(tid >> 8);
@@ -738,6 +760,9 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_kernel(GemmArgs a)
         const bool flat = __builtin_amdgcn_readfirstlane(it.flat) != 0;
 
         ItemCtx t;
+#ifdef CAM_GEMM_TIMELINE
+        t.phase_s = phase_s;
+#endif
         t.Kd = a.Kd;
         t.N = a.N;
         t.m0 = m0;
@@ -853,6 +878,12 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_kernel(GemmArgs a)
             stamp[6] = (int32_t)timeline_t0;
             stamp[7] = (int32_t)wall_clock64();
             stamp[3] = (stamp[3] & 0xffff) | ((int)blockIdx.x << 16);  // split is read at the start of the item only
+            // ticks from the start of the item to its first multiply and to the end of its K loop, in the upper
+            // halves of the column-block and shape words (both below 2^16 and read before an item starts)
+            const int d1 = min(max(phase_s[0] - (int32_t)timeline_t0, 0), 0xffff);
+            const int d2 = min(max(phase_s[1] - (int32_t)timeline_t0, 0), 0x7fff);
+            stamp[4] = (stamp[4] & 0xffff) | (d1 << 16);
+            stamp[5] = (stamp[5] & 0xffff) | (d2 << 16);
         }
 #endif
         if (!flat && tid < kWave) {  // a flat item has taken its successor between its K loop and its epilogue
