@@ -154,7 +154,8 @@ def main():
         s_nt = calib("camCalibRowStores", 1)
         s_pl = calib("camCalibRowStores", 0)
         log("calib: 32768 rows of 7168 B stored to scattered row slots %.2f TB/s (plain stores %.2f), to consecutive "
-            "slots %.2f TB/s (plain %.2f)" % (s_nt[0], s_pl[0], s_nt[1], s_pl[1]))
+            "slots %.2f TB/s (plain %.2f); scattered with a workgroup per row %.2f (%.2f); plain fill of the same "
+            "bytes %.2f (%.2f)" % (s_nt[0], s_pl[0], s_nt[1], s_pl[1], s_nt[2], s_pl[2], s_nt[3], s_pl[3]))
         rd = calib("camCalibStreamRead")
         log("calib: streaming read of 1.5 GiB %.2f TB/s with plain loads, %.2f TB/s non-temporal" % (rd[0], rd[1]))
         do = calib("camCalibDestinationOrder")
@@ -164,7 +165,8 @@ def main():
             mfma_int8_alone=dict(pops=m0[0], ghz=m0[1]), mfma_int8_with_lds_reads=dict(pops=m1[0], ghz=m1[1]),
             mfma_int8_with_random_operands=dict(pops=m2[0], ghz=m2[1]),
             row_stores_tb_per_s=dict(scattered_nt=s_nt[0], scattered_plain=s_pl[0], linear_nt=s_nt[1],
-                                     linear_plain=s_pl[1]),
+                                     linear_plain=s_pl[1], scattered_workgroup_per_row_nt=s_nt[2],
+                                     scattered_workgroup_per_row_plain=s_pl[2], fill_nt=s_nt[3], fill_plain=s_pl[3]),
             stream_read_tb_per_s=dict(plain=rd[0], non_temporal=rd[1]),
             destination_order_us=dict(one_pass=do[0], quantise_tokens=do[1], row_copy=do[2], two_passes=do[3]))
 

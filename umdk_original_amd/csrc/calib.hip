@@ -183,6 +183,42 @@ __global__ __launch_bounds__(256) void store_rows_kernel(const int *slot, int ro
     }
 }
 
+// The same rows with a whole workgroup of four waves on each row (448 of its 512 16-byte pieces: two stores a thread).
+__global__ __launch_bounds__(256) void store_rows_wg_kernel(const int *slot, int rows, int8_t *out, int nt)
+{
+    const int r = blockIdx.x;
+    if (r >= rows) {
+        return;
+    }
+    v4u *dst = (v4u *)(out + (size_t)slot[r] * 7168);
+    const v4u v = {(unsigned)r, threadIdx.x, 3u, 4u};
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+        const int piece = i * 256 + (int)threadIdx.x;
+        if (piece < 448) {
+            if (nt) {
+                __builtin_nontemporal_store(v, dst + piece);
+            } else {
+                dst[piece] = v;
+            }
+        }
+    }
+}
+
+// A plain fill of the same bytes: 16 bytes per thread, consecutive threads on consecutive pieces.
+__global__ __launch_bounds__(256) void fill_kernel(v4u *out, long long n, int nt)
+{
+    const long long i = (long long)blockIdx.x * 256 + threadIdx.x;
+    if (i < n) {
+        const v4u v = {(unsigned)i, 2u, 3u, 4u};
+        if (nt) {
+            __builtin_nontemporal_store(v, out + i);
+        } else {
+            out[i] = v;
+        }
+    }
+}
+
 // Streaming read: 16 bytes per thread, one element per thread.
 __global__ __launch_bounds__(256) void stream_read_kernel(const v4u *in, long long n, int nt, unsigned *sink)
 {
@@ -351,7 +387,8 @@ CALIB_API int camCalibMfmaInt8(int mode, double *out)
 }
 
 // 32768 rows of 7168 bytes, four rotating outputs: out[0] = TB/s to scattered row slots, out[1] = TB/s to consecutive
-// ones (non-temporal stores if nt != 0).
+// ones (a wave per row), out[2] = scattered with a workgroup per row, out[3] = a plain fill of the same bytes
+// (non-temporal stores if nt != 0).
 CALIB_API int camCalibRowStores(int nt, double *out)
 {
     const int rows = kA, rot = 4;
@@ -381,6 +418,28 @@ CALIB_API int camCalibRowStores(int nt, double *out)
             return rc;
         }
         out[which] = (double)rows * kH / (us * 1e-6) / 1e12;
+    }
+    {  // out[2]: scattered rows, a workgroup per row; out[3]: a plain fill of the same bytes
+        double us = 0;
+        int rc = time_launches(
+            [&](int i) {
+                hipLaunchKernelGGL(store_rows_wg_kernel, dim3(rows), dim3(256), 0, 0, slot_scattered, rows, o[i % rot], nt);
+            },
+            8, 40, &us);
+        if (rc != 0) {
+            return rc;
+        }
+        out[2] = (double)rows * kH / (us * 1e-6) / 1e12;
+        const long long n = (long long)rows * kH / 16;
+        rc = time_launches(
+            [&](int i) {
+                hipLaunchKernelGGL(fill_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, 0, (v4u *)o[i % rot], n, nt);
+            },
+            8, 40, &us);
+        if (rc != 0) {
+            return rc;
+        }
+        out[3] = (double)rows * kH / (us * 1e-6) / 1e12;
     }
     return 0;
 }
