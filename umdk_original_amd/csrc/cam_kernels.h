@@ -95,6 +95,7 @@ struct SchedBuild {
     const int64_t *group_list;
     int cumulative, G, nspec;
     int queues;        // workgroups of the GEMM launch the schedule is for (set by the launchers: CUs of the device)
+    int parts;         // workgroups that share the building of one schedule (set by the launchers, 1..8)
     long long max_rows;
     SchedSpec spec[2];
 };

@@ -47,9 +47,10 @@ __global__ __launch_bounds__(kDispWaves * kWave, QUANT == 3 ? 3 : 4) void dispat
     // The first workgroups of the launch build the GEMM schedules (they start first and finish under the row
     // traffic of the others); they depend on nothing this launch writes.
     __shared__ SchedShared sched_s;
-    const int builders = a.sched.nspec;
+    const int builders = a.sched.nspec * a.sched.parts;
     if ((int)blockIdx.x < builders) {
-        build_sched_part<kDispWaves * kWave>(sched_s, a.sched, (int)blockIdx.x, 0, 1);
+        build_sched_part<kDispWaves * kWave>(sched_s, a.sched, (int)blockIdx.x / a.sched.parts,
+                                             (int)blockIdx.x % a.sched.parts, a.sched.parts);
         return;
     }
     const int t = ((int)blockIdx.x - builders) * kDispWaves + (threadIdx.x >> 6);
@@ -120,8 +121,13 @@ hipError_t launch_dispatch(const DispatchArgs &a_in, hipStream_t stream)
         if (qe != hipSuccess) {
             return qe;
         }
+        // a turn of items per builder workgroup where the item tables could be full
+        const int cap = max(a.sched.spec[0].max_items, a.sched.spec[a.sched.nspec - 1].max_items);
+        a.sched.parts = min(max((cap + kDispWaves * kWave - 1) / (kDispWaves * kWave), 1), 8);
+    } else {
+        a.sched.parts = 1;
     }
-    dim3 grid((a.T + kDispWaves - 1) / kDispWaves + a.sched.nspec), block(kDispWaves * kWave);
+    dim3 grid((a.T + kDispWaves - 1) / kDispWaves + a.sched.nspec * a.sched.parts), block(kDispWaves * kWave);
     if (a.smooth != nullptr) {
         if (a.quant != 2 || a.idx == nullptr || a.sched.nspec != 0) {
             return hipErrorInvalidValue;

@@ -895,7 +895,7 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_kernel(GemmArgs a)
 __global__ __launch_bounds__(1024) void build_sched_kernel(SchedBuild sb)
 {
     __shared__ SchedShared sh;
-    build_sched_part<1024>(sh, sb, (int)blockIdx.x, 0, 1);
+    build_sched_part<1024>(sh, sb, (int)blockIdx.y, (int)blockIdx.x, (int)gridDim.x);
 }
 
 // SwiGLU product rows (fp32) -> int8 rows + per-row scale:
@@ -1122,7 +1122,9 @@ hipError_t launch_build_sched(const int64_t *group_list, int cumulative, int G, 
     if (qe != hipSuccess) {
         return qe;
     }
-    hipLaunchKernelGGL(build_sched_kernel, dim3((unsigned)nspec), dim3(1024), 0, stream, sb);
+    const int cap = max(sb.spec[0].max_items, sb.spec[1].max_items);
+    sb.parts = min(max((cap + 1023) / 1024, 1), 4);  // a turn of items per workgroup where the tables could be full
+    hipLaunchKernelGGL(build_sched_kernel, dim3((unsigned)sb.parts, (unsigned)nspec), dim3(1024), 0, stream, sb);
     return hipGetLastError();
 }
 

@@ -167,7 +167,8 @@ __device__ __forceinline__ SchedItem make_item(const ExpertShape &e, int expert,
 
 // The shared-queue form of a schedule (long schedules); sh.rows / off / order / first_item are complete.
 template <int NT>
-__device__ __forceinline__ void build_shared_queues(SchedShared &sh, const SchedSpec &spec, int G, int n_items)
+__device__ __forceinline__ void build_shared_queues(SchedShared &sh, const SchedSpec &spec, int G, int n_items,
+                                                    int part, int parts)
 {
     const int tid = threadIdx.x;
     const int lane = tid & (kWave - 1);
@@ -233,7 +234,7 @@ __device__ __forceinline__ void build_shared_queues(SchedShared &sh, const Sched
         }
     }
     __syncthreads();
-    if (tid == 0) {
+    if (tid == 0 && part == 0) {
         int run = 0;
         for (int x = 0; x < kNumXcd; ++x) {
             sched[kSchedQueueStart + x] = min(run, spec.max_items);
@@ -246,8 +247,8 @@ __device__ __forceinline__ void build_shared_queues(SchedShared &sh, const Sched
         sched[2] = kNumXcd;
         sched[3] = 2;  // bit 1: shared queues
     }
-    // one thread per item
-    for (int i = tid; i < n_items; i += NT) {
+    // one thread per item; the parts take turns of NT items
+    for (int i = part * NT + tid; i < n_items; i += parts * NT) {
         int lo = 0, hi = G;  // largest rank with first_item <= i
         while (hi - lo > 1) {
             const int mid = (lo + hi) >> 1;
@@ -302,15 +303,13 @@ __device__ __forceinline__ void build_shared_queues(SchedShared &sh, const Sched
     }
 }
 
-// Schedule sb.spec[which]; called by all NT threads of a workgroup (NT a multiple of 64, at least 256).  One
-// workgroup builds a schedule: part != 0 returns at once.
+// Schedule sb.spec[which]; called by all NT threads of a workgroup (NT a multiple of 64, at least 256).  `parts`
+// workgroups share a schedule: each works out the same tables in its own LDS, part 0 writes the header and the queue
+// tables, and the items go round the parts in turns of NT (placing an item costs about a microsecond of dependent
+// lookups and divisions, and a long schedule has several thousand).
 template <int NT>
 __device__ __forceinline__ void build_sched_part(SchedShared &sh, const SchedBuild &sb, int which, int part, int parts)
 {
-    (void)parts;
-    if (part != 0) {
-        return;
-    }
     const int G = sb.G;
     const int tid = threadIdx.x;
     const int lane = tid & (kWave - 1);
@@ -401,7 +400,7 @@ __device__ __forceinline__ void build_sched_part(SchedShared &sh, const SchedBui
 
     // long schedules: eight shared queues
     if (n_items / m >= kSharedFrom && m >= kNumXcd) {
-        build_shared_queues<NT>(sh, spec, G, n_items);
+        build_shared_queues<NT>(sh, spec, G, n_items, part, parts);
         return;
     }
 
@@ -446,13 +445,13 @@ __device__ __forceinline__ void build_sched_part(SchedShared &sh, const SchedBui
         }
     }
     __syncthreads();
-    if (tid == 0) {
+    if (tid == 0 && part == 0) {
         sched[0] = min(n_items, spec.max_items);
         sched[1] = sh.total_rows;
         sched[2] = m;
         sched[3] = R + (b > 0 ? 1 : 0) <= 1 ? 1 : 0;  // bit 0: no queue holds a second item, nothing can be taken over
     }
-    for (int w = tid; w <= m; w += NT) {  // the launch has m workgroups: the entries beyond are never read
+    for (int w = tid; w <= m && part == 0; w += NT) {  // m workgroups: the entries beyond are never read
         sched[kSchedQueueStart + w] = min(sh.qstart[w], spec.max_items);
         if (w < m) {
             // the first item of a queue belongs to its workgroup without asking; the counter starts behind it
@@ -460,8 +459,8 @@ __device__ __forceinline__ void build_sched_part(SchedShared &sh, const SchedBui
         }
     }
 
-    // one thread per item
-    for (int i = tid; i < n_items; i += NT) {
+    // one thread per item; the parts take turns of NT items
+    for (int i = part * NT + tid; i < n_items; i += parts * NT) {
         int lo = 0, hi = G;  // largest rank with first_item <= i
         while (hi - lo > 1) {
             const int mid = (lo + hi) >> 1;
