@@ -1123,7 +1123,7 @@ hipError_t launch_build_sched(const int64_t *group_list, int cumulative, int G, 
         return qe;
     }
     const int cap = max(sb.spec[0].max_items, sb.spec[1].max_items);
-    sb.parts = min(max((cap + 1023) / 1024, 1), 4);  // a turn of items per workgroup where the tables could be full
+    sb.parts = min(max(cap / 2048, 1), 4);  // long tables only: two turns of a thousand items cost no more than a second workgroup
     hipLaunchKernelGGL(build_sched_kernel, dim3((unsigned)sb.parts, (unsigned)nspec), dim3(1024), 0, stream, sb);
     return hipGetLastError();
 }
