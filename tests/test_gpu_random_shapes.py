@@ -137,3 +137,74 @@ def test_fused_layer_random_shape(gpu, oracle, seed):
                                         n_active=n_active)
     assert_bits_equal(to_np(etn), want_etn, "expert_token_nums")
     assert_bits_equal(to_np(out), want, "layer output")
+
+
+def _bits16(t):
+    return t.cpu().contiguous().view(torch.int16).numpy().view(np.uint16)
+
+
+@pytest.mark.parametrize("seed", range(10 * SCALE))
+def test_shmem_pair_random_shape(gpu, oracle, seed):
+    rng = np.random.default_rng(4000 + seed)
+    T = int(rng.integers(1, 300))
+    E = int(rng.choice([2, 8, 24, 64, 256]))
+    K = int(rng.integers(1, min(16, E) + 1))
+    H = int(rng.choice([1024, 1032, 2048, 4096, 7168]))
+    quant = int(rng.choice([0, 2]))
+    smooth = quant == 2 and bool(rng.integers(0, 2))
+    fp16 = bool(rng.integers(0, 2))
+    ttype = int(rng.integers(0, 2))
+    comm = 0 if fp16 else int(rng.choice([0, 2]))  # (int8 wire rows are built for bf16 rows)
+    announce("random shmem pair seed=%d T=%d K=%d E=%d H=%d quant=%d smooth=%d fp16=%d type=%d comm=%d" %
+             (seed, T, K, E, H, quant, smooth, fp16, ttype, comm))
+    ids, w = synth.sigmoid_zipf_routing(T, E, K, seed=seed + 70)
+    ids = ids.to(torch.int32)
+    drop = torch.from_numpy(rng.random((T, K)) < 0.1)
+    ids[drop] = -1
+    x = synth.normal_bf16(T, H, seed=seed + 71)
+    if fp16:
+        x = x.half()
+    sm = None
+    if smooth:
+        sm = torch.from_numpy((rng.random((E, H)) * 3.75 + 0.25).astype(np.float32))
+    want = oracle.dispatch_shmem(_bits16(x), ids.numpy(), E, quant, smooth=None if sm is None else sm.numpy(), fp16=fp16,
+                                 token_nums_type=ttype)
+    got = cam.moe_dispatch_shmem(x.to(gpu), ids.to(gpu), None if sm is None else sm.to(gpu), None, 1, 0, E, 1, 0, 0, 1, 0,
+                                 quant, 0, ttype, 0)
+    total = want[5]
+    assert_bits_equal(to_np(got[2]), want[2], "expandIdx")
+    assert_bits_equal(to_np(got[3]), want[3], "expertTokenNums")
+    assert_bits_equal(to_np(got[4]), want[4], "epRecvCount")
+    if quant:
+        assert_bits_equal(to_np(got[0])[:total], want[0][:total], "expandX (int8)")
+        assert_bits_equal(to_np(got[1])[:total].view(np.uint32), want[1][:total].view(np.uint32), "dynamicScales")
+    else:
+        assert_bits_equal(_bits16(got[0])[:total], want[0][:total], "expandX (copy)")
+    # the way back, from rows of the activation type
+    y = synth.normal_bf16(got[0].size(0), H, seed=seed + 72)
+    if fp16:
+        y = y.half()
+    back = cam.moe_combine_shmem(y.to(gpu), ids.to(gpu), got[2], got[4], w.to(gpu), epWorldSize=1, moeExpertNum=E,
+                                 commQuantMode=comm)
+    want_back = oracle.combine_shmem(_bits16(y), ids.numpy(), to_np(got[2]), to_np(got[4]), w.numpy(), E, fp16=fp16,
+                                     comm_quant=comm == 2)
+    assert_bits_equal(_bits16(back), want_back, "combined rows")
+
+
+@pytest.mark.parametrize("seed", range(4 * SCALE))
+def test_fp8_fused_layer_random_shape(gpu, oracle, seed):
+    from test_gpu_fp8 import _layer_inputs, _check_layer, _u8
+    rng = np.random.default_rng(5000 + seed)
+    T = int(rng.integers(1, 160))
+    E = int(rng.choice([2, 4, 8, 16, 32]))
+    K = int(rng.integers(1, min(8, E) + 1))
+    H = int(rng.choice([1024, 1536, 2048]))
+    I = int(rng.choice([512, 768, 1024]))
+    announce("random fp8 layer seed=%d T=%d K=%d E=%d H=%d I=%d" % (seed, T, K, E, H, I))
+    ids, w, x, w1, s1, w2, s2 = _layer_inputs(T, H, E, K, I, seed=seed + 90)
+    out, etn = cam.fused_deep_moe_fp8(x.to(gpu), ids.to(torch.int32).to(gpu), cam.prepack_weight(w1.to(gpu), True),
+                                      s1.to(gpu), cam.prepack_weight(w2.to(gpu), False), s2.to(gpu), w.to(gpu))
+    want, dbg = oracle.fp8_fused_layer(synth.bf16_bits(x), ids.numpy(), w.numpy(), _u8(w1), s1.numpy(), _u8(w2),
+                                       s2.numpy(), debug=True)
+    assert np.array_equal(etn.cpu().numpy(), dbg["cnt"])
+    _check_layer(out.float().cpu().numpy(), want)
