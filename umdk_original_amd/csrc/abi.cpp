@@ -2026,6 +2026,7 @@ camStatus camGroupedMatmulFp8GetWorkspaceSize(const camTensor *x, const camTenso
     const int64_t N = gate_up ? 2 * out->sizes[1] : out->sizes[1];
     CAM_TRY(check_fp8_dims("GroupedMatmulFp8", Kd, N, gate_up));
     CAM_TRY(check_aligned(out, "out", 16));
+    CAM_TRY(check_aligned(xScale, "xScale", 4));  // a row's block scales are fetched as words
     Fp8Weight fw{};
     CAM_TRY(check_fp8_weight(weight, weightScale, "weight", G, Kd, N, &fw));
     cam::SchedSpec sp = sched_spec(A, G, N, Kd, gate_up);

@@ -790,10 +790,42 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_kernel(GemmArgs a)
             if (FP8) {
                 // the item's scales: activation rows x K blocks (transposed, so that the lanes of a fragment read
                 // neighbouring bytes), and one row of K blocks per 64-column group of the item
+                // Only the rows the fragments read (the tile's rows, to the next multiple of 32), four K blocks per
+                // load where a row's scales are whole words, and four loads in flight per thread: fetched a byte at a
+                // time for all 256 rows, with a wait per byte, this took 3-4 us of every item.
                 const int KB = a.Kd >> 7;
-                for (int i = tid; i < 256 * KB; i += kThreads) {
-                    const int r = i / KB, kb = i - r * KB;
-                    a_scale8_s[kb * 256 + r] = a.a_scale8[(long long)(m0 + min(r, rows - 1)) * KB + kb];
+                const int rpad = min(256, (rows + 31) & ~31);
+                if ((KB & 3) == 0) {
+                    const int wpr = KB >> 2;  // words per row
+                    const int total = rpad * wpr;
+                    constexpr int U = 4;
+                    for (int base = tid; base < total; base += U * kThreads) {
+                        uint32_t v[U] = {0u, 0u, 0u, 0u};
+                        int r[U], q[U];
+#pragma unroll
+                        for (int u = 0; u < U; ++u) {
+                            const int i = base + u * kThreads;
+                            r[u] = i / wpr;
+                            q[u] = i - r[u] * wpr;
+                            if (i < total) {
+                                v[u] = *(const uint32_t *)(a.a_scale8 + (long long)(m0 + min(r[u], rows - 1)) * KB + 4 * q[u]);
+                            }
+                        }
+#pragma unroll
+                        for (int u = 0; u < U; ++u) {
+                            if (base + u * kThreads < total) {
+#pragma unroll
+                                for (int j = 0; j < 4; ++j) {
+                                    a_scale8_s[(4 * q[u] + j) * 256 + r[u]] = (uint8_t)(v[u] >> (8 * j));
+                                }
+                            }
+                        }
+                    }
+                } else {
+                    for (int i = tid; i < rpad * KB; i += kThreads) {
+                        const int r = i / KB, kb = i - r * KB;
+                        a_scale8_s[kb * 256 + r] = a.a_scale8[(long long)(m0 + min(r, rows - 1)) * KB + kb];
+                    }
                 }
                 const int ngr = flat ? 8 : 4;
                 const int nblk = a.N >> 7;
