@@ -638,7 +638,7 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_kernel(GemmArgs a)
 {
     __shared__ __attribute__((aligned(1024))) int8_t lds[kLdsBytes];
     __shared__ float row_scale_s[256];
-    __shared__ uint8_t a_scale8_s[FP8 ? kScaleKb * 256 : 4];
+    __shared__ __attribute__((aligned(16))) uint8_t a_scale8_s[FP8 ? kScaleKb * 256 : 4];
     __shared__ uint8_t w_scale8_s[FP8 ? 16 * kScaleKb : 4];
     __shared__ int item_s;
     __shared__ int next_s;
@@ -790,35 +790,28 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_kernel(GemmArgs a)
             if (FP8) {
                 // the item's scales: activation rows x K blocks (transposed, so that the lanes of a fragment read
                 // neighbouring bytes), and one row of K blocks per 64-column group of the item
-                // Only the rows the fragments read (the tile's rows, to the next multiple of 32), four K blocks per
-                // load where a row's scales are whole words, and four loads in flight per thread: fetched a byte at a
-                // time for all 256 rows, with a wait per byte, this took 3-4 us of every item.
+                // Only the rows the fragments read (the tile's rows, to the next multiple of 32), and, where a row's
+                // scales are whole words, four K blocks per load and four loads in flight per thread: fetched a byte
+                // at a time for all 256 rows, with a wait per byte, this took 3-4 us of every item.
                 const int KB = a.Kd >> 7;
                 const int rpad = min(256, (rows + 31) & ~31);
                 if ((KB & 3) == 0) {
-                    const int wpr = KB >> 2;  // words per row
-                    const int total = rpad * wpr;
-                    constexpr int U = 4;
-                    for (int base = tid; base < total; base += U * kThreads) {
-                        uint32_t v[U] = {0u, 0u, 0u, 0u};
-                        int r[U], q[U];
+                    // a thread takes four K blocks of four consecutive rows: four word loads, a 4x4 byte transpose,
+                    // four word stores (neighbouring lanes write neighbouring words)
+                    const int wpr = KB >> 2;    // words per row
+                    const int rgs = rpad >> 2;  // groups of four rows
+                    for (int i = tid; i < rgs * wpr; i += kThreads) {
+                        const int q = i / rgs, rg = i - q * rgs;
+                        uint32_t v[4];
 #pragma unroll
-                        for (int u = 0; u < U; ++u) {
-                            const int i = base + u * kThreads;
-                            r[u] = i / wpr;
-                            q[u] = i - r[u] * wpr;
-                            if (i < total) {
-                                v[u] = *(const uint32_t *)(a.a_scale8 + (long long)(m0 + min(r[u], rows - 1)) * KB + 4 * q[u]);
-                            }
+                        for (int u = 0; u < 4; ++u) {
+                            v[u] = *(const uint32_t *)(a.a_scale8 + (long long)(m0 + min(4 * rg + u, rows - 1)) * KB + 4 * q);
                         }
 #pragma unroll
-                        for (int u = 0; u < U; ++u) {
-                            if (base + u * kThreads < total) {
-#pragma unroll
-                                for (int j = 0; j < 4; ++j) {
-                                    a_scale8_s[(4 * q[u] + j) * 256 + r[u]] = (uint8_t)(v[u] >> (8 * j));
-                                }
-                            }
+                        for (int j = 0; j < 4; ++j) {
+                            const uint32_t w = ((v[0] >> (8 * j)) & 0xffu) | (((v[1] >> (8 * j)) & 0xffu) << 8) |
+                                               (((v[2] >> (8 * j)) & 0xffu) << 16) | (((v[3] >> (8 * j)) & 0xffu) << 24);
+                            *(uint32_t *)(a_scale8_s + (4 * q + j) * 256 + 4 * rg) = w;
                         }
                     }
                 } else {
