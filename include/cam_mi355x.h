@@ -265,10 +265,11 @@ CAM_API camStatus camMoeCombineNormal(void *workspace, uint64_t workspaceSize, c
  *   epRecvCountsOptional int32 [E]: when given, rows at or past its last element are never read.
  *   Same arithmetic and limits as MoeCombineNormal.
  *   recvX may instead hold rows quantised for the wire, int8 [A, H + H/4] (H = out's columns): H int8 values,
- *   then one bf16 scale per block of 8 columns -- the int8 communication quantisation of
- *   AK/moe_combine_shmem/op_kernel/moe_combine_shmem.h:564-592.  Each value is rebuilt as
- *   bf16(float(q) * float(scale)) (:755-773) before it is weighted and summed.  GroupedMatmulDequant writes
- *   such rows when its out tensor is int8.
+ *   then one 16-bit scale per block of 8 columns -- the int8 communication quantisation of
+ *   AK/moe_combine_shmem/op_kernel/moe_combine_shmem.h:564-592.  The scales have the type of the rows the wire
+ *   rows were made from, and out's type says which that is (bf16, or IEEE fp16).  Each value is rebuilt as
+ *   round_to_that_type(float(q) * float(scale)) (:755-773) before it is weighted and summed.
+ *   GroupedMatmulDequant writes such rows (from bf16) when its out tensor is int8.
  *   sharedXOptional [T,H] of out's type: the shared expert's output row of every token, added un-weighted to
  *   the fp32 accumulator after the K routed rows and before the one rounding
  *   (FDM/raw_distributed/cam_moe_distribute_combine.h:757-774; AK/moe_combine_shmem/op_kernel/
@@ -321,8 +322,8 @@ CAM_API camStatus camMoeDispatchShmem(void *workspace, uint64_t workspaceSize, c
  * fp32 [bs,K]; the six optional tensors are reserved in the reference and must be NULL -> out [bs,H] of
  * expandX's type: out[t] = round(sum over k ascending of float(row(t,k)) * expertScales[t,k]), multiply and add
  * rounded separately (AK/moe_combine_shmem/op_kernel/moe_combine_shmem.h:819-912), row(t,k) located as above
- * (:514-556,:833-837).  commQuantMode 2 (bf16 rows only): every row first takes the int8 wire format of :567-592
- * (blocks of 8 columns, bf16 scales) and is rebuilt as :755-773 before it is weighted -- the rounding a row
+ * (:514-556,:833-837).  commQuantMode 2: every row first takes the int8 wire format of :567-592 (blocks of 8
+ * columns, scales of expandX's type) and is rebuilt as :755-773 before it is weighted -- the rounding a row
  * suffers when it crosses ranks; 0: rows are used as they are.  Ids outside [0, moeExpertNum) are skipped.
  * epWorldSize must be 1 (sharedExpertRankNum 0, tpWorldSize <= 1); the shared expert's add-back, which needs a
  * shared-expert rank there, is available as MoeCombineGather's sharedXOptional.

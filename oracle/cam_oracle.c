@@ -19,7 +19,7 @@
  *     1.2e-5 relative of the exact function) in place of the Ascend Exp and Div instructions;
  *   - everything downstream of it (cam_oracle_swiglu_quant's int8 values, the bf16 layer output)
  *     inherits that; the reference's own acceptance bound there is atol 2.0 / rtol 0.02;
- *   - cam_oracle_comm_quant_rows and cam_oracle_dispatch_shmem take the Ascend Div to be the IEEE quotient
+ *   - cam_oracle_comm_quant_rows(_act) and cam_oracle_dispatch_shmem take the Ascend Div to be the IEEE quotient
  *     and every written operation to round once.
  * All-zero rows (division by zero in the reference, AK/.../grouped_matmul_slice_m_per_token_dequant_
  * swiglu_quant_multistage_workspace.h:804 and :252-255) are defined here as q = 0, scale = 0.
@@ -503,8 +503,10 @@ ORACLE_API uint16_t cam_oracle_f32_to_fp16(float x) { return f32_to_fp16(x); }
 
 #define CAM_COMMQ_BLOCK 8
 
-/* x [A,H] bf16 bits -> out [A, H + H/4] bytes */
-ORACLE_API void cam_oracle_comm_quant_rows(const uint16_t *x, int64_t A, int64_t H, uint8_t *out)
+/* x [A,H] bits of the activation type (act: 0 bf16, 1 fp16) -> out [A, H + H/4] bytes: H int8 values, then one
+ * scale of the activation type per block of 8 columns (moe_combine_shmem.h:567-592: block maximum * 1/127, kept in
+ * fp32 for the division, stored rounded to ExpandXType; quotient rounded to fp16, then to int8, both to nearest even). */
+ORACLE_API void cam_oracle_comm_quant_rows_act(const uint16_t *x, int64_t A, int64_t H, int act, uint8_t *out)
 {
     const int64_t pitch = H + H / 4;
 #pragma omp parallel for schedule(static)
@@ -515,7 +517,8 @@ ORACLE_API void cam_oracle_comm_quant_rows(const uint16_t *x, int64_t A, int64_t
         for (int64_t b = 0; b < H / CAM_COMMQ_BLOCK; ++b) {
             float m = 0.0f;
             for (int j = 0; j < CAM_COMMQ_BLOCK; ++j) {
-                float a = fabsf(bf16_to_f32(xr[b * CAM_COMMQ_BLOCK + j]));
+                uint16_t bits = xr[b * CAM_COMMQ_BLOCK + j];
+                float a = fabsf(act ? fp16_to_f32(bits) : bf16_to_f32(bits));
                 m = a > m ? a : m;
             }
             if (m == 0.0f) {
@@ -526,17 +529,24 @@ ORACLE_API void cam_oracle_comm_quant_rows(const uint16_t *x, int64_t A, int64_t
                 continue;
             }
             float s = m * (1.0f / 127.0f);
-            sc[b] = f32_to_bf16(s);
+            sc[b] = act ? f32_to_fp16(s) : f32_to_bf16(s);
             for (int j = 0; j < CAM_COMMQ_BLOCK; ++j) {
-                float v = bf16_to_f32(xr[b * CAM_COMMQ_BLOCK + j]) / s;
+                uint16_t bits = xr[b * CAM_COMMQ_BLOCK + j];
+                float v = (act ? fp16_to_f32(bits) : bf16_to_f32(bits)) / s;
                 q[b * CAM_COMMQ_BLOCK + j] = (int8_t)nearbyintf(fp16_to_f32(f32_to_fp16(v)));
             }
         }
     }
 }
 
-/* packed [A, H + H/4] -> bf16 bits [A,H] */
-ORACLE_API void cam_oracle_comm_dequant_rows(const uint8_t *packed, int64_t A, int64_t H, uint16_t *out)
+ORACLE_API void cam_oracle_comm_quant_rows(const uint16_t *x, int64_t A, int64_t H, uint8_t *out)
+{
+    cam_oracle_comm_quant_rows_act(x, A, H, 0, out);
+}
+
+/* packed [A, H + H/4] -> bits of the activation type [A,H] (moe_combine_shmem.h:755-773: int8 -> fp32, times the
+ * block's scale widened to fp32, rounded to ExpandXType) */
+ORACLE_API void cam_oracle_comm_dequant_rows_act(const uint8_t *packed, int64_t A, int64_t H, int act, uint16_t *out)
 {
     const int64_t pitch = H + H / 4;
 #pragma omp parallel for schedule(static)
@@ -544,9 +554,16 @@ ORACLE_API void cam_oracle_comm_dequant_rows(const uint8_t *packed, int64_t A, i
         const int8_t *q = (const int8_t *)(packed + r * pitch);
         const uint16_t *sc = (const uint16_t *)(packed + r * pitch + H);
         for (int64_t h = 0; h < H; ++h) {
-            out[r * H + h] = f32_to_bf16((float)q[h] * bf16_to_f32(sc[h / CAM_COMMQ_BLOCK]));
+            uint16_t sb = sc[h / CAM_COMMQ_BLOCK];
+            float p = (float)q[h] * (act ? fp16_to_f32(sb) : bf16_to_f32(sb));
+            out[r * H + h] = act ? f32_to_fp16(p) : f32_to_bf16(p);
         }
     }
+}
+
+ORACLE_API void cam_oracle_comm_dequant_rows(const uint8_t *packed, int64_t A, int64_t H, uint16_t *out)
+{
+    cam_oracle_comm_dequant_rows_act(packed, A, H, 0, out);
 }
 
 /* the same with rows and output in the activation type `act` (0 bf16, 1 fp16) */
@@ -693,7 +710,7 @@ ORACLE_API int64_t cam_oracle_dispatch_shmem(const uint16_t *x, const int32_t *i
  * running totals) and the slot's place inside them is expandIdx[t*K+k] (:833-837).  comm_quant != 0 passes every
  * row through the int8 wire format on its way (quantise :567-592, dequantise :755-773) before it is weighted;
  * then acc = acc + float(row) * w[t,k] for k ascending, and one rounding to the activation type (:908-912).
- * Ids outside [0,E) are skipped (the reference does not guard them).  bf16 only when comm_quant != 0. */
+ * Ids outside [0,E) are skipped (the reference does not guard them). */
 ORACLE_API void cam_oracle_combine_shmem(const uint16_t *expand_x, const int32_t *ids, const int32_t *expand_idx,
                                          const int32_t *ep_send_counts, const float *w, int64_t A, int64_t T,
                                          int64_t K, int64_t H, int64_t E, int act, int comm_quant, uint16_t *out)
@@ -713,9 +730,9 @@ ORACLE_API void cam_oracle_combine_shmem(const uint16_t *expand_x, const int32_t
     if (comm_quant) {
         uint8_t *wire = (uint8_t *)malloc((size_t)(A > 0 ? A : 1) * (size_t)(H + H / 4));
         uint16_t *rows = (uint16_t *)malloc((size_t)(A > 0 ? A : 1) * (size_t)H * 2);
-        cam_oracle_comm_quant_rows(expand_x, A, H, wire);
-        cam_oracle_comm_dequant_rows(wire, A, H, rows);
-        cam_oracle_combine_shared(rows, row_of, w, NULL, T, K, H, 0, out);
+        cam_oracle_comm_quant_rows_act(expand_x, A, H, act, wire);
+        cam_oracle_comm_dequant_rows_act(wire, A, H, act, rows);
+        cam_oracle_combine_shared(rows, row_of, w, NULL, T, K, H, act, out);
         free(wire);
         free(rows);
     } else {

@@ -325,22 +325,23 @@ def f32_to_fp16_bits(a):
     return np.array([f(float(v)) for v in a.ravel()], np.uint16).reshape(a.shape)
 
 
-def comm_quant_rows(y_bits):
-    """bf16 rows [A,H] -> wire rows [A, H + H/4] uint8: H int8 values, then H/8 bf16 block scales."""
+def comm_quant_rows(y_bits, fp16=False):
+    """bf16 (or fp16) rows [A,H] -> wire rows [A, H + H/4] uint8: H int8 values, then H/8 block scales of the
+    rows' type."""
     y_bits = _c(y_bits, np.uint16)
     A, H = y_bits.shape
     assert H % 8 == 0
     out = np.zeros((A, H + H // 4), np.uint8)
-    lib().cam_oracle_comm_quant_rows(_p(y_bits), _i64(A), _i64(H), _p(out))
+    lib().cam_oracle_comm_quant_rows_act(_p(y_bits), _i64(A), _i64(H), ctypes.c_int(1 if fp16 else 0), _p(out))
     return out
 
 
-def comm_dequant_rows(packed, H):
+def comm_dequant_rows(packed, H, fp16=False):
     packed = _c(packed, np.uint8)
     A = packed.shape[0]
     assert packed.shape[1] == H + H // 4
     out = np.zeros((A, H), np.uint16)
-    lib().cam_oracle_comm_dequant_rows(_p(packed), _i64(A), _i64(H), _p(out))
+    lib().cam_oracle_comm_dequant_rows_act(_p(packed), _i64(A), _i64(H), ctypes.c_int(1 if fp16 else 0), _p(out))
     return out
 
 

@@ -249,7 +249,7 @@ def test_combine_shmem_validation():
     st, ws2, _ = _lib.phase1("MoeCombineShmem", _combine_shmem_args(comm=2))
     assert st == CAM_OK and ws2 >= ws0 + 8 * (1024 + 256)  # the wire rows live in the workspace
     assert _lib.phase1("MoeCombineShmem", _combine_shmem_args(dtype=torch.float16))[0] == CAM_OK
-    assert _lib.phase1("MoeCombineShmem", _combine_shmem_args(comm=2, dtype=torch.float16))[0] == CAM_ERR_UNSUPPORTED
+    assert _lib.phase1("MoeCombineShmem", _combine_shmem_args(comm=2, dtype=torch.float16))[0] == CAM_OK
     assert _lib.phase1("MoeCombineShmem", _combine_shmem_args(comm=1))[0] == CAM_ERR_RANGE
     for pos in (6, 7, 8, 9, 10):  # reserved inputs
         a = _combine_shmem_args()

@@ -81,6 +81,28 @@ def test_combine_from_wire_rows_bit_exact(gpu, oracle, T, K, E, H):
     _wire_case(gpu, oracle, T, K, E, H, seed=T + K + 5)
 
 
+@pytest.mark.parametrize("T,K,E,H", [(33, 8, 64, 7168), (21, 3, 8, 1032)])
+def test_combine_from_wire_rows_of_fp16_rows(gpu, oracle, T, K, E, H):
+    """Wire rows made from IEEE fp16 rows carry fp16 block scales; an fp16 output selects that reading."""
+    announce("combine from fp16 wire rows T=%d K=%d E=%d H=%d" % (T, K, E, H))
+    ids, w = synth.sigmoid_zipf_routing(T, E, K, seed=T + 9)
+    idx_np = ids.numpy()
+    cnt, off, pos, _ = plan_oracle(oracle, idx_np, E)
+    A = T * K
+    y = synth.normal_bf16(A, H, seed=T + 10).half()
+    y[0] = 0
+    y[1] = y[1] * 1e-4   # block scales in fp16's subnormal range
+    y[2] = y[2] * 1e4
+    bits = y.view(torch.int16).numpy().view(np.uint16)
+    packed = oracle.comm_quant_rows(bits, fp16=True)
+    row_of = oracle.rows_from_pos(idx_np, off, pos, E)
+    want = oracle.combine_act(oracle.comm_dequant_rows(packed, H, fp16=True), row_of, w.numpy(), True)
+    out = torch.empty((T, H), dtype=torch.float16, device=gpu)
+    got = cam.moe_combine_gather(torch.from_numpy(packed.view(np.int8)).to(gpu), None,
+                                 torch.from_numpy(row_of.reshape(T, K)).to(gpu), w.to(gpu), out=out)
+    assert_bits_equal(got.cpu().view(torch.int16).numpy().view(np.uint16), want, "combined x from fp16 wire rows")
+
+
 def test_combine_from_wire_rows_full_size(gpu, oracle):
     """C4 shape with wire rows: bit-exact against the oracle, and close to the combine of the unquantised rows."""
     announce("combine from wire rows, C4 full size")

@@ -154,7 +154,7 @@ def test_shmem_pair_random_shape(gpu, oracle, seed):
     smooth = quant == 2 and bool(rng.integers(0, 2))
     fp16 = bool(rng.integers(0, 2))
     ttype = int(rng.integers(0, 2))
-    comm = 0 if fp16 else int(rng.choice([0, 2]))  # (int8 wire rows are built for bf16 rows)
+    comm = int(rng.choice([0, 2]))
     announce("random shmem pair seed=%d T=%d K=%d E=%d H=%d quant=%d smooth=%d fp16=%d type=%d comm=%d" %
              (seed, T, K, E, H, quant, smooth, fp16, ttype, comm))
     ids, w = synth.sigmoid_zipf_routing(T, E, K, seed=seed + 70)

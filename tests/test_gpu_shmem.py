@@ -53,7 +53,8 @@ def test_dispatch_shmem_bit_exact(gpu, oracle, T, K, E, H, quant, smooth, fp16, 
 
 @pytest.mark.parametrize("T,K,E,H,comm,fp16", [(1, 1, 2, 1024, 0, False), (64, 8, 32, 7168, 0, False),
                                                 (37, 4, 8, 1032, 2, False), (300, 8, 64, 4096, 2, False),
-                                                (50, 3, 16, 2048, 0, True)])
+                                                (50, 3, 16, 2048, 0, True), (45, 4, 8, 1032, 2, True),
+                                                (200, 8, 64, 7168, 2, True)])
 def test_combine_shmem_bit_exact(gpu, oracle, T, K, E, H, comm, fp16):
     announce("combine shmem T=%d K=%d E=%d H=%d comm=%d fp16=%d" % (T, K, E, H, comm, fp16))
     ids, w = synth.sigmoid_zipf_routing(T, E, K, seed=T + E + 1)

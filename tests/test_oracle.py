@@ -575,6 +575,40 @@ def test_comm_quant_rows_definition_and_layout(oracle):
     assert (err <= scf[:, :, None] * 0.51 + np.abs(oracle_bits_to_f32(bits)).reshape(A, H // 8, 8) * 2 ** -6 + 1e-30).all()
 
 
+def test_comm_quant_rows_of_fp16_rows_keep_fp16_scales(oracle):
+    """The same wire format from IEEE fp16 rows: the block scales are stored as fp16 (the reference keeps them in the
+    rows' type, moe_combine_shmem.h:572,581) and the rows come back rounded to fp16.  Checked against numpy's own
+    float16 / float32 arithmetic."""
+    A, H = 29, 1024
+    rng = np.random.default_rng(12)
+    x = rng.normal(0, 1, size=(A, H)).astype(np.float16)
+    x[2] = 0
+    x[3, :8] = 0
+    x[4, 8:16] = np.array([6e-5, -3e-5, 1e-5, 0, 6e-8, 0, 0, 0], np.float16)   # a block of (near-)subnormals
+    x[5, 16:24] = np.array([60000, -65504, 1, 2, 3, 4, 5, 6], np.float16)      # the top of the range
+    bits = x.view(np.uint16)
+    packed = oracle.comm_quant_rows(bits, fp16=True)
+    q = packed[:, :H].view(np.int8)
+    sc_bits = np.ascontiguousarray(packed[:, H:]).view(np.uint16)
+    blk = x.astype(np.float32).reshape(A, H // 8, 8)
+    m = np.max(np.abs(blk), axis=2).astype(np.float32)
+    s = (m * np.float32(1.0 / 127.0)).astype(np.float32)
+    with np.errstate(divide="ignore", invalid="ignore", over="ignore"):
+        v = (blk / s[:, :, None]).astype(np.float32)
+        want_q = np.rint(v.astype(np.float16).astype(np.float32))
+        want_s = s.astype(np.float16)
+    want_q[m == 0] = 0
+    assert np.array_equal(q, want_q.astype(np.int8).reshape(A, H))
+    assert np.array_equal(sc_bits, want_s.view(np.uint16))
+    back = oracle.comm_dequant_rows(packed, H, fp16=True)
+    with np.errstate(over="ignore"):
+        want_back = (q.astype(np.float32).reshape(A, H // 8, 8) * want_s.astype(np.float32)[:, :, None]).astype(np.float16)
+    assert np.array_equal(back, want_back.reshape(A, H).view(np.uint16))
+    # bf16 rows through the same entry points are unchanged by the new argument
+    xb = synth.bf16_bits(synth.normal_bf16(5, H, seed=3))
+    assert np.array_equal(oracle.comm_quant_rows(xb), oracle.comm_quant_rows(xb, fp16=False))
+
+
 def test_comm_quant_double_rounding_is_kept(oracle):
     """x / s just below a half-integer rounds up to it in fp16 and then to the even neighbour: the reference casts
     float -> half -> int8 (moe_combine_shmem.h:587-589), and so must a restatement."""

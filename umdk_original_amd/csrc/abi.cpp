@@ -1059,7 +1059,8 @@ camStatus camMoeCombineGatherGetWorkspaceSize(const camTensor *recvX, const camT
     CAM_TRY(check_tensor(slotRow, "slotRow", 2, CAM_DT_INT32));
     CAM_TRY(check_tensor(recvTopkWeights, "recvTopkWeights", 2, CAM_DT_FLOAT));
     const bool wire = recvX->dtype == CAM_DT_INT8;
-    CAM_TRY(check_tensor(out, "out", 2, wire ? CAM_DT_BF16 : recvX->dtype));
+    // (wire rows carry block scales of the type they were quantised from, which is the type they come back as)
+    CAM_TRY(check_tensor(out, "out", 2, wire ? (out->dtype == CAM_DT_FLOAT16 ? CAM_DT_FLOAT16 : CAM_DT_BF16) : recvX->dtype));
     const int64_t A = recvX->sizes[0], H = out->sizes[1];
     const int64_t T = recvTopkWeights->sizes[0], K = recvTopkWeights->sizes[1];
     if (recvX->sizes[1] != (wire ? H + H / 4 : H)) {
@@ -1120,7 +1121,7 @@ camStatus camMoeCombineGatherGetWorkspaceSize(const camTensor *recvX, const camT
     g.H = (int)H;
     g.A = A;
     g.wire_rows = wire ? 1 : 0;
-    g.act_fp16 = recvX->dtype == CAM_DT_FLOAT16;
+    g.act_fp16 = (wire ? out->dtype : recvX->dtype) == CAM_DT_FLOAT16;
     g.out = (uint16_t *)out->data;
     auto run = [g](void *, hipStream_t s) -> hipError_t { return cam::launch_combine(g, s); };
     return finish_phase1(kOpCombGather, 0, run, workspaceSize, executor);
@@ -1366,9 +1367,6 @@ camStatus camMoeCombineShmemGetWorkspaceSize(
         return fail(CAM_ERR_RANGE, "row counts do not fit 32 bits");
     }
     const bool wire = commQuantMode == 2;
-    if (wire && expandX->dtype != CAM_DT_BF16) {
-        return fail(CAM_ERR_UNSUPPORTED, "MoeCombineShmem: commQuantMode 2 is built for bf16 rows only");
-    }
     CAM_TRY(check_aligned(expandX, "expandX", 16));
     CAM_TRY(check_aligned(out, "out", 16));
     Carver c;
@@ -1396,7 +1394,7 @@ camStatus camMoeCombineShmemGetWorkspaceSize(
         g.slot_row = slot;
         if (wire) {  // every row takes the int8 wire format on its way (moe_combine_shmem.h:567-592,755-773)
             uint8_t *rows = (uint8_t *)ws + o_wire;
-            e = cam::launch_comm_quant(g.y, g.A, g.H, counts + (iE - 1), rows, s);
+            e = cam::launch_comm_quant(g.y, g.act_fp16, g.A, g.H, counts + (iE - 1), rows, s);
             if (e != hipSuccess) {
                 return e;
             }
@@ -1621,7 +1619,7 @@ camStatus camGroupedMatmulDequantGetWorkspaceSize(const camTensor *x, const camT
         if (e != hipSuccess) {
             return e;
         }
-        return cam::launch_comm_quant(rows, gc.A, g.N, sp.sched + 1, wire_out, s);  // sched[1]: rows that exist
+        return cam::launch_comm_quant(rows, 0, gc.A, g.N, sp.sched + 1, wire_out, s);  // sched[1]: rows that exist
     };
     return finish_phase1(kOpGmm2, c.off, run, workspaceSize, executor);
 }

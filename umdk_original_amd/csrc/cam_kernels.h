@@ -135,7 +135,7 @@ hipError_t launch_invert_src_info(const int32_t *src_info, int64_t A, const int3
                                   int32_t *slot_row, hipStream_t stream);
 struct CombineArgs {
     const uint16_t *y;        // [A,H] bf16 bits, or wire rows [A, H + H/4] bytes (wire_rows != 0)
-    int wire_rows;            // rows are H int8 values + H/8 bf16 block scales (launch_comm_quant's output)
+    int wire_rows;            // rows are H int8 values + H/8 block scales of the activation type (launch_comm_quant's output)
     int act_fp16;             // rows and output are IEEE fp16 instead of bf16 (not with wire_rows)
     const int32_t *slot_row;  // [T,K] row of slot (t,k) (<0: skip)
     const int32_t *src_info;  // optional: when set, slot_row entries are verified against the triples
@@ -154,7 +154,7 @@ hipError_t launch_rows_from_counts(const int32_t *ids, const int32_t *expand_idx
                                    int64_t n, int E, int64_t A, int32_t *slot_row, hipStream_t stream);
 // bf16 rows [A,H] -> wire rows [A, H + H/4] bytes: per block of 8 columns int8 values and one bf16 scale.
 // row_limit: optional device scalar; rows >= *row_limit are left untouched.
-hipError_t launch_comm_quant(const uint16_t *y, int64_t A, int H, const int32_t *row_limit, uint8_t *out,
+hipError_t launch_comm_quant(const uint16_t *y, int act_fp16, int64_t A, int H, const int32_t *row_limit, uint8_t *out,
                              hipStream_t stream);
 
 // ---------------------------------------------------------------------------------------------

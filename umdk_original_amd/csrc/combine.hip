@@ -67,7 +67,9 @@ __global__ void rows_from_counts_kernel(const int32_t *__restrict__ ids, const i
     slot_row[i] = (int32_t)row;
 }
 
-// bf16 rows -> wire rows.  One thread per block of 8 columns.
+// Rows of the activation type (ACT: 0 = bf16, 1 = IEEE fp16) -> wire rows, whose block scales are of that type
+// too (moe_combine_shmem.h:567-592 keeps them as ExpandXType).  One thread per block of 8 columns.
+template <int ACT>
 __global__ __launch_bounds__(256) void comm_quant_kernel(const uint16_t *__restrict__ y, long long A, int H,
                                                          const int32_t *__restrict__ row_limit,
                                                          uint8_t *__restrict__ out)
@@ -85,8 +87,8 @@ __global__ __launch_bounds__(256) void comm_quant_kernel(const uint16_t *__restr
     float m = 0.0f;
 #pragma unroll
     for (int c = 0; c < 4; ++c) {
-        x[2 * c] = bf16_bits_to_f32(v[c] & 0xffffu);
-        x[2 * c + 1] = bf16_bits_to_f32(v[c] >> 16);
+        x[2 * c] = ACT == 0 ? bf16_bits_to_f32(v[c] & 0xffffu) : fp16_bits_to_f32(v[c] & 0xffffu);
+        x[2 * c + 1] = ACT == 0 ? bf16_bits_to_f32(v[c] >> 16) : fp16_bits_to_f32(v[c] >> 16);
         m = fmaxf(m, fmaxf(fabsf(x[2 * c]), fabsf(x[2 * c + 1])));
     }
     const long long pitch = (long long)H + H / 4;
@@ -94,7 +96,7 @@ __global__ __launch_bounds__(256) void comm_quant_kernel(const uint16_t *__restr
     uint16_t sbits = 0;
     if (m != 0.0f) {
         const float s = __fmul_rn(m, 1.0f / 127.0f);
-        sbits = (uint16_t)f32_to_bf16_bits(s);
+        sbits = (uint16_t)(ACT == 0 ? f32_to_bf16_bits(s) : f32_to_fp16_bits(s));
 #pragma unroll
         for (int j = 0; j < 8; ++j) {
             const _Float16 h = (_Float16)__fdiv_rn(x[j], s);  // round to nearest even
@@ -171,11 +173,14 @@ __global__ __launch_bounds__(kCombThreads) void combine_kernel(CombineArgs a, in
 #pragma unroll
             for (int j = 0; j < kCombBatch; ++j) {
                 if (ok[j] && WIRE) {
-                    const float sc = bf16_bits_to_f32(v[j][2]);
+                    const float sc = comb_act_to_f32<ACT>(v[j][2]);
 #pragma unroll
                     for (int c = 0; c < 8; ++c) {
                         const int q = (int)(int8_t)((v[j][c >> 2] >> (8 * (c & 3))) & 0xffu);
-                        const float x = bf16_bits_to_f32(f32_to_bf16_bits(__fmul_rn((float)q, sc)));
+                        // the row as it leaves the wire: rounded to the activation type (moe_combine_shmem.h:755-773)
+                        const float p = __fmul_rn((float)q, sc);
+                        const float x = ACT == 0 ? bf16_bits_to_f32(f32_to_bf16_bits(p))
+                                                 : fp16_bits_to_f32(f32_to_fp16_bits(p));
                         acc[c] = __fadd_rn(acc[c], __fmul_rn(x, w[j]));
                     }
                 } else if (ok[j]) {
@@ -323,8 +328,8 @@ hipError_t launch_rows_from_counts(const int32_t *ids, const int32_t *expand_idx
     return hipGetLastError();
 }
 
-hipError_t launch_comm_quant(const uint16_t *y, int64_t A, int H, const int32_t *row_limit, uint8_t *out,
-                             hipStream_t stream)
+hipError_t launch_comm_quant(const uint16_t *y, int act_fp16, int64_t A, int H, const int32_t *row_limit,
+                             uint8_t *out, hipStream_t stream)
 {
     if (A <= 0) {
         return hipSuccess;
@@ -337,8 +342,13 @@ hipError_t launch_comm_quant(const uint16_t *y, int64_t A, int H, const int32_t 
     if (blocks > 0x7fffffffll) {
         return hipErrorInvalidValue;
     }
-    hipLaunchKernelGGL(comm_quant_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, y, (long long)A, H, row_limit,
-                       out);
+    if (act_fp16) {
+        hipLaunchKernelGGL(comm_quant_kernel<1>, dim3((unsigned)blocks), dim3(256), 0, stream, y, (long long)A, H,
+                           row_limit, out);
+    } else {
+        hipLaunchKernelGGL(comm_quant_kernel<0>, dim3((unsigned)blocks), dim3(256), 0, stream, y, (long long)A, H,
+                           row_limit, out);
+    }
     return hipGetLastError();
 }
 
@@ -347,7 +357,7 @@ hipError_t launch_combine(const CombineArgs &a, hipStream_t stream)
     if (a.T <= 0) {
         return hipSuccess;
     }
-    if (a.H % 8 != 0 || (a.wire_rows && a.act_fp16)) {
+    if (a.H % 8 != 0) {
         return hipErrorInvalidValue;
     }
     const int segs = (a.H / 8 + kCombThreads - 1) / kCombThreads;
@@ -355,7 +365,9 @@ hipError_t launch_combine(const CombineArgs &a, hipStream_t stream)
     if (blocks > 0x7fffffffll) {
         return hipErrorInvalidValue;
     }
-    if (a.wire_rows && a.H % 64 == 0) {
+    if (a.wire_rows && a.act_fp16) {
+        hipLaunchKernelGGL((combine_kernel<true, 1>), dim3((unsigned)blocks), dim3(kCombThreads), 0, stream, a, segs);
+    } else if (a.wire_rows && a.H % 64 == 0) {
         const int segs16 = (a.H / 16 + kCombThreads - 1) / kCombThreads;
         hipLaunchKernelGGL(combine_wire16_kernel, dim3((unsigned)(a.T * segs16)), dim3(kCombThreads), 0, stream, a,
                            segs16);
