@@ -208,3 +208,23 @@ def test_fp8_fused_layer_random_shape(gpu, oracle, seed):
                                        s2.numpy(), debug=True)
     assert np.array_equal(etn.cpu().numpy(), dbg["cnt"])
     _check_layer(out.float().cpu().numpy(), want)
+
+
+def test_dispatch_and_combine_at_the_largest_parameters(gpu, oracle):
+    """Every parameter at its limit at once: 512 experts, top-16, hidden 7168, and twice the batch the reference's
+    tiling admits (16384 tokens, 262144 routing entries of which one in 513 names no expert)."""
+    T, K, E, H = 16384, 16, 512, 7168
+    announce("largest parameters: T=%d K=%d E=%d H=%d" % (T, K, E, H))
+    rng = np.random.default_rng(T)
+    ids = torch.from_numpy(rng.integers(-1, E, size=(T, K)).astype(np.int64))
+    x = synth.normal_bf16(T, H, seed=T + 1)
+    d = cam.moe_dispatch_fused(x.to(gpu), ids.to(gpu), E, quant_mode=2)
+    idx_np = ids.numpy()
+    _check_fused(oracle, d, x, idx_np, E, 2)
+    cnt, off, pos, _ = plan_oracle(oracle, idx_np, E, skip_out_of_range=True)
+    total = int(cnt.sum())
+    w = torch.from_numpy(rng.random((T, K)).astype(np.float32))
+    y = synth.normal_bf16(total, H, seed=T + 2)
+    got = cam.moe_combine_gather(y.to(gpu), None, d["slot_row"], w.to(gpu))
+    want = oracle.combine(synth.bf16_bits(y), oracle.rows_from_pos(idx_np, off, pos, E), w.numpy())
+    assert_bits_equal(to_np(got), want, "combined x")
